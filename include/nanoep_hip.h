@@ -1,0 +1,134 @@
+/*
+ * nanoep_hip.h -- C ABI of the MI355X (gfx950) expert-parallel dispatch / combine kernels.
+ *
+ * One rank, one GPU.  Every entry point takes plain device pointers, sizes and a HIP stream
+ * (passed as void* so that the header needs no HIP include), enqueues work on that stream,
+ * allocates nothing, throws nothing and returns a status code (NANOEP_OK == 0).
+ *
+ * Shapes use the reference's letters: T source tokens, H hidden, K top-k, L local experts,
+ * N received rows (tokens with at least one valid choice), C padded expanded capacity.
+ *
+ * The handle tensors are the seven the reference's dispatch returns
+ * (csrc/include/nano_ep/pipeline.hpp:13-21 in the reference):
+ *   recv_metadata  int32 [N, K+2] = [src_rank(=0), src_token, K x (local expert id | expanded slot | -1)]
+ *   expert_counts  int64 [L]      actual assignments per expert
+ *   expert_offsets int64 [L+1]    exclusive prefix of counts rounded up to `alignment`; [L] == C
+ *   dst_slots      int64 [T, 1]   receive row of each source token, -1 when it is not sent
+ *   send_counts    int64 [1]      == N
+ *   topk_snapshot  int64 [T, K]   copy of the routing ids
+ *   recv_rank_prefix int64 [1]    == N
+ */
+#ifndef NANOEP_HIP_H_
+#define NANOEP_HIP_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define NANOEP_OK 0
+#define NANOEP_ERR_INVALID_ARGUMENT 1 /* shape / pointer / alignment precondition violated */
+#define NANOEP_ERR_HIP 2              /* a HIP runtime call failed; see nanoep_last_hip_error() */
+#define NANOEP_ERR_WORKSPACE 3        /* workspace too small */
+#define NANOEP_ERR_TIMEOUT 4          /* host wait for the layout counts timed out */
+#define NANOEP_ERR_ROUTING 5          /* layout kernel saw an expert id outside [-1, L) or a duplicate */
+
+/* Bits of the routing status word the layout kernels publish (host_counts[3]). */
+#define NANOEP_ROUTING_BAD_EXPERT 1
+#define NANOEP_ROUTING_DUPLICATE 2
+
+/* Number of int64 words in the host mailbox passed to nanoep_layout / nanoep_wait_counts. */
+#define NANOEP_HOST_COUNT_WORDS 4
+
+int nanoep_abi_version(void);
+const char* nanoep_status_string(int status);
+/* hipGetErrorString of the last HIP failure seen on this thread ("" when none). */
+const char* nanoep_last_hip_error(void);
+
+/* Compute-unit count of `device` (the reference's "device SM count",
+ * nano_ep/backends/cuda.py:108-109). */
+int nanoep_device_cu_count(int device, int* out_cus);
+
+/* Byte offsets of the reference's peer window regions; a pure function kept so that a caller
+ * written against csrc/bindings.cpp:47-58 / csrc/layout.hpp:59-98 still finds it.
+ * out = {signal_offset, count_offset, payload_offset, return_offset, num_bytes}. */
+int nanoep_window_layout(int ranks, int64_t max_tokens, int hidden, int topk, int64_t num_experts,
+                         int allow_multiple_reduction, int64_t out[5]);
+
+/* Device scratch needed by nanoep_layout for (T, K, L). */
+size_t nanoep_layout_workspace_bytes(int64_t num_tokens, int num_topk, int64_t num_local_experts);
+
+/*
+ * Routing layout: histogram + device-wide exclusive scan + stable token-order slot assignment.
+ * Replaces count_and_notify / finalize_receive_counts (csrc/dispatch_main.cuh:116-210, :70-114),
+ * the send-slot assignment of dispatch_payload_rows (csrc/dispatch_main.cuh:278-311) and
+ * build_receive_metadata_row (csrc/dispatch_epilogue.cuh:20-47); results follow
+ * reference_layout (nano_ep/testing/oracle.py:70-104) with rows and slots in token order.
+ *
+ * recv_metadata must have room for T rows; the first N are written.
+ * token_slots (optional, int32 [T, K]) receives slot[t,k] (or the local id when !expand), -1 when
+ * masked: the same information as dst_slots + recv_metadata in one lookup.  It is not one of the
+ * reference's handle tensors; nanoep_dispatch / nanoep_combine run a little faster when given it.
+ * host_counts is pinned, device-visible host memory of NANOEP_HOST_COUNT_WORDS int64:
+ * the call sets word 0 to -1, the device later stores {N, C, A (total assignments), status}
+ * with word 0 last, so a host that sees word 0 >= 0 may read the rest.
+ */
+int nanoep_layout(const int64_t* topk_idx, int64_t num_tokens, int num_topk, int64_t num_local_experts,
+                  int64_t alignment, int expand, int32_t* recv_metadata, int64_t* expert_counts,
+                  int64_t* expert_offsets, int64_t* dst_slots, int64_t* send_counts, int64_t* topk_snapshot,
+                  int64_t* recv_rank_prefix, int32_t* token_slots, void* workspace, size_t workspace_bytes,
+                  int64_t* host_counts, void* stream);
+
+/* Spin on the mailbox until the layout enqueued on `stream` has published its counts
+ * (the reference's wait_dispatch_counts, csrc/peer.cu:198-227).  out = {N, C, A, status}. */
+int nanoep_wait_counts(int64_t* host_counts, void* stream, double timeout_seconds,
+                       int64_t out[NANOEP_HOST_COUNT_WORDS]);
+
+/*
+ * Dispatch permute / expand.  Replaces dispatch_payload_rows + dispatch_epilogue_kernel +
+ * do_zero_padding (csrc/dispatch_main.cuh:215-354, csrc/dispatch_epilogue.cuh:123-250, :50-117);
+ * results follow reference_dispatch (nano_ep/testing/oracle.py:107-147).
+ *   compact : recv_x[row] = x[t]; recv_topk_idx[row,:] = local ids; recv_weights[row,:] = weights[t,:]
+ *   expanded: recv_x[slot] = x[t]; recv_weights[slot] = weights[t,k]; with zero_padding the rows
+ *             [offsets[e]+counts[e], offsets[e+1]) and their weights are zero-filled.
+ * Work is walked in source-token order: dst_slots[t] names the receive row whose metadata holds
+ * the token's slots (token_slots, when not NULL and expanded, replaces that two-step lookup).
+ * x / recv_x are bf16, 16-byte aligned, H % 8 == 0.  weights / recv_weights / recv_topk_idx may be
+ * NULL (recv_topk_idx must be NULL when expanded).  num_cus is the reference's SM budget
+ * (0 = whole device): it is range-checked against the device's compute-unit count and otherwise
+ * ignored, because these kernels are sized by the work, not by a cooperative grid.
+ */
+int nanoep_dispatch(const void* x, const float* weights, const int32_t* recv_metadata, const int64_t* dst_slots,
+                    const int32_t* token_slots, const int64_t* expert_counts, const int64_t* expert_offsets,
+                    int64_t recv_count, int64_t expanded_capacity, int64_t num_tokens, int hidden, int num_topk,
+                    int64_t num_local_experts, int64_t alignment, int expand, int zero_padding, void* recv_x,
+                    int64_t* recv_topk_idx, float* recv_weights, int num_cus, void* stream);
+
+/*
+ * Combine gather-reduce.  Replaces combine_return_rows + combine_epilogue_kernel
+ * (csrc/combine_main.cuh:38-246, csrc/combine_epilogue.cuh:58-202); results follow
+ * reference_combine (nano_ep/testing/oracle.py:150-186) and reference_combined
+ * (nano_ep/testing/native_combine.py:168-195) for one rank:
+ *   out_x[t] = bf16_rne( sum over valid k ascending of f32(y[slot[t,k]]) (+ f32(bias[t])) )
+ * (compact: the single row y[row(t)]); tokens that were not sent get 0 (+bias).
+ * multiple_reduction != 0 with expand rounds the sum of two or more rows to bf16 once before
+ * the final fp32 pass, as the reference's allow_multiple_reduction mode does.
+ * out_weights[t,k] = valid ? (expand ? weights[slot] : weights[row,k]) : 0.
+ * y_rows is the row count of y (C when expanded, N when compact).
+ */
+int nanoep_combine(const void* y, const float* weights, const void* bias, const int32_t* recv_metadata,
+                   const int64_t* dst_slots, const int32_t* token_slots, int64_t recv_count, int64_t y_rows,
+                   int64_t num_tokens, int hidden, int num_topk, int expand, int multiple_reduction, void* out_x,
+                   float* out_weights, int num_cus, void* stream);
+
+/* Plain 16-byte-vector device copy of `bytes` (multiple of 16); the known-size kernel used to
+ * scale the profiler's HBM byte counters.  No counterpart in the reference. */
+int nanoep_copy_bytes(const void* src, void* dst, size_t bytes, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+
+#endif /* NANOEP_HIP_H_ */

@@ -1,0 +1,536 @@
+// PyTorch-ROCm host extension for one rank's dispatch / combine.
+//
+// This file owns what the reference's host pipeline owns (csrc/pipeline.cu:340-489,
+// csrc/dispatch_epilogue.cpp:18-75, csrc/combine_epilogue.cpp:27-64 in the reference): argument
+// validation, output allocation, stream ordering between the caller's stream and the buffer's
+// communication stream, and the completion event.  All device work goes through the C ABI of
+// include/nanoep_hip.h.  The module exports the reference's operator surface
+// (csrc/bindings.cpp:11-86) with the same positional order, so a caller written against the
+// reference's backend module binds to this one unchanged.
+
+#include <ATen/hip/HIPContext.h>
+#include <ATen/hip/impl/HIPGuardImplMasqueradingAsCUDA.h>
+#include <ATen/hip/impl/HIPStreamMasqueradingAsCUDA.h>
+#include <c10/core/Event.h>
+#include <hip/hip_runtime_api.h>
+#include <torch/extension.h>
+
+#include <array>
+#include <limits>
+#include <memory>
+#include <string>
+#include <tuple>
+#include <vector>
+
+#include "nanoep_hip.h"
+
+namespace py = pybind11;
+
+namespace nanoep {
+
+using Stream = c10::hip::HIPStreamMasqueradingAsCUDA;
+using StreamGuard = c10::hip::HIPStreamGuardMasqueradingAsCUDA;
+using OptionalStreamGuard = c10::hip::OptionalHIPStreamGuardMasqueradingAsCUDA;
+using DeviceGuard = c10::hip::HIPGuardMasqueradingAsCUDA;
+
+namespace {
+
+constexpr int64_t kHiddenAlignment = 256;  // the reference's H % 256 == 0 contract
+constexpr double kCountTimeoutSeconds = 60.0;
+
+void check_status(int status, const char* what) {
+    if (status == NANOEP_OK)
+        return;
+    TORCH_CHECK(false, "nanoep ", what, " failed: ", nanoep_status_string(status), " ", nanoep_last_hip_error());
+}
+
+void check_hip(hipError_t status, const char* what) {
+    TORCH_CHECK(status == hipSuccess, "HIP call ", what, " failed: ", hipGetErrorString(status));
+}
+
+Stream external_stream(int64_t handle, c10::DeviceIndex device) {
+    return c10::hip::getStreamFromExternalMasqueradingAsCUDA(reinterpret_cast<hipStream_t>(handle), device);
+}
+
+void wait_on(const Stream& waiter, const Stream& producer) {
+    c10::Event ready(c10::DeviceType::CUDA);
+    ready.record(producer.unwrap());
+    waiter.unwrap().wait(ready);
+}
+
+// Compute-unit budget: 0 or the device size mean the whole device (the reference's
+// resolve_main_sms, csrc/pipeline.cu:20-24).
+int resolve_cu_budget(int num_sms, c10::DeviceIndex device) {
+    const int device_cus = at::cuda::getDeviceProperties(device)->multiProcessorCount;
+    TORCH_CHECK(num_sms >= 0 && num_sms <= device_cus, "num_sms must be between 0 and the device CU count (", device_cus, ")");
+    return num_sms == device_cus ? 0 : num_sms;
+}
+
+}  // namespace
+
+// Holds what one rank needs at world_size == 1: the device, the pinned host mailbox the layout
+// kernels publish N / C into, and (only if somebody asks for it) a window-sized byte tensor.
+// It keeps the reference's PeerRuntime method set (csrc/bindings.cpp:59-83) so setup code written
+// for the reference runs; there are no peers, so handles are opaque tags and barriers are no-ops.
+class PeerRuntime {
+   public:
+    PeerRuntime(int rank, int world_size, int64_t num_bytes) : num_bytes_(num_bytes) {
+        TORCH_CHECK(world_size == 1 && rank == 0,
+                    "this build runs one rank on one GPU (world_size == 1); got rank ", rank, " of ", world_size);
+        TORCH_CHECK(num_bytes >= 0, "window size must be non-negative");
+        check_hip(hipGetDevice(&device_), "hipGetDevice");
+        void* mailbox = nullptr;
+        check_hip(hipHostMalloc(&mailbox, NANOEP_HOST_COUNT_WORDS * sizeof(int64_t), hipHostMallocMapped | hipHostMallocCoherent),
+                  "hipHostMalloc");
+        host_counts_ = static_cast<int64_t*>(mailbox);
+        for (int i = 0; i < NANOEP_HOST_COUNT_WORDS; ++i)
+            host_counts_[i] = -1;
+    }
+
+    ~PeerRuntime() {
+        if (host_counts_ != nullptr)
+            (void)hipHostFree(host_counts_);
+    }
+
+    PeerRuntime(const PeerRuntime&) = delete;
+    PeerRuntime& operator=(const PeerRuntime&) = delete;
+
+    int rank() const { return 0; }
+    int world_size() const { return 1; }
+    int device() const { return device_; }
+    int64_t* host_counts() const {
+        TORCH_CHECK(!closed_, "PeerRuntime is closed");
+        return host_counts_;
+    }
+
+    py::bytes export_local_handle() const {
+        std::string tag(64, '\0');
+        tag.replace(0, 9, "nanoep-r1");
+        return py::bytes(tag);
+    }
+
+    void import_peer_handles(const std::vector<py::bytes>& handles) {
+        TORCH_CHECK(!closed_, "PeerRuntime is closed");
+        if (handles.size() != 1)
+            throw py::value_error("expected exactly one handle (world_size == 1)");
+        for (const auto& handle : handles)
+            if (py::len(handle) != 64)
+                throw py::value_error("Each IPC handle must contain exactly 64 bytes");
+        mappings_open_ = true;
+    }
+
+    torch::Tensor local_window() {
+        TORCH_CHECK(!closed_, "PeerRuntime is closed");
+        if (!window_.defined()) {
+            DeviceGuard guard(static_cast<c10::DeviceIndex>(device_));
+            window_ = torch::zeros({num_bytes_}, torch::dtype(torch::kUInt8).device(torch::kCUDA, device_));
+        }
+        return window_;
+    }
+
+    torch::Tensor peer_addresses() {
+        auto window = local_window();
+        auto addresses = torch::empty({1}, torch::dtype(torch::kInt64));
+        addresses[0] = reinterpret_cast<int64_t>(window.data_ptr());
+        return addresses.to(window.device());
+    }
+
+    // No peers: an epoch barrier has nobody to meet.
+    void barrier(int64_t) const { TORCH_CHECK(!closed_, "PeerRuntime is closed"); }
+    void barrier_at(int64_t, int64_t) const { TORCH_CHECK(!closed_, "PeerRuntime is closed"); }
+
+    void close_peer_mappings() { mappings_open_ = false; }
+
+    void close() {
+        if (closed_)
+            return;
+        TORCH_CHECK(!mappings_open_, "close_peer_mappings must run before close");
+        window_ = torch::Tensor();
+        closed_ = true;
+    }
+
+   private:
+    int device_ = 0;
+    int64_t num_bytes_ = 0;
+    int64_t* host_counts_ = nullptr;
+    torch::Tensor window_;
+    bool mappings_open_ = false;
+    bool closed_ = false;
+};
+
+// Recorded on the communication stream; waiting orders the consumer stream after it and tells
+// the caching allocator that the protected tensors are used there
+// (csrc/include/nano_ep/event.hpp:12-28 in the reference).
+struct CompletionEvent {
+    std::shared_ptr<c10::Event> event;
+    std::vector<torch::Tensor> tensors;
+
+    CompletionEvent(const Stream& stream, std::vector<torch::Tensor> outputs)
+        : event(std::make_shared<c10::Event>(c10::DeviceType::CUDA)), tensors(std::move(outputs)) {
+        event->record(stream.unwrap());
+    }
+
+    void wait(const Stream& stream) const {
+        stream.unwrap().wait(*event);
+        for (const auto& tensor : tensors)
+            if (tensor.defined() && tensor.numel() > 0)
+                tensor.record_stream(stream.unwrap());
+    }
+
+    void current_stream_wait() const { wait(c10::hip::getCurrentHIPStreamMasqueradingAsCUDA()); }
+};
+
+namespace {
+
+void check_payload_inputs(const torch::Tensor& x,
+                          const torch::Tensor& indices,
+                          const c10::optional<torch::Tensor>& weights,
+                          int device,
+                          int64_t num_experts,
+                          int64_t max_tokens) {
+    TORCH_CHECK(x.is_cuda() && x.get_device() == device && x.dim() == 2 && x.is_contiguous(),
+                "x must be contiguous CUDA [T,H] on the runtime device");
+    TORCH_CHECK(x.scalar_type() == torch::kBFloat16, "dispatch x must be bfloat16");
+    TORCH_CHECK(x.size(1) > 0 && x.size(1) % kHiddenAlignment == 0, "dispatch hidden must be a positive multiple of 256");
+    TORCH_CHECK(x.numel() == 0 || reinterpret_cast<uintptr_t>(x.data_ptr()) % 16 == 0,
+                "dispatch x data pointer must be 16-byte aligned");
+    TORCH_CHECK(indices.device() == x.device() && indices.scalar_type() == torch::kInt64 && indices.dim() == 2 &&
+                    indices.size(0) == x.size(0) && indices.is_contiguous(),
+                "indices must be contiguous CUDA int64 [T,K] on the x device");
+    TORCH_CHECK(indices.size(1) > 0 && indices.size(1) <= 32, "num_topk must be in [1, 32]");
+    TORCH_CHECK(num_experts > 0, "num_experts must be positive and divisible by world_size");
+    TORCH_CHECK(max_tokens <= std::numeric_limits<int32_t>::max(), "max_tokens exceeds int32 metadata range");
+    TORCH_CHECK(max_tokens > 0 && x.size(0) <= max_tokens, "source token count exceeds max_tokens");
+    if (weights.has_value()) {
+        TORCH_CHECK(weights->device() == x.device() && weights->scalar_type() == torch::kFloat32 &&
+                        weights->sizes() == indices.sizes() && weights->is_contiguous(),
+                    "weights must be contiguous CUDA float32 [T,K] on the x device");
+    }
+}
+
+void check_cached_tensor(const torch::Tensor& tensor,
+                         const torch::Tensor& reference,
+                         at::IntArrayRef shape,
+                         const char* name,
+                         at::ScalarType dtype = torch::kInt64) {
+    TORCH_CHECK(tensor.device() == reference.device() && tensor.scalar_type() == dtype && tensor.sizes() == shape && tensor.is_contiguous(),
+                "cached ", name, " has invalid CUDA storage or shape");
+}
+
+void check_handle_metadata(const std::vector<torch::Tensor>& metadata, const torch::Tensor& x, int64_t source_tokens, int64_t topk,
+                           int64_t local_experts) {
+    const int64_t recv_count = metadata[0].dim() == 2 ? metadata[0].size(0) : -1;
+    check_cached_tensor(metadata[0], x, {recv_count, topk + 2}, "recv_metadata", torch::kInt32);
+    check_cached_tensor(metadata[1], x, {local_experts}, "expert_counts");
+    check_cached_tensor(metadata[2], x, {local_experts + 1}, "expert_offsets");
+    check_cached_tensor(metadata[3], x, {source_tokens, 1}, "dst_slots");
+    check_cached_tensor(metadata[4], x, {1}, "send_counts");
+    check_cached_tensor(metadata[5], x, {source_tokens, topk}, "source_topk_snapshot");
+    check_cached_tensor(metadata[6], x, {1}, "recv_rank_prefix");
+}
+
+// The optional eighth handle tensor: int32 [T,K] slot table written by the layout kernels.
+const int32_t* slot_table(const std::vector<torch::Tensor>& metadata, int64_t tokens, int64_t topk, bool expand) {
+    if (!expand || metadata.size() < 8 || !metadata[7].defined())
+        return nullptr;
+    const auto& table = metadata[7];
+    TORCH_CHECK(table.device() == metadata[0].device() && table.scalar_type() == torch::kInt32 && table.is_contiguous() &&
+                    table.dim() == 2 && table.size(0) == tokens && table.size(1) == topk,
+                "cached slot table has invalid CUDA storage or shape");
+    return table.numel() == 0 ? nullptr : table.data_ptr<int32_t>();
+}
+
+// Communication stream waits for the producer of the inputs: the caller's stream, an explicit
+// event, or both (csrc/pipeline.cu:364-377 in the reference).
+void order_comm_after_inputs(const Stream& comm, const Stream& compute, int64_t previous_event, bool async_op) {
+    if (previous_event != -1) {
+        if (!async_op && comm != compute)
+            wait_on(comm, compute);
+        check_hip(hipStreamWaitEvent(comm.stream(), reinterpret_cast<hipEvent_t>(previous_event), 0), "hipStreamWaitEvent");
+    } else if (comm != compute) {
+        wait_on(comm, compute);
+    }
+}
+
+}  // namespace
+
+using DispatchResult =
+    std::tuple<std::vector<torch::Tensor>, std::vector<torch::Tensor>, std::array<int64_t, 2>, std::shared_ptr<CompletionEvent>>;
+
+DispatchResult dispatch(PeerRuntime& runtime,
+                        const torch::Tensor& x,
+                        const torch::Tensor& indices,
+                        const c10::optional<torch::Tensor>& weights,
+                        int64_t num_experts,
+                        int64_t max_tokens,
+                        int64_t alignment,
+                        const std::vector<torch::Tensor>& cached_metadata,
+                        int64_t cached_expanded_capacity,
+                        bool /*allow_multiple_reduction*/,
+                        bool expand,
+                        bool zero_padding,
+                        int num_sms,
+                        int64_t comm_stream,
+                        int64_t previous_event,
+                        bool async_op) {
+    const bool cached = !cached_metadata.empty();
+    TORCH_CHECK(!cached || cached_metadata.size() == 7 || cached_metadata.size() == 8,
+                "cached metadata must contain the seven prepared tensors from dispatch (plus the optional slot table)");
+    const auto& routing = cached ? cached_metadata[5] : indices;
+    int64_t* host_counts = runtime.host_counts();
+    check_payload_inputs(x, routing, weights, runtime.device(), num_experts, max_tokens);
+    TORCH_CHECK(alignment > 0, "alignment must be positive");
+    const auto device = static_cast<c10::DeviceIndex>(runtime.device());
+    DeviceGuard device_guard(device);
+    const int cu_budget = resolve_cu_budget(num_sms, device);
+
+    const int64_t tokens = x.size(0);
+    const int64_t hidden = x.size(1);
+    const int64_t topk = routing.size(1);
+    const int64_t local_experts = num_experts;
+
+    const auto compute = c10::hip::getCurrentHIPStreamMasqueradingAsCUDA(device);
+    const auto comm = external_stream(comm_stream, device);
+    order_comm_after_inputs(comm, compute, previous_event, async_op);
+
+    StreamGuard comm_guard(comm.unwrap());
+    // Sync results belong to the caller's stream, async results to the communication stream
+    // (protected by record_stream when the consumer waits on the completion event).
+    const auto allocate_for_consumer = [&](auto&& make) {
+        OptionalStreamGuard allocation_guard;
+        if (!async_op)
+            allocation_guard.reset_stream(compute.unwrap());
+        return make();
+    };
+
+    std::vector<torch::Tensor> metadata;
+    int64_t recv_count = 0;
+    int64_t expanded_capacity = 0;
+    if (cached) {
+        check_handle_metadata(cached_metadata, x, tokens, topk, local_experts);
+        metadata = cached_metadata;
+        recv_count = cached_metadata[0].size(0);
+        expanded_capacity = cached_expanded_capacity;
+        TORCH_CHECK(recv_count <= tokens && expanded_capacity >= 0, "cached handle does not match the payload");
+    } else {
+        hipStreamCaptureStatus capture = hipStreamCaptureStatusNone;
+        check_hip(hipStreamIsCapturing(comm.stream(), &capture), "hipStreamIsCapturing");
+        TORCH_CHECK(capture == hipStreamCaptureStatusNone, "Fresh dispatch with host count polling cannot be captured in a HIP graph");
+
+        const auto int64_options = routing.options();
+        torch::Tensor recv_metadata, expert_counts, expert_offsets, dst_slots, send_counts, snapshot, prefix, token_slots;
+        allocate_for_consumer([&] {
+            recv_metadata = torch::empty({tokens, topk + 2}, int64_options.dtype(torch::kInt32));
+            expert_counts = torch::empty({local_experts}, int64_options);
+            expert_offsets = torch::empty({local_experts + 1}, int64_options);
+            dst_slots = torch::empty({tokens, 1}, int64_options);
+            send_counts = torch::empty({1}, int64_options);
+            snapshot = torch::empty_like(routing);
+            prefix = torch::empty({1}, int64_options);
+            if (expand)
+                token_slots = torch::empty({tokens, topk}, int64_options.dtype(torch::kInt32));
+            return 0;
+        });
+        const size_t workspace_bytes = nanoep_layout_workspace_bytes(tokens, static_cast<int>(topk), local_experts);
+        TORCH_CHECK(workspace_bytes > 0, "unsupported routing geometry for the layout kernels");
+        auto workspace = torch::empty({static_cast<int64_t>(workspace_bytes)}, int64_options.dtype(torch::kUInt8));
+        check_status(nanoep_layout(routing.data_ptr<int64_t>(), tokens, static_cast<int>(topk), local_experts, alignment, expand ? 1 : 0,
+                                   recv_metadata.data_ptr<int32_t>(), expert_counts.data_ptr<int64_t>(),
+                                   expert_offsets.data_ptr<int64_t>(), dst_slots.data_ptr<int64_t>(), send_counts.data_ptr<int64_t>(),
+                                   snapshot.data_ptr<int64_t>(), prefix.data_ptr<int64_t>(),
+                                   expand ? token_slots.data_ptr<int32_t>() : nullptr, workspace.data_ptr(), workspace_bytes,
+                                   host_counts, comm.stream()),
+                     "layout");
+        int64_t counts[NANOEP_HOST_COUNT_WORDS] = {0, 0, 0, 0};
+        const int status = nanoep_wait_counts(host_counts, comm.stream(), kCountTimeoutSeconds, counts);
+        if (status == NANOEP_ERR_ROUTING) {
+            TORCH_CHECK(false, "dispatch routing ids must be -1 or distinct expert ids in [0, ", local_experts, ")",
+                        (counts[3] & NANOEP_ROUTING_BAD_EXPERT) ? "; found an id out of range" : "",
+                        (counts[3] & NANOEP_ROUTING_DUPLICATE) ? "; found a duplicate expert within a token" : "");
+        }
+        check_status(status, "wait_counts");
+        recv_count = counts[0];
+        expanded_capacity = counts[1];
+        TORCH_CHECK(recv_count >= 0 && recv_count <= tokens, "dispatch receive count exceeds the source token count");
+        metadata = {recv_metadata.narrow(0, 0, recv_count), expert_counts, expert_offsets, dst_slots, send_counts, snapshot, prefix};
+        if (expand)
+            metadata.push_back(token_slots);  // private eighth entry: slot[t,k] in one lookup
+    }
+    TORCH_CHECK(!expand || expanded_capacity <= std::numeric_limits<int32_t>::max(), "expanded capacity exceeds int32 metadata range");
+
+    const int64_t rows = expand ? expanded_capacity : recv_count;
+    torch::Tensor out_x, out_indices, out_weights;
+    allocate_for_consumer([&] {
+        out_x = torch::empty({rows, hidden}, x.options());
+        out_indices = expand ? torch::empty({0}, routing.options()) : torch::empty({recv_count, topk}, routing.options());
+        out_weights = !weights.has_value() ? torch::empty({0}, x.options().dtype(torch::kFloat32))
+                      : expand            ? torch::empty({expanded_capacity}, x.options().dtype(torch::kFloat32))
+                                          : torch::empty({recv_count, topk}, x.options().dtype(torch::kFloat32));
+        return 0;
+    });
+
+    if (recv_count > 0) {
+        check_status(
+            nanoep_dispatch(x.data_ptr(), weights.has_value() ? weights->data_ptr<float>() : nullptr, metadata[0].data_ptr<int32_t>(),
+                            metadata[3].data_ptr<int64_t>(), slot_table(metadata, tokens, topk, expand), metadata[1].data_ptr<int64_t>(),
+                            metadata[2].data_ptr<int64_t>(), recv_count, expanded_capacity, tokens,
+                            static_cast<int>(hidden), static_cast<int>(topk), local_experts, alignment, expand ? 1 : 0,
+                            zero_padding ? 1 : 0, out_x.data_ptr(), expand ? nullptr : out_indices.data_ptr<int64_t>(),
+                            weights.has_value() ? out_weights.data_ptr<float>() : nullptr, cu_budget, comm.stream()),
+            "dispatch");
+    }
+
+    std::vector<torch::Tensor> outputs{out_x, out_indices, out_weights};
+    std::shared_ptr<CompletionEvent> event;
+    if (async_op) {
+        if (x.numel() > 0)
+            x.record_stream(comm.unwrap());
+        if (!cached && indices.numel() > 0)
+            indices.record_stream(comm.unwrap());
+        if (weights.has_value() && weights->numel() > 0)
+            weights->record_stream(comm.unwrap());
+        for (const auto& tensor : cached_metadata)
+            if (tensor.numel() > 0)
+                tensor.record_stream(comm.unwrap());
+        auto protected_tensors = outputs;
+        protected_tensors.insert(protected_tensors.end(), metadata.begin(), metadata.end());
+        event = std::make_shared<CompletionEvent>(comm, std::move(protected_tensors));
+    } else if (comm != compute) {
+        wait_on(compute, comm);
+    }
+    return std::make_tuple(std::move(outputs), std::move(metadata), std::array<int64_t, 2>{recv_count, expanded_capacity}, std::move(event));
+}
+
+using CombineResult = std::tuple<std::vector<torch::Tensor>, std::shared_ptr<CompletionEvent>>;
+
+CombineResult combine(PeerRuntime& runtime,
+                      const torch::Tensor& x,
+                      const std::vector<torch::Tensor>& metadata,
+                      const c10::optional<torch::Tensor>& weights,
+                      const c10::optional<torch::Tensor>& bias,
+                      int64_t max_tokens,
+                      bool expand,
+                      bool allow_multiple_reduction,
+                      int num_sms,
+                      int64_t comm_stream,
+                      int64_t previous_event,
+                      bool async_op) {
+    TORCH_CHECK((metadata.size() == 7 || metadata.size() == 8) && x.dim() == 2 && metadata[5].dim() == 2,
+                "combine requires a 2D payload and seven prepared metadata tensors");
+    (void)runtime.host_counts();  // rejects a closed runtime
+    const auto device = static_cast<c10::DeviceIndex>(runtime.device());
+    DeviceGuard device_guard(device);
+    TORCH_CHECK(x.is_cuda() && x.get_device() == device && x.is_contiguous() && x.size(1) > 0,
+                "combine x must be contiguous CUDA [N,H] or [C,H] on the runtime device");
+    TORCH_CHECK(x.scalar_type() == torch::kBFloat16, "combine x must be bfloat16");
+    TORCH_CHECK(reinterpret_cast<uintptr_t>(x.data_ptr()) % 16 == 0, "combine x data pointer must be 16-byte aligned");
+    TORCH_CHECK(x.size(1) % kHiddenAlignment == 0, "combine hidden must be a positive multiple of 256");
+    TORCH_CHECK(metadata[1].dim() == 1 && metadata[1].numel() > 0,
+                "combine metadata requires a [T,K] source snapshot and [L] expert counts");
+
+    const int64_t recv_count = metadata[0].dim() == 2 ? metadata[0].size(0) : -1;
+    const int64_t source_tokens = metadata[5].size(0);
+    const int64_t hidden = x.size(1);
+    const int64_t topk = metadata[5].size(1);
+    const int64_t local_experts = metadata[1].numel();
+    TORCH_CHECK(topk > 0 && topk <= 32 && topk <= local_experts && source_tokens <= max_tokens && recv_count <= max_tokens,
+                "combine routing geometry exceeds expert/token capacity");
+    check_handle_metadata(metadata, x, source_tokens, topk, local_experts);
+    TORCH_CHECK(expand ? (x.size(0) >= recv_count && (recv_count != 0 || x.size(0) == 0)) : x.size(0) == recv_count,
+                "combine x rows do not match the receive layout");
+    if (weights.has_value()) {
+        const bool shape_matches = expand ? (weights->dim() == 1 && weights->size(0) == x.size(0))
+                                          : (weights->dim() == 2 && weights->size(0) == recv_count && weights->size(1) == topk);
+        TORCH_CHECK(weights->device() == x.device() && weights->scalar_type() == torch::kFloat32 && weights->is_contiguous() && shape_matches,
+                    "combine weights must be contiguous CUDA float32 [N,K] or expanded [C] on the x device");
+    }
+    if (bias.has_value()) {
+        TORCH_CHECK(bias->device() == x.device() && bias->scalar_type() == torch::kBFloat16 && bias->is_contiguous() &&
+                        bias->sizes() == at::IntArrayRef({source_tokens, hidden}),
+                    "combine bias must be contiguous [T,H], with the output dtype on the x device");
+    }
+    const int cu_budget = resolve_cu_budget(num_sms, device);
+
+    const auto compute = c10::hip::getCurrentHIPStreamMasqueradingAsCUDA(device);
+    const auto comm = external_stream(comm_stream, device);
+    order_comm_after_inputs(comm, compute, previous_event, async_op);
+    StreamGuard comm_guard(comm.unwrap());
+
+    torch::Tensor combined_x, combined_weights;
+    {
+        OptionalStreamGuard allocation_guard;
+        if (!async_op)
+            allocation_guard.reset_stream(compute.unwrap());
+        combined_x = torch::empty({source_tokens, hidden}, x.options());
+        combined_weights = torch::empty(weights.has_value() ? std::vector<int64_t>{source_tokens, topk} : std::vector<int64_t>{0},
+                                        x.options().dtype(torch::kFloat32));
+    }
+    if (source_tokens > 0) {
+        check_status(nanoep_combine(x.data_ptr(), weights.has_value() ? weights->data_ptr<float>() : nullptr,
+                                    bias.has_value() ? bias->data_ptr() : nullptr, metadata[0].data_ptr<int32_t>(),
+                                    metadata[3].data_ptr<int64_t>(), slot_table(metadata, source_tokens, topk, expand), recv_count,
+                                    x.size(0), source_tokens, static_cast<int>(hidden),
+                                    static_cast<int>(topk), expand ? 1 : 0, allow_multiple_reduction ? 1 : 0, combined_x.data_ptr(),
+                                    weights.has_value() ? combined_weights.data_ptr<float>() : nullptr, cu_budget, comm.stream()),
+                     "combine");
+    }
+
+    std::vector<torch::Tensor> outputs{combined_x, combined_weights};
+    std::shared_ptr<CompletionEvent> event;
+    if (async_op) {
+        if (x.numel() > 0)
+            x.record_stream(comm.unwrap());
+        if (weights.has_value() && weights->numel() > 0)
+            weights->record_stream(comm.unwrap());
+        if (bias.has_value() && bias->numel() > 0)
+            bias->record_stream(comm.unwrap());
+        for (const auto& tensor : metadata)
+            if (tensor.numel() > 0)
+                tensor.record_stream(comm.unwrap());
+        event = std::make_shared<CompletionEvent>(comm, outputs);
+    } else if (comm != compute) {
+        wait_on(compute, comm);
+    }
+    return std::make_tuple(std::move(outputs), std::move(event));
+}
+
+std::vector<int64_t> window_layout(int ranks, int64_t tokens, int hidden, int topk, int64_t num_experts, bool allow_multiple_reduction) {
+    int64_t out[5] = {0, 0, 0, 0, 0};
+    const int status = nanoep_window_layout(ranks, tokens, hidden, topk, num_experts, allow_multiple_reduction ? 1 : 0, out);
+    if (status != NANOEP_OK)
+        throw py::value_error("window_layout requires ranks/topk in [1,32], positive capacity/hidden and num_experts divisible by ranks");
+    return {out[0], out[1], out[2], out[3], out[4]};
+}
+
+}  // namespace nanoep
+
+PYBIND11_MODULE(TORCH_EXTENSION_NAME, module) {
+    module.doc() = "MI355X dispatch / combine host extension (ahead-of-time HIP kernels behind a C ABI)";
+    module.attr("abi_version") = nanoep_abi_version();
+    // Kernels are compiled ahead of time: the JIT warm-up entry points are accepted and ignored.
+    module.def("init_jit", [](const std::string&) {});
+    module.def("prepare_dispatch", [](py::args, py::kwargs) {});
+    module.def("prepare_combine", [](py::args, py::kwargs) {});
+    module.def("dispatch", &nanoep::dispatch, py::arg("runtime"), py::arg("x"), py::arg("indices"), py::arg("weights"),
+               py::arg("num_experts"), py::arg("max_tokens"), py::arg("alignment"), py::arg("cached_metadata"),
+               py::arg("cached_expanded_capacity"), py::arg("allow_multiple_reduction"), py::arg("expand"), py::arg("zero_padding"),
+               py::arg("num_sms"), py::arg("comm_stream"), py::arg("previous_event") = -1, py::arg("async_op") = true,
+               py::call_guard<py::gil_scoped_release>());
+    module.def("combine", &nanoep::combine, py::arg("runtime"), py::arg("x"), py::arg("metadata"), py::arg("weights"), py::arg("bias"),
+               py::arg("max_tokens"), py::arg("expand"), py::arg("allow_multiple_reduction"), py::arg("num_sms"), py::arg("comm_stream"),
+               py::arg("previous_event") = -1, py::arg("async_op") = true, py::call_guard<py::gil_scoped_release>());
+    module.def("window_layout", &nanoep::window_layout, py::arg("ranks"), py::arg("tokens"), py::arg("hidden"), py::arg("topk"),
+               py::arg("num_experts"), py::arg("allow_multiple_reduction") = false);
+    py::class_<nanoep::PeerRuntime>(module, "PeerRuntime")
+        .def(py::init<int, int, int64_t>())
+        .def("export_local_handle", &nanoep::PeerRuntime::export_local_handle)
+        .def("import_peer_handles", &nanoep::PeerRuntime::import_peer_handles)
+        .def("peer_addresses", &nanoep::PeerRuntime::peer_addresses)
+        .def("local_window", &nanoep::PeerRuntime::local_window)
+        .def("barrier", &nanoep::PeerRuntime::barrier)
+        .def("barrier", &nanoep::PeerRuntime::barrier_at)
+        .def("close_peer_mappings", &nanoep::PeerRuntime::close_peer_mappings)
+        .def("close", &nanoep::PeerRuntime::close);
+    py::class_<nanoep::CompletionEvent, std::shared_ptr<nanoep::CompletionEvent>>(module, "CompletionEvent")
+        .def("current_stream_wait", &nanoep::CompletionEvent::current_stream_wait);
+}

@@ -1,0 +1,287 @@
+"""GPU parity of the HIP kernels against the CPU oracle, called through the C ABI.
+
+Bar: bit-exact for the layout, the indices and the dispatched payload (a byte copy, NaN payloads
+included); bit-exact for combine on every non-NaN output (fixed ascending-k fp32 accumulation,
+one round-to-nearest-even cast), NaN <-> NaN otherwise.  Cases mirror the reference's
+tests/native/test_native_dispatch.py:211-310 and tests/native/test_native_combine.py:30-77.
+"""
+
+import pytest
+import torch
+
+import cabi
+import cases
+from oracle import nanoep_oracle as oracle
+
+pytestmark = pytest.mark.gpu
+
+POISON = 0xA5
+
+
+def bits(tensor):
+    return tensor.contiguous().view(torch.int16) if tensor.dtype == torch.bfloat16 else tensor.contiguous().view(torch.int32)
+
+
+def assert_bits_equal(actual, expected, what):
+    assert actual.shape == expected.shape, f"{what}: shape {tuple(actual.shape)} != {tuple(expected.shape)}"
+    assert actual.dtype == expected.dtype, what
+    assert torch.equal(bits(actual.cpu()), bits(expected)), f"{what}: bit mismatch"
+
+
+def assert_layout(metadata, counts, expected: oracle.Layout, expand):
+    assert counts[0] == expected.recv_count and counts[1] == expected.expanded_capacity
+    assert counts[2] == int(expected.expert_counts.sum()) and counts[3] == 0
+    for actual, want, name in zip(
+        metadata,
+        expected.metadata(expand),
+        ["recv_metadata", "expert_counts", "expert_offsets", "dst_slots", "send_counts", "topk_snapshot", "recv_rank_prefix"],
+    ):
+        assert actual.dtype == want.dtype and actual.is_contiguous(), name
+        assert tuple(actual.shape) == tuple(want.shape), name
+        assert torch.equal(actual.cpu(), want), name
+    if expand:
+        # private slot table: slot[t,k] for every source token, -1 when masked
+        table = torch.full(expected.topk_idx.shape, -1, dtype=torch.int32)
+        table[expected.src_tokens] = expected.expanded_slots.to(torch.int32)
+        assert torch.equal(metadata[7].cpu(), table), "token_slots"
+
+
+def run_dispatch_combine(device, idx, hidden, experts, alignment, expand, zero_padding, weighted, *, seed=0, num_cus=0):
+    tokens, topk = idx.shape
+    x = cases.payload(tokens, hidden, seed=123 + seed)
+    w = cases.gate_weights(tokens, topk, seed=7 + seed) if weighted else None
+    expected_layout = oracle.layout(idx, experts, alignment)
+    metadata, counts = cabi.layout(idx.to(device), experts, alignment, expand)
+    assert_layout(metadata, counts, expected_layout, expand)
+
+    want_x, want_idx, want_w, _ = oracle.dispatch(x, idx, experts, w, do_expand=expand, alignment=alignment, lay=expected_layout)
+    got_x, got_idx, got_w = cabi.dispatch(
+        x.to(device), None if w is None else w.to(device), metadata, counts, experts, alignment, expand, zero_padding,
+        num_cus=num_cus, poison=POISON,
+    )
+    torch.cuda.synchronize()
+    if expand:
+        # the same handle without the private slot table must give the same bytes
+        plain_x, _, plain_w = cabi.dispatch(
+            x.to(device), None if w is None else w.to(device), metadata, counts, experts, alignment, expand, zero_padding,
+            num_cus=num_cus, poison=POISON, use_table=False,
+        )
+        assert torch.equal(plain_x.view(torch.int16), got_x.view(torch.int16))
+        assert plain_w is None or torch.equal(plain_w.view(torch.int32), got_w.view(torch.int32))
+        assert got_idx is None
+        live = torch.zeros(counts[1], dtype=torch.bool)
+        live[expected_layout.expanded_slots[expected_layout.expanded_slots >= 0]] = True
+        assert_bits_equal(got_x.cpu()[live], want_x[live], "expanded x")
+        if weighted:
+            assert_bits_equal(got_w.cpu()[live], want_w[live], "expanded weights")
+        gaps = ~live
+        if zero_padding:
+            assert_bits_equal(got_x.cpu()[gaps], torch.zeros_like(want_x[gaps]), "gap rows")
+            if weighted:
+                assert_bits_equal(got_w.cpu()[gaps], torch.zeros_like(want_w[gaps]), "gap weights")
+        else:
+            # untouched rows keep the poison: the kernel writes nothing it does not own
+            assert (got_x.cpu()[gaps].view(torch.uint8) == POISON).all()
+    else:
+        assert_bits_equal(got_x, want_x, "compact x")
+        assert torch.equal(got_idx.cpu(), want_idx)
+        if weighted:
+            assert_bits_equal(got_w, want_w, "compact weights")
+
+    # identity-free combine: feed arbitrary expert outputs, compare with the oracle's accumulation
+    rows = counts[1] if expand else counts[0]
+    y = cases.payload(rows, hidden, seed=999 + seed)
+    yw = None
+    if weighted:
+        yw = cases.gate_weights(rows, 1, seed=5).flatten() if expand else cases.gate_weights(rows, topk, seed=5)
+    bias = cases.payload(tokens, hidden, seed=31 + seed) if seed % 2 else None
+    for multi in (False, True):
+        want_out, want_ow = oracle.combine(
+            y, expected_layout.recv_metadata(expand), expected_layout.dst_slots, do_expand=expand, weights=yw, bias=bias,
+            multiple_reduction=multi,
+        )
+        got_out, got_ow = cabi.combine(
+            y.to(device), None if yw is None else yw.to(device), None if bias is None else bias.to(device), metadata,
+            counts, expand, multiple_reduction=multi, num_cus=num_cus, poison=POISON,
+        )
+        torch.cuda.synchronize()
+        assert_bits_equal(got_out, want_out, f"combine x multi={multi}")
+        if weighted:
+            assert_bits_equal(got_ow, want_ow, "combine weights")
+        if expand:
+            plain_out, plain_ow = cabi.combine(
+                y.to(device), None if yw is None else yw.to(device), None if bias is None else bias.to(device), metadata,
+                counts, expand, multiple_reduction=multi, num_cus=num_cus, poison=POISON, use_table=False,
+            )
+            assert_bits_equal(plain_out, want_out, f"combine x without slot table multi={multi}")
+            if weighted:
+                assert_bits_equal(plain_ow, want_ow, "combine weights without slot table")
+    return metadata, counts
+
+
+LAYOUTS = [(False, False), (True, False), (True, True)]
+LAYOUT_IDS = ["compact", "expanded", "expanded-zero-padding"]
+
+
+@pytest.mark.parametrize(
+    "expand,zero_padding,weighted,kind,hidden,alignment",
+    [
+        pytest.param(False, False, True, "mixed", 256, 1, id="compact-weighted"),
+        pytest.param(False, False, False, "masked", 512, 4, id="compact-masked"),
+        pytest.param(False, False, True, "skew", 768, 16, id="compact-skew"),
+        pytest.param(True, False, True, "mixed", 512, 4, id="expanded-weighted"),
+        pytest.param(True, False, False, "masked", 768, 16, id="expanded-masked"),
+        pytest.param(True, True, True, "mixed", 768, 16, id="expanded-zero-padding"),
+        pytest.param(True, True, False, "skew", 256, 4, id="expanded-skew"),
+    ],
+)
+def test_small_cases(device, expand, zero_padding, weighted, kind, hidden, alignment):
+    idx = cases.routing(kind, 5, 3, 3, seed=0)
+    run_dispatch_combine(device, idx, hidden, 3, alignment, expand, zero_padding, weighted, seed=1)
+
+
+@pytest.mark.parametrize("expand,zero_padding", LAYOUTS, ids=LAYOUT_IDS)
+def test_multiple_blocks(device, expand, zero_padding):
+    idx = cases.routing("mixed", 19, 3, 3, seed=3)
+    run_dispatch_combine(device, idx, 512, 3, 16, expand, zero_padding, True, seed=2)
+
+
+@pytest.mark.parametrize(
+    "expand,zero_padding,weighted,hidden",
+    [
+        pytest.param(False, False, True, 512, id="compact"),
+        pytest.param(True, False, False, 768, id="expanded"),
+        pytest.param(True, True, True, 512, id="expanded-zero-padding"),
+    ],
+)
+def test_more_tokens_than_resident_waves(device, expand, zero_padding, weighted, hidden):
+    cus = torch.cuda.get_device_properties(device).multi_processor_count
+    tokens = cus * 32 + 3
+    idx = cases.routing("skew", tokens, 3, 3)
+    idx[:3] = -1
+    idx[::2, 1:] = -1
+    run_dispatch_combine(device, idx, hidden, 3, 128, expand, zero_padding, weighted, seed=3)
+    # the same work under a small CU budget exercises the grid-stride loop
+    run_dispatch_combine(device, idx, hidden, 3, 128, expand, zero_padding, weighted, seed=4, num_cus=2)
+
+
+@pytest.mark.parametrize(
+    "experts,tokens,alignment,weighted,zero_padding",
+    [
+        pytest.param(3, 1, 128, True, True, id="single-wave-zero-padding"),
+        pytest.param(40, 9, 1, False, False, id="multiple-waves-unaligned"),
+        pytest.param(65, 9, 4, True, True, id="multiple-waves-zero-padding"),
+    ],
+)
+def test_padding_gaps_across_expert_waves(device, experts, tokens, alignment, weighted, zero_padding):
+    selected = [2, 33, experts - 1] if experts > 32 else [0, 1, 2]
+    idx = torch.tensor([selected] * tokens, dtype=torch.int64)
+    if tokens > 1:
+        idx[::2, 1] = -1
+        idx[::3, 2] = -1
+    run_dispatch_combine(device, idx, 256, experts, alignment, True, zero_padding, weighted, seed=5)
+
+
+@pytest.mark.parametrize(
+    "name,tokens,hidden,experts,topk,kind,expand,alignment,zero_padding",
+    [
+        pytest.param("mixtral", 4096, 4096, 8, 2, "random", True, 1, False, id="mixtral-4096x4096-e8-k2"),
+        pytest.param("dsv3", 4096, 7168, 256, 8, "dropout", True, 1, True, id="dsv3-4096x7168-e256-k8"),
+        pytest.param("dsv3-a128", 4096, 7168, 256, 8, "dropout", True, 128, True, id="dsv3-align128"),
+        pytest.param("qwen3", 8192, 2048, 128, 8, "biased", True, 128, True, id="qwen3-8192x2048-e128-k8"),
+        pytest.param("ep8", 32768, 7168, 32, 8, "zipf", False, 1, False, id="ep8-share-32768x7168-l32-k8"),
+    ],
+)
+def test_baseline_shapes(device, name, tokens, hidden, experts, topk, kind, expand, alignment, zero_padding):
+    idx = cases.routing(kind, tokens, experts, topk, seed=11)
+    run_dispatch_combine(device, idx, hidden, experts, alignment, expand, zero_padding, True, seed=6)
+
+
+@pytest.mark.parametrize("topk,experts,hidden", [(1, 4, 256), (5, 16, 1024), (12, 40, 512), (32, 64, 256), (32, 32, 2048)])
+@pytest.mark.parametrize("expand", [False, True], ids=["compact", "expanded"])
+def test_topk_range(device, topk, experts, hidden, expand):
+    """Every top-k the API admits (1..32), including the ones that need two gather groups."""
+    idx = cases.routing("dropout", 77, experts, topk, seed=topk)
+    run_dispatch_combine(device, idx, hidden, experts, 8, expand, expand, True, seed=topk)
+
+
+def test_empty_inputs(device):
+    for expand in (False, True):
+        idx = torch.empty((0, 4), dtype=torch.int64)
+        metadata, counts = cabi.layout(idx.to(device), 8, 4, expand)
+        assert counts == (0, 0, 0, 0)
+        assert torch.equal(metadata[1].cpu(), torch.zeros(8, dtype=torch.int64))
+        assert torch.equal(metadata[2].cpu(), torch.zeros(9, dtype=torch.int64))
+        x = torch.empty((0, 256), dtype=torch.bfloat16, device=device)
+        got_x, _, _ = cabi.dispatch(x, None, metadata, counts, 8, 4, expand, True)
+        assert got_x.shape == (0, 256)
+        out, _ = cabi.combine(got_x, None, None, metadata, counts, expand)
+        assert out.shape == (0, 256)
+    # all tokens masked: nothing received, combine still writes zeros (+bias) for every token
+    idx = cases.routing("masked", 7, 4, 2)
+    run_dispatch_combine(device, idx, 256, 4, 8, True, True, True, seed=7)
+
+
+def test_routing_errors_are_reported(device):
+    idx = torch.tensor([[0, 1], [5, 1]], dtype=torch.int64)  # 5 is outside [0, 4)
+    _, counts = cabi.layout(idx.to(device), 4, 1, True, raise_on_routing=False)
+    assert counts[3] & 1
+    idx = torch.tensor([[0, 1], [2, 2]], dtype=torch.int64)  # duplicate inside a token
+    _, counts = cabi.layout(idx.to(device), 4, 1, True, raise_on_routing=False)
+    assert counts[3] & 2
+    with pytest.raises(cabi.NanoEPError):
+        cabi.layout(idx.to(device), 4, 1, True)
+
+
+def test_special_values_survive_dispatch_and_round_in_combine(device):
+    """NaN payloads, infinities, -0 and subnormals are copied bit for bit; combine's 0 + x turns
+    -0 into +0 and keeps subnormal sums exact."""
+    tokens, hidden, experts, topk = 6, 256, 4, 2
+    idx = torch.tensor([[0, 1], [1, 2], [3, -1], [-1, 2], [0, 3], [2, 1]], dtype=torch.int64)
+    patterns = torch.tensor([0x7FC1, 0xFFC0, 0x7F81, 0x7F80, 0xFF80, 0x8000, 0x0001, 0x8001, 0x007F, 0x3F80], dtype=torch.int32)
+    raw = patterns.repeat((tokens * hidden + len(patterns) - 1) // len(patterns))[: tokens * hidden]
+    x = raw.to(torch.int16).view(torch.bfloat16).reshape(tokens, hidden).contiguous()
+    metadata, counts = cabi.layout(idx.to(device), experts, 1, True)
+    got_x, _, _ = cabi.dispatch(x.to(device), None, metadata, counts, experts, 1, True, False)
+    lay = oracle.layout(idx, experts, 1)
+    want_x, _, _, _ = oracle.dispatch(x, idx, experts, None, do_expand=True, lay=lay)
+    assert_bits_equal(got_x, want_x, "special values")
+    got, _ = cabi.combine(got_x, None, None, metadata, counts, True)
+    want, _ = oracle.combine(want_x, lay.recv_metadata(True), lay.dst_slots, do_expand=True)
+    got_cpu = got.cpu()
+    nan = torch.isnan(want)
+    assert torch.equal(torch.isnan(got_cpu), nan)
+    assert torch.equal(bits(got_cpu)[~nan], bits(want)[~nan])
+
+
+def test_reversed_handle_order_is_honoured(device):
+    """Combine must follow the handle, not assume token-ordered slots (the reference's
+    expert_inputs builds handles with reversed receive and slot order)."""
+    idx = cases.routing("mixed", 11, 3, 3, seed=9)
+    lay = oracle.layout(idx, 3, 4)
+    order = torch.arange(lay.recv_count).flip(0)
+    slots = lay.expanded_slots[order].clone()
+    local = lay.local_topk_idx[order]
+    for expert, count in enumerate(lay.expert_counts.tolist()):
+        start = int(lay.expert_offsets[expert])
+        mask = local == expert
+        slots[mask] = 2 * start + count - 1 - slots[mask]
+    tokens = lay.src_tokens[order]
+    dst = torch.full((11, 1), -1, dtype=torch.int64)
+    dst[tokens, 0] = torch.arange(lay.recv_count)
+    for expand in (False, True):
+        body = slots if expand else local
+        meta = torch.cat((torch.zeros_like(tokens)[:, None], tokens[:, None], body), dim=1).to(torch.int32)
+        rows = lay.expanded_capacity if expand else lay.recv_count
+        y = cases.payload(rows, 256, seed=4)
+        w = cases.gate_weights(rows, 1).flatten() if expand else cases.gate_weights(rows, 3)
+        metadata = [meta.to(device), None, None, dst.to(device)]
+        counts = (lay.recv_count, lay.expanded_capacity, 0, 0)
+        got, got_w = cabi.combine(y.to(device), w.to(device), None, metadata, counts, expand)
+        want, want_w = oracle.combine_scalar(y, meta, dst, do_expand=expand, weights=w)
+        assert_bits_equal(got, want, "reversed handle x")
+        assert_bits_equal(got_w, want_w, "reversed handle weights")
+
+
+def test_window_layout_known_answer():
+    assert cabi.window_layout(2, 8, 256, 2, 4) == [0, 96, 160, 160, 9888]
