@@ -1,0 +1,406 @@
+"""GPU tests of the public API (EPConfig / Buffer.dispatch / Buffer.combine) against the CPU oracle.
+
+The cases restate what the reference checks at world_size == 1: the README round trip
+(README.md:44-70), fresh + cached replay with pointer-stable metadata and untouched earlier results
+(tests/native/test_native_dispatch.py:93-208), async_op / previous_event stream handling and the
+exact multiplicity round trip (tests/distributed/worker.py:180-343), plus the five BASELINE shapes.
+"""
+
+import pytest
+import torch
+from torch.utils import deterministic
+
+import cases
+from nanoep_amd import Buffer, CudaBuffer, EPConfig
+from nanoep_amd._native import load_extension
+from oracle import nanoep_oracle as oracle
+
+pytestmark = pytest.mark.gpu
+
+
+def bits(tensor):
+    tensor = tensor.detach().cpu().contiguous()
+    return tensor.view(torch.int16) if tensor.dtype == torch.bfloat16 else tensor.view(torch.int32)
+
+
+def assert_same_bits(actual, expected, what=""):
+    assert tuple(actual.shape) == tuple(expected.shape), what
+    assert actual.dtype == expected.dtype, what
+    assert torch.equal(bits(actual), bits(expected)), f"{what}: bit mismatch"
+
+
+def assert_handle(handle, expected: oracle.Layout, expand, alignment, buffer):
+    assert handle.owner is buffer and handle.do_expand is expand and handle.alignment == alignment
+    assert (handle.rank, handle.world_size) == (0, 1)
+    layout = handle.layout
+    assert layout.recv_count == expected.recv_count and layout.expanded_capacity == expected.expanded_capacity
+    got = [layout.recv_metadata, layout.expert_counts, layout.expert_offsets, handle.dst_slots, handle.send_counts,
+           handle.topk_idx, layout.recv_rank_prefix]
+    for actual, want in zip(got, expected.metadata(expand)):
+        assert actual.is_cuda and actual.is_contiguous() and actual.dtype == want.dtype
+        assert torch.equal(actual.cpu(), want)
+
+
+def assert_dispatch_result(result, x, idx, weights, experts, expand, alignment, zero_padding):
+    want_x, want_idx, want_w, lay = oracle.dispatch(x, idx, experts, weights, do_expand=expand, alignment=alignment)
+    got_x = result.x.cpu()
+    assert result.x.dtype == torch.bfloat16 and result.x.is_contiguous()
+    if expand:
+        assert result.topk_idx is None
+        live = torch.zeros(lay.expanded_capacity, dtype=torch.bool)
+        live[lay.expanded_slots[lay.expanded_slots >= 0]] = True
+        assert got_x.shape == want_x.shape
+        assert_same_bits(got_x[live], want_x[live], "expanded x")
+        if weights is not None:
+            assert_same_bits(result.topk_weights.cpu()[live], want_w[live], "expanded weights")
+        if zero_padding:
+            assert_same_bits(got_x[~live], want_x[~live], "gap rows are zero")
+            if weights is not None:
+                assert_same_bits(result.topk_weights.cpu()[~live], want_w[~live], "gap weights are zero")
+    else:
+        assert_same_bits(got_x, want_x, "compact x")
+        assert torch.equal(result.topk_idx.cpu(), want_idx)
+        if weights is not None:
+            assert_same_bits(result.topk_weights, want_w, "compact weights")
+    if weights is None:
+        assert result.topk_weights is None
+    return lay
+
+
+def test_readme_round_trip(device):
+    """BASELINE config 1: identity experts weighted once, combine reproduces x."""
+    config = EPConfig(num_experts=2, num_topk=2, hidden=256, num_max_tokens_per_rank=16)
+    x = cases.payload(16, 256, seed=0).to(device)
+    indices = torch.tensor([[0, 1]], dtype=torch.int64).repeat(16, 1).to(device)
+    weights = torch.full((16, 2), 0.5, dtype=torch.float32, device=device)
+    with CudaBuffer(None, config) as buffer:
+        received = buffer.dispatch(x, topk_idx=indices, weights=weights, do_expand=True, zero_padding=True)
+        assert received.x.shape == (32, 256) and received.topk_weights.shape == (32,)
+        expert_x = (received.x.float() * received.topk_weights[:, None]).to(received.x.dtype)
+        result = buffer.combine(expert_x, received.handle)
+        torch.testing.assert_close(result.x, x, rtol=0, atol=0)
+        assert result.topk_weights is None and result.event is None
+
+
+@pytest.mark.parametrize(
+    "expand,zero_padding,weighted,kind,hidden,alignment",
+    [
+        pytest.param(False, False, True, "mixed", 256, 1, id="compact-weighted"),
+        pytest.param(False, False, False, "masked", 512, 4, id="compact-masked"),
+        pytest.param(False, False, True, "skew", 768, 16, id="compact-skew"),
+        pytest.param(True, False, True, "mixed", 512, 4, id="expanded-weighted"),
+        pytest.param(True, False, False, "masked", 768, 16, id="expanded-masked"),
+        pytest.param(True, True, True, "mixed", 768, 16, id="expanded-zero-padding"),
+        pytest.param(True, True, False, "skew", 256, 4, id="expanded-skew"),
+    ],
+)
+def test_fresh_and_cached_replay(device, expand, zero_padding, weighted, kind, hidden, alignment):
+    tokens, experts, topk = 19, 3, 3
+    idx = cases.routing(kind, tokens, experts, topk, seed=2)
+    x = cases.payload(tokens, hidden)
+    w = cases.gate_weights(tokens, topk)
+    buffer = Buffer(None, EPConfig(experts, topk, hidden, 32))
+    try:
+        idx_dev = idx.to(device)
+        fresh = buffer.dispatch(
+            x.to(device), topk_idx=idx_dev, weights=w.to(device) if weighted else None, do_expand=expand,
+            alignment=alignment, zero_padding=zero_padding,
+        )
+        lay = assert_dispatch_result(fresh, x, idx, w if weighted else None, experts, expand, alignment, zero_padding)
+        assert_handle(fresh.handle, lay, expand, alignment, buffer)
+        handle = fresh.handle
+        assert handle.num_sms == torch.cuda.get_device_properties(device).multi_processor_count
+        assert handle.x_dtype == torch.bfloat16 and handle.config == buffer._config
+        saved = [t.cpu().clone() for t in (fresh.x, fresh.topk_weights, fresh.topk_idx) if t is not None]
+        metadata = [handle.layout.recv_metadata, handle.layout.expert_counts, handle.layout.expert_offsets, handle.dst_slots,
+                    handle.send_counts, handle.topk_idx, handle.layout.recv_rank_prefix]
+        pointers = [t.data_ptr() for t in metadata]
+        saved_metadata = [t.cpu().clone() for t in metadata]
+        idx_dev.fill_(99)  # the handle owns a snapshot: later edits of the caller's ids must not matter
+
+        for step, replay_weighted in enumerate((not weighted, weighted), start=1):
+            new_x, new_w = x + 2 * step, -w + step
+            replay = buffer.dispatch(
+                new_x.to(device), weights=new_w.to(device) if replay_weighted else None, handle=handle,
+                zero_padding=zero_padding,
+            )
+            assert replay.handle is handle
+            assert_dispatch_result(replay, new_x, idx, new_w if replay_weighted else None, experts, expand, alignment, zero_padding)
+            assert [t.data_ptr() for t in metadata] == pointers
+            for actual, expected in zip(metadata, saved_metadata):
+                assert torch.equal(actual.cpu(), expected)
+            # earlier results own their storage: later calls leave every byte of them alone
+            for actual, expected in zip([t for t in (fresh.x, fresh.topk_weights, fresh.topk_idx) if t is not None], saved):
+                assert torch.equal(actual.cpu().view(torch.uint8), expected.view(torch.uint8))
+
+        # combine on the replayed layout, weights returned at their original k with masked slots zero
+        rows = handle.layout.expanded_capacity if expand else handle.layout.recv_count
+        y = cases.payload(rows, hidden, seed=77)
+        yw = cases.gate_weights(rows, 1).flatten() if expand else cases.gate_weights(rows, topk)
+        bias = cases.payload(tokens, hidden, seed=78)
+        result = buffer.combine(y.to(device), handle, weights=yw.to(device), bias=bias.to(device))
+        want, want_w = oracle.combine(y, lay.recv_metadata(expand), lay.dst_slots, do_expand=expand, weights=yw, bias=bias)
+        assert_same_bits(result.x, want, "combined x")
+        assert_same_bits(result.topk_weights, want_w, "combined weights")
+    finally:
+        buffer.close()
+
+
+@pytest.mark.parametrize("expand", [False, True], ids=["compact", "expanded"])
+def test_async_streams_and_previous_event(device, expand):
+    tokens, experts, topk, hidden = 301, 16, 4, 1024
+    idx = cases.routing("dropout", tokens, experts, topk, seed=5)
+    x_cpu = cases.payload(tokens, hidden)
+    w_cpu = cases.gate_weights(tokens, topk)
+    with Buffer(None, EPConfig(experts, topk, hidden, 512)) as buffer:
+        producer, consumer = torch.cuda.Stream(), torch.cuda.Stream()
+        with torch.cuda.stream(producer):
+            x, w, idx_dev = x_cpu.to(device, non_blocking=True), w_cpu.to(device), idx.to(device)
+            torch.cuda._sleep(2_000_000)  # make a missing dependency on the producer visible
+            x = x * 1
+            ready = torch.cuda.Event()
+            ready.record()
+        with torch.cuda.stream(consumer):
+            received = buffer.dispatch(
+                x, topk_idx=idx_dev, weights=w, do_expand=expand, alignment=8, zero_padding=expand,
+                previous_event=ready, async_op=True,
+            )
+            assert received.event is not None
+            assert any(item is received.handle for item in received.event.keepalive)
+            received.event.current_stream_wait()
+            lay = assert_dispatch_result(received, x_cpu, idx, w_cpu, experts, expand, 8, expand)
+            y = received.x * 1
+            combined = buffer.combine(y, received.handle, weights=received.topk_weights, async_op=True)
+            combined.event.current_stream_wait()
+            want, want_w = oracle.combine(
+                oracle.dispatch(x_cpu, idx, experts, w_cpu, do_expand=expand, alignment=8)[0],
+                lay.recv_metadata(expand), lay.dst_slots, do_expand=expand,
+                weights=oracle.dispatch(x_cpu, idx, experts, w_cpu, do_expand=expand, alignment=8)[2],
+            )
+            assert_same_bits(combined.x, want, "async combine")
+            assert_same_bits(combined.topk_weights, want_w, "async combine weights")
+            expected_weights = w_cpu.masked_fill(idx < 0, 0)
+            assert_same_bits(combined.topk_weights, expected_weights, "weights return to their source slot")
+        torch.cuda.synchronize()
+
+
+def test_exact_multiplicity_round_trip(device):
+    """combine(dispatch(x)) == x * multiplicity + bias exactly in bf16 for small-integer x."""
+    tokens, experts, topk, hidden = 64, 6, 3, 256
+    idx = cases.routing("mixed", tokens, experts, topk, seed=31)
+    x_cpu = torch.full((tokens, hidden), 3, dtype=torch.bfloat16)
+    with Buffer(None, EPConfig(experts, topk, hidden, 64)) as buffer:
+        for expand in (False, True):
+            received = buffer.dispatch(x_cpu.to(device) + 0, topk_idx=idx.to(device), do_expand=expand, alignment=4,
+                                       zero_padding=expand, async_op=True)
+            scratch = torch.empty_like(x_cpu, device=device)
+            scratch.fill_(-77)  # allocator churn while the communication stream may still be busy
+            received.event.current_stream_wait()
+            assert received.topk_weights is None
+            combined = buffer.combine(received.x, received.handle, bias=torch.ones_like(x_cpu, device=device), async_op=expand)
+            if expand:
+                combined.event.current_stream_wait()
+            valid = (idx >= 0).sum(dim=1)
+            multiplicity = valid if expand else (valid > 0).to(torch.int64)
+            expected = x_cpu * multiplicity.to(torch.bfloat16).unsqueeze(1) + 1
+            torch.testing.assert_close(combined.x.cpu(), expected, rtol=0, atol=0)
+            assert combined.topk_weights is None
+
+
+def test_rounding_probe_and_multiple_reduction(device):
+    """256 + 1 - 256: fp32 accumulation keeps the 1 that a bf16 partial sum would lose; the
+    allow_multiple_reduction mode rounds the partial sum to bf16 before the bias and may lose it."""
+    hidden = 256
+    idx = torch.tensor([[0, 1, 2]], dtype=torch.int64)
+    for multi, expected in ((False, 1.0 + 0.5), (True, 1.0 + 0.5)):
+        with Buffer(None, EPConfig(3, 3, hidden, 4), allow_multiple_reduction=multi) as buffer:
+            x = torch.zeros((1, hidden), dtype=torch.bfloat16, device=device)
+            received = buffer.dispatch(x, topk_idx=idx.to(device), do_expand=True)
+            y = torch.empty((3, hidden), dtype=torch.bfloat16, device=device)
+            slots = received.handle.layout.recv_metadata[0, 2:].tolist()
+            y[slots[0]] = 256.0
+            y[slots[1]] = 1.0
+            y[slots[2]] = -256.0
+            bias = torch.full((1, hidden), 0.5, dtype=torch.bfloat16, device=device)
+            out = buffer.combine(y, received.handle, bias=bias).x
+            assert torch.all(out.float() == expected), (multi, out[0, :4])
+    # a partial sum that is not representable in bf16: 256 + 1 = 257 rounds to 256 before the bias
+    with Buffer(None, EPConfig(3, 3, hidden, 4), allow_multiple_reduction=True) as buffer:
+        idx2 = torch.tensor([[0, 1, -1]], dtype=torch.int64)
+        received = buffer.dispatch(torch.zeros((1, hidden), dtype=torch.bfloat16, device=device), topk_idx=idx2.to(device), do_expand=True)
+        slots = received.handle.layout.recv_metadata[0, 2:].tolist()
+        y = torch.zeros((2, hidden), dtype=torch.bfloat16, device=device)
+        y[slots[0]] = 256.0
+        y[slots[1]] = 1.0
+        bias = torch.full((1, hidden), 1.0, dtype=torch.bfloat16, device=device)
+        out = buffer.combine(y, received.handle, bias=bias).x
+        assert torch.all(out.float() == 256.0)  # bf16(256 + 1) = 256, then bf16(256 + 1) = 256
+    with Buffer(None, EPConfig(3, 3, hidden, 4)) as buffer:
+        received = buffer.dispatch(torch.zeros((1, hidden), dtype=torch.bfloat16, device=device), topk_idx=idx2.to(device), do_expand=True)
+        out = buffer.combine(y, received.handle, bias=bias).x
+        assert torch.all(out.float() == 258.0)  # bf16(256 + 1 + 1) = 258
+
+
+def test_argument_errors(device):
+    config = EPConfig(4, 2, 256, 8)
+    buffer, other = Buffer(None, config), Buffer(None, config)
+    x = cases.payload(8, 256).to(device)
+    idx = cases.routing("random", 8, 4, 2).to(device)
+    try:
+        with pytest.raises(ValueError, match="requires topk_idx"):
+            buffer.dispatch(x)
+        with pytest.raises(ValueError, match="alignment"):
+            buffer.dispatch(x, topk_idx=idx, alignment=0)
+        with pytest.raises(ValueError, match="do_expand"):
+            buffer.dispatch(x, topk_idx=idx, do_expand=1)
+        with pytest.raises(ValueError, match="hidden"):
+            buffer.dispatch(x[:, :128].contiguous(), topk_idx=idx)
+        with pytest.raises(ValueError, match="shape"):
+            buffer.dispatch(x, topk_idx=idx[:, :1].contiguous())
+        cus = torch.cuda.get_device_properties(device).multi_processor_count
+        for bad in (-1, cus + 1, True, 1.5):
+            with pytest.raises(ValueError, match="num_sms"):
+                buffer.dispatch(x, topk_idx=idx, num_sms=bad)
+        received = buffer.dispatch(x, topk_idx=idx, do_expand=True, alignment=4, num_sms=7)
+        assert received.handle.num_sms == 7
+        assert buffer.dispatch(x, topk_idx=idx, num_sms=0).handle.num_sms == cus
+        with pytest.raises(ValueError, match="another CudaBuffer"):
+            other.dispatch(x, handle=received.handle)
+        with pytest.raises(ValueError, match="omit topk_idx"):
+            buffer.dispatch(x, topk_idx=idx, handle=received.handle)
+        with pytest.raises(ValueError, match="alignment"):
+            buffer.dispatch(x, handle=received.handle, alignment=8)
+        with pytest.raises(ValueError, match="layout"):
+            buffer.dispatch(x, handle=received.handle, do_expand=False)
+        with pytest.raises(ValueError, match="bfloat16"):
+            buffer.combine(received.x.float(), received.handle)
+        with pytest.raises(ValueError, match="another CudaBuffer"):
+            other.combine(received.x, received.handle)
+        with pytest.raises(ValueError, match="weights"):
+            buffer.combine(received.x, received.handle, weights=torch.zeros(3, device=device))
+        with pytest.raises(ValueError, match="bias"):
+            buffer.combine(received.x, received.handle, bias=torch.zeros((8, 256), device=device))
+        # data-dependent routing errors come back as RuntimeError instead of a device trap
+        bad_idx = idx.clone()
+        bad_idx[0, 0] = 4
+        with pytest.raises(RuntimeError, match="out of range"):
+            buffer.dispatch(x, topk_idx=bad_idx)
+        bad_idx[0] = 1
+        with pytest.raises(RuntimeError, match="duplicate"):
+            buffer.dispatch(x, topk_idx=bad_idx)
+        # the buffer stays usable after a rejected routing
+        again = buffer.dispatch(x, topk_idx=idx, do_expand=True, alignment=4)
+        assert again.handle.layout.recv_count == received.handle.layout.recv_count
+        buffer.close()
+        buffer.close()
+        with pytest.raises(RuntimeError, match="closed"):
+            buffer.dispatch(x, topk_idx=idx)
+        with pytest.raises(RuntimeError, match="closed"):
+            buffer.combine(received.x, received.handle)
+    finally:
+        buffer.close()
+        other.close()
+    with pytest.raises(TypeError):
+        Buffer(None, config, allow_multiple_reduction=1)
+    with pytest.raises(ValueError, match="256"):
+        Buffer(None, EPConfig(4, 2, 128, 8))
+
+
+def test_deterministic_fill_is_rejected_by_the_api_but_not_the_backend(device):
+    """The API refuses deterministic algorithms + fill_uninitialized_memory (as the reference does);
+    the native module accepts them, and the poison torch then writes into every torch.empty output
+    proves that dispatch and combine write every byte they own."""
+    native = load_extension()
+    enabled = torch.are_deterministic_algorithms_enabled()
+    warn_only = torch.is_deterministic_algorithms_warn_only_enabled()
+    fill = deterministic.fill_uninitialized_memory
+    tokens, experts, topk, hidden = 37, 5, 3, 512
+    idx = cases.routing("mixed", tokens, experts, topk, seed=8)
+    x, w = cases.payload(tokens, hidden), cases.gate_weights(tokens, topk)
+    config = EPConfig(experts, topk, hidden, 64)
+    buffer = Buffer(None, config)
+    torch.use_deterministic_algorithms(True)
+    deterministic.fill_uninitialized_memory = True
+    try:
+        with pytest.raises(RuntimeError, match="fill_uninitialized_memory"):
+            buffer.dispatch(x.to(device), topk_idx=idx.to(device))
+        stream = torch.cuda.Stream()
+        stream.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(stream):
+            for expand, zero_padding in ((False, False), (True, True)):
+                outputs, metadata, counts, event = native.dispatch(
+                    buffer._runtime, x.to(device), idx.to(device), w.to(device), experts, 64, 4, [], 0, False,
+                    expand=expand, zero_padding=zero_padding, num_sms=0, comm_stream=stream.cuda_stream,
+                )
+                assert event is not None  # async_op defaults to True at the native boundary
+                event.current_stream_wait()
+                want_x, want_idx, want_w, lay = oracle.dispatch(x, idx, experts, w, do_expand=expand, alignment=4)
+                assert list(counts) == [lay.recv_count, lay.expanded_capacity]
+                assert_same_bits(outputs[0], want_x, "every output row is written")
+                assert_same_bits(outputs[2], want_w, "every output weight is written")
+                assert (outputs[1].shape == (0,)) if expand else torch.equal(outputs[1].cpu(), want_idx)
+                y = outputs[0]
+                results, event = native.combine(buffer._runtime, y, metadata, outputs[2], None, 64, expand, False, 0, stream.cuda_stream)
+                event.current_stream_wait()
+                want, want_ow = oracle.combine(want_x, lay.recv_metadata(expand), lay.dst_slots, do_expand=expand, weights=want_w)
+                assert_same_bits(results[0], want, "every combined row is written")
+                assert_same_bits(results[1], want_ow, "every combined weight is written")
+        stream.synchronize()
+    finally:
+        deterministic.fill_uninitialized_memory = fill
+        torch.use_deterministic_algorithms(enabled, warn_only=warn_only)
+        buffer.close()
+
+
+@pytest.mark.parametrize(
+    "tokens,hidden,experts,topk,kind,expand,alignment,zero_padding,cached_iterations",
+    [
+        pytest.param(4096, 4096, 8, 2, "random", True, 1, False, 1, id="mixtral"),
+        pytest.param(4096, 7168, 256, 8, "dropout", True, 1, True, 1, id="deepseek-v3"),
+        pytest.param(32768, 7168, 32, 8, "zipf", False, 1, False, 3, id="ep8-share-cached"),
+        pytest.param(8192, 2048, 128, 8, "biased", True, 128, True, 1, id="qwen3-async"),
+    ],
+)
+def test_baseline_configs_through_the_api(device, tokens, hidden, experts, topk, kind, expand, alignment, zero_padding,
+                                          cached_iterations):
+    idx = cases.routing(kind, tokens, experts, topk, seed=11)
+    x = cases.payload(tokens, hidden)
+    logits = cases.gate_weights(tokens, topk, seed=3)
+    w = torch.softmax(logits, dim=1)
+    asynchronous = kind == "biased"
+    with Buffer(None, EPConfig(experts, topk, hidden, tokens)) as buffer:
+        side = torch.cuda.Stream() if asynchronous else torch.cuda.current_stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            x_dev, w_dev = x.to(device), w.to(device)
+            received = buffer.dispatch(x_dev, topk_idx=idx.to(device), weights=w_dev, do_expand=expand, alignment=alignment,
+                                       zero_padding=zero_padding, async_op=asynchronous)
+            if asynchronous:
+                received.event.current_stream_wait()
+            lay = assert_dispatch_result(received, x, idx, w, experts, expand, alignment, zero_padding)
+            assert_handle(received.handle, lay, expand, alignment, buffer)
+            for _ in range(cached_iterations):
+                replay = buffer.dispatch(x_dev, weights=w_dev, handle=received.handle, zero_padding=zero_padding,
+                                         async_op=asynchronous)
+                if asynchronous:
+                    replay.event.current_stream_wait()
+                assert replay.handle is received.handle
+                # identity experts apply each gate weight once (expanded) or sum the weighted copies (compact)
+                if expand:
+                    y = (replay.x.float() * replay.topk_weights[:, None]).to(torch.bfloat16)
+                else:
+                    gate = torch.where(replay.topk_idx >= 0, replay.topk_weights, torch.zeros_like(replay.topk_weights)).sum(1)
+                    y = (replay.x.float() * gate[:, None]).to(torch.bfloat16)
+                combined = buffer.combine(y, replay.handle, weights=replay.topk_weights, async_op=asynchronous)
+                if asynchronous:
+                    combined.event.current_stream_wait()
+            want, want_w = oracle.combine(y.cpu(), lay.recv_metadata(expand), lay.dst_slots, do_expand=expand,
+                                          weights=replay.topk_weights.cpu())
+            assert_same_bits(combined.x, want, "combined x")
+            assert_same_bits(combined.topk_weights, want_w, "combined weights")
+            assert_same_bits(combined.topk_weights, w.masked_fill(idx < 0, 0), "weights return to their k")
+            # size-independent property: the weighted identity round trip stays close to x
+            scale = torch.where(idx >= 0, w, torch.zeros_like(w)).sum(1, keepdim=True)
+            torch.testing.assert_close(combined.x.cpu().float(), x.float() * scale, rtol=0.03, atol=0.03)
+        torch.cuda.current_stream().wait_stream(side)
+        torch.cuda.synchronize()
