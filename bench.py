@@ -1,0 +1,248 @@
+#!/usr/bin/env python3
+"""Benchmark of the dispatch / combine hot path on one MI355X.
+
+A step is one cached-handle dispatch followed by one combine of the DeepSeek-V3-shaped batch
+(4096 tokens x 7168 bf16, 256 experts, top-8, 10% of choices masked, expanded layout with
+zero_padding) through the public API, with every input already resident in HBM.  The script prints
+ONE JSON line: whole-step achieved HBM bandwidth (algorithmic bytes / wall time), the per-kernel
+microseconds measured with HIP events on the stream the kernels run on, the roofline of the
+dominant kernel and a CPU baseline (the torch-CPU oracle timed on this host's cores).
+"""
+
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import re
+import statistics
+import sys
+import time
+from pathlib import Path
+
+ROOT = Path(__file__).resolve().parent
+if str(ROOT) not in sys.path:
+    sys.path.insert(0, str(ROOT))
+
+HBM_PEAK_GBS = 8000.0  # MI355X published HBM3E peak
+
+
+def log(*parts):
+    print(*parts, file=sys.stderr, flush=True)
+
+
+def parse_args():
+    parser = argparse.ArgumentParser(description=__doc__)
+    parser.add_argument("--gpus", type=int, default=1)
+    parser.add_argument("--steps", type=int, default=200)
+    parser.add_argument("--warmup", type=int, default=50)
+    parser.add_argument("--workload", default="deepseek-v3")
+    parser.add_argument("--cpu-seconds", type=float, default=15.0, help="CPU baseline budget; 0 skips it")
+    return parser.parse_args()
+
+
+def measured_traffic(kernel: str, workload: str):
+    """HBM bytes per launch from the committed profiler summary, if there is one."""
+    path = ROOT / "profiles" / f"{kernel}_{workload}_pmc.txt"
+    if not path.exists():
+        return None
+    match = re.search(r"^traffic_bytes_per_launch:\s*([0-9.eE+]+)", path.read_text(), flags=re.M)
+    return float(match.group(1)) if match else None
+
+
+def cpu_baseline(workload, x, idx, weights, budget_seconds):
+    """The vectorised torch-CPU oracle on the same batch: dispatch + combine, bounded in time."""
+    import torch
+
+    from nanoep_amd import workloads
+    from oracle import nanoep_oracle as oracle
+
+    cores = min(16, os.cpu_count() or 1)
+    torch.set_num_threads(cores)
+    layout = oracle.layout(idx, workload.experts, workload.alignment)
+    received, capacity = layout.recv_count, layout.expanded_capacity
+    assignments = int(layout.expert_counts.sum())
+    nbytes = workloads.dispatch_bytes(workload, received, assignments, capacity) + workloads.combine_bytes(workload, received, assignments)
+    metadata = layout.recv_metadata(workload.expand)
+
+    def step():
+        out_x, _, _, _ = oracle.dispatch(x, idx, workload.experts, weights, do_expand=workload.expand,
+                                         alignment=workload.alignment, lay=layout)
+        oracle.combine(out_x, metadata, layout.dst_slots, do_expand=workload.expand)
+
+    step()  # warm caches and the allocator
+    times = []
+    started = time.perf_counter()
+    while True:
+        t0 = time.perf_counter()
+        step()
+        times.append(time.perf_counter() - t0)
+        if time.perf_counter() - started > budget_seconds or len(times) >= 20:
+            break
+    seconds = statistics.median(times)
+    return {
+        "value": round(nbytes / seconds / 1e9, 3),
+        "unit": "GB/s",
+        "cores": cores,
+        "kind": "port",
+        "us_per_step": round(seconds * 1e6, 1),
+        "sample": f"{len(times)} timed steps (cached-layout dispatch + combine) of the full {workload.name} batch "
+                  f"with the vectorised torch-CPU oracle, {cores} threads",
+    }
+
+
+def main():
+    args = parse_args()
+    if args.gpus != 1:
+        log("bench.py measures one rank on ONE GPU; --gpus", args.gpus, "is not supported (no collectives are part of this path)")
+        return 2
+
+    import torch
+
+    from nanoep_amd import Buffer, EPConfig, workloads
+
+    if args.workload not in workloads.WORKLOADS:
+        log("unknown workload", args.workload, "choose from", sorted(workloads.WORKLOADS))
+        return 2
+    workload = workloads.WORKLOADS[args.workload]
+    device = torch.device("cuda", 0)
+    torch.cuda.set_device(device)
+
+    rotation = 4
+    batches = [workloads.make_inputs(workload, seed=seed) for seed in range(rotation)]
+    x_cpu, idx_cpu, w_cpu = batches[0]
+    xs = [batch[0].to(device) for batch in batches]
+    idx = idx_cpu.to(device)
+    weights = w_cpu.to(device)
+
+    buffer = Buffer(None, EPConfig(workload.experts, workload.topk, workload.hidden, workload.tokens))
+    stream = buffer.comm_stream  # run the loop on the stream the kernels are launched on
+    result = {}
+    with torch.cuda.stream(stream):
+        # fresh dispatch: layout kernels + host wait for N/C + permute, as seen by the caller
+        fresh_times = []
+        for _ in range(10):
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            received = buffer.dispatch(xs[0], topk_idx=idx, weights=weights, do_expand=workload.expand,
+                                       alignment=workload.alignment, zero_padding=workload.zero_padding)
+            torch.cuda.synchronize()
+            fresh_times.append(time.perf_counter() - t0)
+        handle = received.handle
+        n_recv, capacity = handle.layout.recv_count, handle.layout.expanded_capacity
+        assignments = int(handle.layout.expert_counts.sum().item())
+        d_bytes = workloads.dispatch_bytes(workload, n_recv, assignments, capacity)
+        c_bytes = workloads.combine_bytes(workload, n_recv, assignments)
+
+        ring = [received.x, received.x.clone(), received.x.clone()]  # combine reads a two-steps-old dispatch output
+
+        def do_dispatch(i):
+            out = buffer.dispatch(xs[i % rotation], weights=weights, handle=handle, zero_padding=workload.zero_padding)
+            ring[i % 3] = out.x
+
+        def do_combine(i):
+            return buffer.combine(ring[(i + 1) % 3], handle)
+
+        def step(i):
+            do_dispatch(i)
+            return do_combine(i)
+
+        def timed(fn, count):
+            """(wall seconds, GPU seconds between two HIP events on the kernels' stream) of `count` calls."""
+            begin, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            begin.record(stream)
+            for i in range(count):
+                fn(i)
+            end.record(stream)
+            torch.cuda.synchronize()
+            return time.perf_counter() - t0, begin.elapsed_time(end) * 1e-3
+
+        for i in range(args.warmup):
+            step(i)
+        wall, gpu_step_seconds = timed(step, args.steps)
+        # the two kernels on their own, back to back, for the per-kernel rooflines
+        timed(do_dispatch, max(1, args.warmup // 2))
+        _, gpu_dispatch_seconds = timed(do_dispatch, args.steps)
+        timed(do_combine, max(1, args.warmup // 2))
+        _, gpu_combine_seconds = timed(do_combine, args.steps)
+
+    ms_per_step = wall / args.steps * 1e3
+    d_us = gpu_dispatch_seconds / args.steps * 1e6
+    c_us = gpu_combine_seconds / args.steps * 1e6
+    value = (d_bytes + c_bytes) / (ms_per_step * 1e-3) / 1e9
+    result.update(
+        {
+            "metric": "dispatch+combine achieved HBM bandwidth (algorithmic bytes / wall time), 4096x7168 bf16, 256 experts top-8",
+            "value": round(value, 1),
+            "unit": "GB/s",
+            "n_gpus": 1,
+            "steps": args.steps,
+            "warmup": args.warmup,
+            "ms_per_step": round(ms_per_step, 5),
+            "higher_is_better": True,
+            "scaling": "weak",
+            "vs_baseline": None,
+            "dtype": "f32",
+            "payload_dtype": "bf16",
+            "data": "synthetic",
+            "config": {
+                "workload": workload.name,
+                "description": workload.description,
+                "tokens": workload.tokens,
+                "hidden": workload.hidden,
+                "experts": workload.experts,
+                "topk": workload.topk,
+                "layout": "expanded" if workload.expand else "compact",
+                "alignment": workload.alignment,
+                "zero_padding": workload.zero_padding,
+                "received_rows": n_recv,
+                "assignments": assignments,
+                "expanded_capacity": capacity,
+                "step": "cached-handle dispatch + combine through Buffer.dispatch / Buffer.combine",
+            },
+            "frac_of_hbm_peak": round(value / HBM_PEAK_GBS, 4),
+            "gpu_us_per_step": round(gpu_step_seconds / args.steps * 1e6, 2),
+            "dispatch_us": round(d_us, 2),
+            "dispatch_GBps": round(d_bytes / d_us / 1e3, 1),
+            "combine_us": round(c_us, 2),
+            "combine_GBps": round(c_bytes / c_us / 1e3, 1),
+            "fresh_dispatch_us_host": round(statistics.median(fresh_times) * 1e6, 1),
+            "dispatch_bytes": d_bytes,
+            "combine_bytes": c_bytes,
+            "roofline": {
+                "kernel": "dispatch_rows_kernel",
+                "bound": "hbm",
+                "achieved": round(d_bytes / d_us / 1e3, 1),
+                "peak": HBM_PEAK_GBS,
+                "unit": "GB/s",
+                "frac": round(d_bytes / d_us / 1e3 / HBM_PEAK_GBS, 4),
+                "traffic": measured_traffic("dispatch_rows_kernel", workload.name),
+                "algorithmic_bytes": d_bytes,
+                "avg_us": round(d_us, 2),
+            },
+            "roofline_combine": {
+                "kernel": "combine_rows_kernel",
+                "bound": "hbm",
+                "achieved": round(c_bytes / c_us / 1e3, 1),
+                "peak": HBM_PEAK_GBS,
+                "unit": "GB/s",
+                "frac": round(c_bytes / c_us / 1e3 / HBM_PEAK_GBS, 4),
+                "traffic": measured_traffic("combine_rows_kernel", workload.name),
+                "algorithmic_bytes": c_bytes,
+                "avg_us": round(c_us, 2),
+            },
+        }
+    )
+    buffer.close()
+    del xs, ring
+    torch.cuda.empty_cache()
+    if args.cpu_seconds > 0:
+        result["cpu_baseline"] = cpu_baseline(workload, x_cpu, idx_cpu, w_cpu, args.cpu_seconds)
+    print(json.dumps(result), flush=True)
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())

@@ -339,6 +339,11 @@ class CudaBuffer:
 
         return NativeCombineResult(x=outputs[0], topk_weights=outputs[1] if weights is not None else None, event=event)
 
+    @property
+    def comm_stream(self) -> torch.cuda.Stream:
+        """The stream dispatch and combine kernels are launched on."""
+        return self._comm_stream
+
     def close(self):
         """Drain the GPU and release the runtime.  Idempotent; dispatch/combine fail afterwards."""
         if self._closed:
