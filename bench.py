@@ -38,6 +38,8 @@ def parse_args():
     parser.add_argument("--warmup", type=int, default=50)
     parser.add_argument("--workload", default="deepseek-v3")
     parser.add_argument("--cpu-seconds", type=float, default=15.0, help="CPU baseline budget; 0 skips it")
+    parser.add_argument("--calibration-copy-mib", type=int, default=0,
+                        help="also launch the plain copy kernel on this many MiB (known-size reference for profiler byte counters)")
     return parser.parse_args()
 
 
@@ -235,6 +237,22 @@ def main():
             },
         }
     )
+    if args.calibration_copy_mib > 0:
+        import ctypes
+
+        library = ctypes.CDLL(str(ROOT / "nanoep_amd" / "libnanoep_hip.so"))
+        library.nanoep_copy_bytes.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_size_t, ctypes.c_void_p]
+        nbytes = args.calibration_copy_mib << 20
+        source = torch.full((nbytes,), 3, dtype=torch.uint8, device=device)
+        target = torch.empty_like(source)
+        torch.cuda.synchronize()
+        for _ in range(3):
+            status = library.nanoep_copy_bytes(source.data_ptr(), target.data_ptr(), nbytes, torch.cuda.current_stream().cuda_stream)
+            assert status == 0, status
+        torch.cuda.synchronize()
+        assert torch.equal(source[:4096], target[:4096])
+        result["calibration_copy_bytes"] = nbytes
+        del source, target
     buffer.close()
     del xs, ring
     torch.cuda.empty_cache()

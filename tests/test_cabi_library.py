@@ -1,0 +1,67 @@
+"""The C-ABI library loads without a GPU, exports every symbol the header declares, and its pure
+or argument-checking entry points behave (no compute call is made here)."""
+
+import ctypes
+
+import pytest
+
+import cabi
+from oracle import nanoep_oracle as oracle
+
+
+def test_every_declared_symbol_is_exported():
+    declared = cabi.declared_symbols()
+    assert {"nanoep_layout", "nanoep_dispatch", "nanoep_combine", "nanoep_wait_counts", "nanoep_window_layout",
+            "nanoep_layout_workspace_bytes", "nanoep_copy_bytes", "nanoep_abi_version"} <= set(declared)
+    library = cabi.lib()
+    for name in declared:
+        assert hasattr(library, name), f"{name} is declared in include/nanoep_hip.h but not exported"
+
+
+def test_version_and_status_strings():
+    library = cabi.lib()
+    assert library.nanoep_abi_version() == 1
+    texts = [library.nanoep_status_string(code).decode() for code in range(0, 7)]
+    assert texts[0] == "ok" and len(set(texts[:6])) == 6 and texts[6] == "unknown status"
+    assert library.nanoep_last_hip_error().decode() == ""
+
+
+@pytest.mark.parametrize("args", [(2, 8, 256, 2, 4, False), (1, 16, 256, 2, 2, False), (8, 4096, 7168, 8, 256, True),
+                                  (4, 5, 512, 3, 12, True), (1, 32768, 7168, 8, 32, False)])
+def test_window_layout_matches_the_oracle(args):
+    assert cabi.window_layout(*args) == oracle.window_layout(*args)
+
+
+def test_window_layout_known_answer_and_errors():
+    assert cabi.window_layout(2, 8, 256, 2, 4) == [0, 96, 160, 160, 9888]
+    out = (ctypes.c_int64 * 5)()
+    library = cabi.lib()
+    for bad in ((0, 8, 256, 2, 4), (33, 8, 256, 2, 64), (2, 0, 256, 2, 4), (2, 8, 0, 2, 4), (2, 8, 256, 33, 4), (2, 8, 256, 2, 5)):
+        assert library.nanoep_window_layout(*bad, 0, out) == 1
+
+
+def test_workspace_size_grows_with_the_problem():
+    library = cabi.lib()
+    small = library.nanoep_layout_workspace_bytes(16, 2, 2)
+    large = library.nanoep_layout_workspace_bytes(4096, 8, 256)
+    assert 0 < small < large
+    assert large >= 4096 * 8 * 4 + 4096 * 4 + (4096 // 256) * 257 * 4
+    assert library.nanoep_layout_workspace_bytes(-1, 8, 256) == 0
+    assert library.nanoep_layout_workspace_bytes(16, 0, 2) == 0
+
+
+def test_argument_checks_come_before_any_device_work():
+    library = cabi.lib()
+    null = None
+    # hidden not a multiple of 8, top-k out of range, negative counts, unaligned pointers
+    assert library.nanoep_dispatch(null, null, null, null, null, null, null, 0, 0, 0, 7, 2, 4, 1, 0, 0, null, null, null, 0, null) == 1
+    assert library.nanoep_dispatch(null, null, null, null, null, null, null, 0, 0, 0, 256, 33, 4, 1, 0, 0, null, null, null, 0, null) == 1
+    assert library.nanoep_dispatch(null, null, null, null, null, null, null, 5, 0, 4, 256, 2, 4, 1, 0, 0, null, null, null, 0, null) == 1
+    assert library.nanoep_dispatch(8, null, null, null, null, null, null, 0, 0, 0, 256, 2, 4, 1, 0, 0, null, null, null, 0, null) == 1
+    assert library.nanoep_combine(null, null, null, null, null, null, 0, 0, 0, 250, 2, 1, 0, null, null, 0, null) == 1
+    assert library.nanoep_combine(null, null, null, null, null, null, 3, 0, 2, 256, 2, 1, 0, null, null, 0, null) == 1
+    assert library.nanoep_copy_bytes(null, null, 24, null) == 1
+    assert library.nanoep_layout(null, -1, 2, 4, 1, 0, null, null, null, null, null, null, null, null, null, 0, null, null) == 1
+    assert library.nanoep_layout(null, 4, 2, 4, 0, 0, null, null, null, null, null, null, null, null, null, 0, null, null) == 1
+    out = (ctypes.c_int64 * 4)()
+    assert library.nanoep_wait_counts(null, null, 0.0, out) == 1

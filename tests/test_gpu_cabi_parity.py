@@ -254,6 +254,18 @@ def test_special_values_survive_dispatch_and_round_in_combine(device):
     assert torch.equal(bits(got_cpu)[~nan], bits(want)[~nan])
 
 
+def test_accumulation_is_fp32_in_ascending_k(device):
+    """((0 + 2^30) - 2^30) + 64 = 64 only when rows are added in ascending k in fp32; 256 + 1 - 256 = 1
+    only with an fp32 accumulator."""
+    idx = torch.tensor([[0, 1, 2]], dtype=torch.int64)
+    metadata, counts = cabi.layout(idx.to(device), 3, 1, True)
+    for rows, want in (([2.0**30, -(2.0**30), 64.0], 64.0), ([64.0, 2.0**30, -(2.0**30)], 0.0), ([256.0, 1.0, -256.0], 1.0)):
+        y = torch.tensor(rows, dtype=torch.bfloat16).reshape(3, 1).repeat(1, 256).contiguous()
+        for use_table in (True, False):
+            got, _ = cabi.combine(y.to(device), None, None, metadata, counts, True, use_table=use_table)
+            assert (got.float().cpu() == want).all(), (rows, use_table)
+
+
 def test_reversed_handle_order_is_honoured(device):
     """Combine must follow the handle, not assume token-ordered slots (the reference's
     expert_inputs builds handles with reversed receive and slot order)."""
