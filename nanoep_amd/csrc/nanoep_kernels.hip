@@ -71,7 +71,7 @@ int env_int(const char* name, int fallback) {
 int layout_tokens_per_block(int64_t local_experts) {
     for (int tokens = 256; tokens >= 32; tokens /= 2) {
         const size_t words = static_cast<size_t>(tokens / 32);
-        if (static_cast<size_t>(local_experts + 1) * words * 6 <= kLayoutLdsBudget)
+        if (static_cast<size_t>(local_experts + 1) * (words * 6 + 4) <= kLayoutLdsBudget)
             return tokens;
     }
     return 0;
@@ -118,11 +118,13 @@ __global__ void layout_count_kernel(const int64_t* __restrict__ topk_idx,
                                     int32_t* __restrict__ local_row) {
     extern __shared__ uint32_t layout_lds[];
     const int rows = local_experts + 1;
+    // bit rows are words + 1 apart: an odd stride spreads the experts a wavefront touches over the LDS banks
+    const int stride = words + 1;
     uint32_t* bits = layout_lds;
-    auto* prefix = reinterpret_cast<uint16_t*>(bits + static_cast<size_t>(rows) * words);
+    auto* prefix = reinterpret_cast<uint16_t*>(bits + static_cast<size_t>(rows) * stride);
     __shared__ int block_bad;
 
-    for (int i = threadIdx.x; i < rows * words; i += blockDim.x)
+    for (int i = threadIdx.x; i < rows * stride; i += blockDim.x)
         bits[i] = 0;
     if (threadIdx.x == 0)
         block_bad = 0;
@@ -142,7 +144,7 @@ __global__ void layout_count_kernel(const int64_t* __restrict__ topk_idx,
             const int64_t expert = topk_idx[token * num_topk + k];
             snapshot[token * num_topk + k] = expert;
             if (expert >= 0 && expert < local_experts) {
-                const uint32_t old = atomicOr(&bits[static_cast<size_t>(expert) * words + word], bit);
+                const uint32_t old = atomicOr(&bits[static_cast<size_t>(expert) * stride + word], bit);
                 if (old & bit)
                     bad |= NANOEP_ROUTING_DUPLICATE;
                 any = true;
@@ -151,7 +153,7 @@ __global__ void layout_count_kernel(const int64_t* __restrict__ topk_idx,
             }
         }
         if (any)
-            atomicOr(&bits[static_cast<size_t>(local_experts) * words + word], bit);
+            atomicOr(&bits[static_cast<size_t>(local_experts) * stride + word], bit);
         if (bad)
             atomicOr(&block_bad, bad);
     }
@@ -161,7 +163,7 @@ __global__ void layout_count_kernel(const int64_t* __restrict__ topk_idx,
         int running = 0;
         for (int w = 0; w < words; ++w) {
             prefix[static_cast<size_t>(row) * words + w] = static_cast<uint16_t>(running);
-            running += __popc(bits[static_cast<size_t>(row) * words + w]);
+            running += __popc(bits[static_cast<size_t>(row) * stride + w]);
         }
         block_counts[static_cast<int64_t>(blockIdx.x) * rows + row] = running;
     }
@@ -175,13 +177,13 @@ __global__ void layout_count_kernel(const int64_t* __restrict__ topk_idx,
             const int64_t expert = topk_idx[token * num_topk + k];
             int rank = -1;
             if (expert >= 0 && expert < local_experts) {
-                const size_t at = static_cast<size_t>(expert) * words + word;
-                rank = prefix[at] + __popc(bits[at] & below);
+                rank = prefix[static_cast<size_t>(expert) * words + word] +
+                       __popc(bits[static_cast<size_t>(expert) * stride + word] & below);
             }
             local_rank[token * num_topk + k] = rank;
         }
-        const size_t at = static_cast<size_t>(local_experts) * words + word;
-        local_row[token] = (bits[at] & bit) ? prefix[at] + __popc(bits[at] & below) : -1;
+        const uint32_t received = bits[static_cast<size_t>(local_experts) * stride + word];
+        local_row[token] = (received & bit) ? prefix[static_cast<size_t>(local_experts) * words + word] + __popc(received & below) : -1;
     }
 }
 
@@ -789,7 +791,7 @@ int nanoep_layout(const int64_t* topk_idx, int64_t num_tokens, int num_topk, int
     __atomic_store_n(&host_counts[0], int64_t{-1}, __ATOMIC_RELEASE);
     const int count_threads = tokens_per_block < kWave ? kWave : tokens_per_block;
     if (blocks > 0) {
-        const size_t lds = static_cast<size_t>(experts + 1) * words * 6;
+        const size_t lds = static_cast<size_t>(experts + 1) * (words * 6 + 4);
         layout_count_kernel<<<blocks, count_threads, lds, stream>>>(topk_idx, num_tokens, num_topk, experts, words,
                                                                      topk_snapshot, ws.block_counts, ws.block_status,
                                                                      ws.local_rank, ws.local_row);

@@ -242,12 +242,29 @@ const int32_t* slot_table(const std::vector<torch::Tensor>& metadata, int64_t to
 
 // Communication stream waits for the producer of the inputs: the caller's stream, an explicit
 // event, or both (csrc/pipeline.cu:364-377 in the reference).
+// An external-stream wrapper never compares equal to a pool stream object, so identity is decided
+// on the raw handles: when the caller already runs on the communication stream no event is needed.
+bool same_queue(const Stream& a, const Stream& b) { return a.stream() == b.stream(); }
+
+// Stream the kernels are enqueued on.  An asynchronous call uses the buffer's communication stream.
+// A synchronous call must leave its results ordered on the caller's stream, so it runs there
+// directly instead of bouncing through the communication stream with two cross-stream events; it
+// still comes after everything enqueued earlier on the communication stream.
+Stream work_stream(int64_t comm_handle, const Stream& compute, c10::DeviceIndex device, bool async_op) {
+    const auto comm = external_stream(comm_handle, device);
+    if (async_op || same_queue(comm, compute))
+        return comm;
+    if (hipStreamQuery(comm.stream()) == hipErrorNotReady)
+        wait_on(compute, comm);
+    return compute;
+}
+
 void order_comm_after_inputs(const Stream& comm, const Stream& compute, int64_t previous_event, bool async_op) {
     if (previous_event != -1) {
-        if (!async_op && comm != compute)
+        if (!async_op && !same_queue(comm, compute))
             wait_on(comm, compute);
         check_hip(hipStreamWaitEvent(comm.stream(), reinterpret_cast<hipEvent_t>(previous_event), 0), "hipStreamWaitEvent");
-    } else if (comm != compute) {
+    } else if (!same_queue(comm, compute)) {
         wait_on(comm, compute);
     }
 }
@@ -290,7 +307,7 @@ DispatchResult dispatch(PeerRuntime& runtime,
     const int64_t local_experts = num_experts;
 
     const auto compute = c10::hip::getCurrentHIPStreamMasqueradingAsCUDA(device);
-    const auto comm = external_stream(comm_stream, device);
+    const auto comm = work_stream(comm_stream, compute, device, async_op);
     order_comm_after_inputs(comm, compute, previous_event, async_op);
 
     StreamGuard comm_guard(comm.unwrap());
@@ -395,7 +412,7 @@ DispatchResult dispatch(PeerRuntime& runtime,
         auto protected_tensors = outputs;
         protected_tensors.insert(protected_tensors.end(), metadata.begin(), metadata.end());
         event = std::make_shared<CompletionEvent>(comm, std::move(protected_tensors));
-    } else if (comm != compute) {
+    } else if (!same_queue(comm, compute)) {
         wait_on(compute, comm);
     }
     return std::make_tuple(std::move(outputs), std::move(metadata), std::array<int64_t, 2>{recv_count, expanded_capacity}, std::move(event));
@@ -452,7 +469,7 @@ CombineResult combine(PeerRuntime& runtime,
     const int cu_budget = resolve_cu_budget(num_sms, device);
 
     const auto compute = c10::hip::getCurrentHIPStreamMasqueradingAsCUDA(device);
-    const auto comm = external_stream(comm_stream, device);
+    const auto comm = work_stream(comm_stream, compute, device, async_op);
     order_comm_after_inputs(comm, compute, previous_event, async_op);
     StreamGuard comm_guard(comm.unwrap());
 
@@ -488,7 +505,7 @@ CombineResult combine(PeerRuntime& runtime,
             if (tensor.numel() > 0)
                 tensor.record_stream(comm.unwrap());
         event = std::make_shared<CompletionEvent>(comm, outputs);
-    } else if (comm != compute) {
+    } else if (!same_queue(comm, compute)) {
         wait_on(compute, comm);
     }
     return std::make_tuple(std::move(outputs), std::move(event));

@@ -53,7 +53,6 @@ def run_dispatch_combine(device, idx, hidden, experts, alignment, expand, zero_p
     expected_layout = oracle.layout(idx, experts, alignment)
     metadata, counts = cabi.layout(idx.to(device), experts, alignment, expand)
     assert_layout(metadata, counts, expected_layout, expand)
-
     want_x, want_idx, want_w, _ = oracle.dispatch(x, idx, experts, w, do_expand=expand, alignment=alignment, lay=expected_layout)
     got_x, got_idx, got_w = cabi.dispatch(
         x.to(device), None if w is None else w.to(device), metadata, counts, experts, alignment, expand, zero_padding,
