@@ -573,13 +573,16 @@ __global__ void __launch_bounds__(1024) combine_rows_kernel(const u32x4* __restr
         received = row >= 0 && row < recv_count;
         fields = recv_metadata + (received ? row : 0) * (num_topk + 2) + 2;
     }
+    // Compact rows need their per-k fields only to return weights: a received row always carries
+    // at least one valid choice, so the payload path skips that dependent load.
+    const bool need_fields = expand || (chunk == 0 && out_weights != nullptr);
     int field = -1;
-    if (received && lane < num_topk)
+    if (need_fields && received && lane < num_topk)
         field = fields[lane];
     const bool valid = expand ? (field >= 0 && field < y_rows) : field >= 0;
     const uint64_t valid_mask = __ballot(valid);
     // compact: the token's single received row stands in for k = 0
-    const uint64_t gather_mask = expand ? valid_mask : (valid_mask != 0 ? 1ull : 0ull);
+    const uint64_t gather_mask = expand ? valid_mask : ((received && row < y_rows) ? 1ull : 0ull);
     const int gathered = gather_mask == 0 ? 0 : (expand ? num_topk : 1);
 
     u32x4 bias_data = {0u, 0u, 0u, 0u};

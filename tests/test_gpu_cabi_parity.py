@@ -292,6 +292,26 @@ def test_reversed_handle_order_is_honoured(device):
         want, want_w = oracle.combine_scalar(y, meta, dst, do_expand=expand, weights=w)
         assert_bits_equal(got, want, "reversed handle x")
         assert_bits_equal(got_w, want_w, "reversed handle weights")
+        # cached dispatch follows the same handle: every row lands where the metadata says
+        x = cases.payload(11, 256, seed=6)
+        xw = cases.gate_weights(11, 3, seed=8)
+        metadata = [meta.to(device), lay.expert_counts.to(device), lay.expert_offsets.to(device), dst.to(device)]
+        got_x, got_idx, got_xw = cabi.dispatch(x.to(device), xw.to(device), metadata, counts, 3, 4, expand, True)
+        got_x, got_xw = got_x.cpu(), got_xw.cpu()
+        for row, token in enumerate(tokens.tolist()):
+            if expand:
+                for k in range(3):
+                    slot = int(slots[row, k])
+                    if slot >= 0:
+                        assert torch.equal(got_x[slot].view(torch.int16), x[token].view(torch.int16))
+                        assert got_xw[slot] == xw[token, k]
+            else:
+                assert torch.equal(got_x[row].view(torch.int16), x[token].view(torch.int16))
+                assert torch.equal(got_xw[row], xw[token]) and torch.equal(got_idx.cpu()[row], local[row])
+        if expand:
+            live = torch.zeros(lay.expanded_capacity, dtype=torch.bool)
+            live[slots[slots >= 0]] = True
+            assert (got_x[~live].view(torch.int16) == 0).all() and (got_xw[~live] == 0).all()
 
 
 def test_window_layout_known_answer():
