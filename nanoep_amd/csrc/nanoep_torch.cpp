@@ -254,7 +254,11 @@ Stream work_stream(int64_t comm_handle, const Stream& compute, c10::DeviceIndex 
     const auto comm = external_stream(comm_handle, device);
     if (async_op || same_queue(comm, compute))
         return comm;
-    if (hipStreamQuery(comm.stream()) == hipErrorNotReady)
+    // While the caller's stream is being captured into a graph no other stream may be queried;
+    // a captured call is ordered by the graph alone.
+    hipStreamCaptureStatus capture = hipStreamCaptureStatusNone;
+    check_hip(hipStreamIsCapturing(compute.stream(), &capture), "hipStreamIsCapturing");
+    if (capture == hipStreamCaptureStatusNone && hipStreamQuery(comm.stream()) == hipErrorNotReady)
         wait_on(compute, comm);
     return compute;
 }

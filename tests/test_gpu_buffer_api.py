@@ -404,3 +404,44 @@ def test_baseline_configs_through_the_api(device, tokens, hidden, experts, topk,
             torch.testing.assert_close(combined.x.cpu().float(), x.float() * scale, rtol=0.03, atol=0.03)
         torch.cuda.current_stream().wait_stream(side)
         torch.cuda.synchronize()
+
+
+def test_cached_dispatch_and_combine_replay_in_a_hip_graph(device):
+    """Cached dispatch and combine launch one kernel each and wait on nothing, so they can be
+    captured; every replay (with eager work and synchronisations in between) matches eager results.
+    Fresh dispatch polls the host for N/C and must refuse capture."""
+    tokens, experts, topk, hidden = 512, 32, 4, 2048
+    idx = cases.routing("dropout", tokens, experts, topk, seed=21)
+    w = cases.gate_weights(tokens, topk).to(device)
+    with Buffer(None, EPConfig(experts, topk, hidden, tokens)) as buffer:
+        static_x = cases.payload(tokens, hidden, seed=1).to(device)
+        fresh = buffer.dispatch(static_x, topk_idx=idx.to(device), weights=w, do_expand=True, alignment=16, zero_padding=True)
+        handle = fresh.handle
+        torch.cuda.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            replay = buffer.dispatch(static_x, weights=w, handle=handle, zero_padding=True)
+            expert_x = (replay.x.float() * replay.topk_weights[:, None]).to(torch.bfloat16)
+            combined = buffer.combine(expert_x, handle, weights=replay.topk_weights)
+        for step in range(4):
+            new_x = cases.payload(tokens, hidden, seed=100 + step).to(device)
+            static_x.copy_(new_x)
+            graph.replay()
+            torch.cuda.synchronize()
+            eager = buffer.dispatch(new_x, weights=w, handle=handle, zero_padding=True)
+            eager_y = (eager.x.float() * eager.topk_weights[:, None]).to(torch.bfloat16)
+            eager_combined = buffer.combine(eager_y, handle, weights=eager.topk_weights)
+            torch.cuda.synchronize()
+            assert_same_bits(replay.x, eager.x.cpu(), f"graph replay {step}: dispatched rows")
+            assert_same_bits(combined.x, eager_combined.x.cpu(), f"graph replay {step}: combined rows")
+            assert_same_bits(combined.topk_weights, eager_combined.topk_weights.cpu(), f"graph replay {step}: weights")
+        idx_dev = idx.to(device)
+        torch.cuda.synchronize()
+        probe = torch.cuda.CUDAGraph()
+        with pytest.raises(RuntimeError, match="captured"):
+            with torch.cuda.graph(probe):
+                buffer.dispatch(static_x, topk_idx=idx_dev, weights=w, do_expand=True)
+        torch.cuda.synchronize()
+        # the buffer still works after the refused capture
+        again = buffer.dispatch(static_x, topk_idx=idx_dev, weights=w, do_expand=True, alignment=16, zero_padding=True)
+        assert again.handle.layout.expanded_capacity == handle.layout.expanded_capacity
