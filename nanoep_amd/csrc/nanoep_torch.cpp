@@ -324,6 +324,30 @@ DispatchResult dispatch(PeerRuntime& runtime,
         return make();
     };
 
+    const auto float_options = x.options().dtype(torch::kFloat32);
+    torch::Tensor out_x, out_indices, out_weights;
+    // x_rows rows of payload (and expanded weights), n_rows rows of compact indices / weights
+    const auto allocate_outputs = [&](int64_t x_rows, int64_t n_rows) {
+        allocate_for_consumer([&] {
+            out_x = torch::empty({x_rows, hidden}, x.options());
+            out_indices = expand ? torch::empty({0}, routing.options()) : torch::empty({n_rows, topk}, routing.options());
+            out_weights = !weights.has_value() ? torch::empty({0}, float_options)
+                          : expand            ? torch::empty({x_rows}, float_options)
+                                              : torch::empty({n_rows, topk}, float_options);
+            return 0;
+        });
+    };
+    const auto launch_permute = [&](const std::vector<torch::Tensor>& handle, int64_t received, int64_t capacity) {
+        check_status(
+            nanoep_dispatch(x.data_ptr(), weights.has_value() ? weights->data_ptr<float>() : nullptr, handle[0].data_ptr<int32_t>(),
+                            handle[3].data_ptr<int64_t>(), slot_table(handle, tokens, topk, expand), handle[1].data_ptr<int64_t>(),
+                            handle[2].data_ptr<int64_t>(), received, capacity, tokens, static_cast<int>(hidden),
+                            static_cast<int>(topk), local_experts, alignment, expand ? 1 : 0, zero_padding ? 1 : 0, out_x.data_ptr(),
+                            expand ? nullptr : out_indices.data_ptr<int64_t>(),
+                            weights.has_value() ? out_weights.data_ptr<float>() : nullptr, cu_budget, comm.stream()),
+            "dispatch");
+    };
+
     std::vector<torch::Tensor> metadata;
     int64_t recv_count = 0;
     int64_t expanded_capacity = 0;
@@ -333,6 +357,11 @@ DispatchResult dispatch(PeerRuntime& runtime,
         recv_count = cached_metadata[0].size(0);
         expanded_capacity = cached_expanded_capacity;
         TORCH_CHECK(recv_count <= tokens && expanded_capacity >= 0, "cached handle does not match the payload");
+        TORCH_CHECK(!expand || expanded_capacity <= std::numeric_limits<int32_t>::max(),
+                    "expanded capacity exceeds int32 metadata range");
+        allocate_outputs(expand ? expanded_capacity : recv_count, recv_count);
+        if (recv_count > 0)
+            launch_permute(metadata, recv_count, expanded_capacity);
     } else {
         hipStreamCaptureStatus capture = hipStreamCaptureStatusNone;
         check_hip(hipStreamIsCapturing(comm.stream(), &capture), "hipStreamIsCapturing");
@@ -352,6 +381,9 @@ DispatchResult dispatch(PeerRuntime& runtime,
                 token_slots = torch::empty({tokens, topk}, int64_options.dtype(torch::kInt32));
             return 0;
         });
+        metadata = {recv_metadata, expert_counts, expert_offsets, dst_slots, send_counts, snapshot, prefix};
+        if (expand)
+            metadata.push_back(token_slots);  // private eighth entry: slot[t,k] in one lookup
         const size_t workspace_bytes = nanoep_layout_workspace_bytes(tokens, static_cast<int>(topk), local_experts);
         TORCH_CHECK(workspace_bytes > 0, "unsupported routing geometry for the layout kernels");
         auto workspace = torch::empty({static_cast<int64_t>(workspace_bytes)}, int64_options.dtype(torch::kUInt8));
@@ -362,6 +394,21 @@ DispatchResult dispatch(PeerRuntime& runtime,
                                    expand ? token_slots.data_ptr<int32_t>() : nullptr, workspace.data_ptr(), workspace_bytes,
                                    host_counts, comm.stream()),
                      "layout");
+
+        // The exact shapes (N, C) are only known once the layout kernels have run.  Waiting for
+        // them before launching the permute would leave the GPU idle for a host round trip, so the
+        // outputs are allocated at their upper bound (every choice valid plus every expert's worst
+        // alignment gap), the permute is enqueued right behind the layout, and the results are
+        // narrowed to the exact shapes afterwards.  When the bound is far above what routing can
+        // need (huge alignments) the exact-allocation order is kept.
+        const int64_t gap_bound = expand ? local_experts * (alignment - 1) : 0;
+        const int64_t row_bound = expand ? tokens * topk + gap_bound : tokens;
+        const bool speculative = tokens > 0 && gap_bound <= tokens * topk / 4 + 1024 && row_bound <= std::numeric_limits<int32_t>::max();
+        if (speculative) {
+            allocate_outputs(row_bound, tokens);
+            launch_permute(metadata, tokens, row_bound);
+        }
+
         int64_t counts[NANOEP_HOST_COUNT_WORDS] = {0, 0, 0, 0};
         const int status = nanoep_wait_counts(host_counts, comm.stream(), kCountTimeoutSeconds, counts);
         if (status == NANOEP_ERR_ROUTING) {
@@ -373,32 +420,21 @@ DispatchResult dispatch(PeerRuntime& runtime,
         recv_count = counts[0];
         expanded_capacity = counts[1];
         TORCH_CHECK(recv_count >= 0 && recv_count <= tokens, "dispatch receive count exceeds the source token count");
-        metadata = {recv_metadata.narrow(0, 0, recv_count), expert_counts, expert_offsets, dst_slots, send_counts, snapshot, prefix};
-        if (expand)
-            metadata.push_back(token_slots);  // private eighth entry: slot[t,k] in one lookup
-    }
-    TORCH_CHECK(!expand || expanded_capacity <= std::numeric_limits<int32_t>::max(), "expanded capacity exceeds int32 metadata range");
-
-    const int64_t rows = expand ? expanded_capacity : recv_count;
-    torch::Tensor out_x, out_indices, out_weights;
-    allocate_for_consumer([&] {
-        out_x = torch::empty({rows, hidden}, x.options());
-        out_indices = expand ? torch::empty({0}, routing.options()) : torch::empty({recv_count, topk}, routing.options());
-        out_weights = !weights.has_value() ? torch::empty({0}, x.options().dtype(torch::kFloat32))
-                      : expand            ? torch::empty({expanded_capacity}, x.options().dtype(torch::kFloat32))
-                                          : torch::empty({recv_count, topk}, x.options().dtype(torch::kFloat32));
-        return 0;
-    });
-
-    if (recv_count > 0) {
-        check_status(
-            nanoep_dispatch(x.data_ptr(), weights.has_value() ? weights->data_ptr<float>() : nullptr, metadata[0].data_ptr<int32_t>(),
-                            metadata[3].data_ptr<int64_t>(), slot_table(metadata, tokens, topk, expand), metadata[1].data_ptr<int64_t>(),
-                            metadata[2].data_ptr<int64_t>(), recv_count, expanded_capacity, tokens,
-                            static_cast<int>(hidden), static_cast<int>(topk), local_experts, alignment, expand ? 1 : 0,
-                            zero_padding ? 1 : 0, out_x.data_ptr(), expand ? nullptr : out_indices.data_ptr<int64_t>(),
-                            weights.has_value() ? out_weights.data_ptr<float>() : nullptr, cu_budget, comm.stream()),
-            "dispatch");
+        TORCH_CHECK(!expand || expanded_capacity <= std::numeric_limits<int32_t>::max(),
+                    "expanded capacity exceeds int32 metadata range");
+        metadata[0] = recv_metadata.narrow(0, 0, recv_count);
+        if (speculative) {
+            TORCH_CHECK(!expand || expanded_capacity <= row_bound, "expanded capacity exceeds its upper bound");
+            out_x = out_x.narrow(0, 0, expand ? expanded_capacity : recv_count);
+            if (!expand)
+                out_indices = out_indices.narrow(0, 0, recv_count);
+            if (weights.has_value())
+                out_weights = out_weights.narrow(0, 0, expand ? expanded_capacity : recv_count);
+        } else {
+            allocate_outputs(expand ? expanded_capacity : recv_count, recv_count);
+            if (recv_count > 0)
+                launch_permute(metadata, recv_count, expanded_capacity);
+        }
     }
 
     std::vector<torch::Tensor> outputs{out_x, out_indices, out_weights};
