@@ -11,9 +11,11 @@
 //   layout_count_kernel  : one workgroup per block of tokens; LDS bit matrix (expert x token) built
 //                          with LDS atomics, popcount prefixes give the in-block stable rank of
 //                          every (token,k) and the block's per-expert histogram.
-//   layout_scan_kernel   : one workgroup; exclusive scan of the block histograms per expert, then the
-//                          aligned exclusive scan over experts; publishes N, C to the host mailbox.
-//   layout_assign_kernel : slot = offset[e] + block_base[b][e] + in-block rank; writes the handle.
+//   layout_scan_assign_kernel : (few blocks) every workgroup sums the block histograms into LDS,
+//                          scans the aligned expert totals and writes its tokens' part of the handle;
+//                          workgroup 0 publishes N, C to the host mailbox.
+//   layout_scan_kernel + layout_assign_kernel : (many blocks) the same in two launches, with one
+//                          workgroup doing the scans: slot = offset[e] + block_base[b][e] + rank.
 //   dispatch_rows_kernel : one wavefront per (receive row, row chunk): 128-bit loads of the source
 //                          row held in registers, stored to every destination row; extra work items
 //                          zero-fill the alignment gaps.
@@ -28,6 +30,7 @@
 #include <cstdlib>
 #include <cstring>
 #include <ctime>
+#include <type_traits>
 
 #include "nanoep_hip.h"
 
@@ -62,6 +65,19 @@ int env_int(const char* name, int fallback) {
     return std::atoi(text);
 }
 
+// Calls f with the smallest compile-time bound in {4, 8, 16, 32} that covers num_topk.
+template <typename F>
+void with_topk_cap(int num_topk, F&& f) {
+    if (num_topk <= 4)
+        f(std::integral_constant<int, 4>{});
+    else if (num_topk <= 8)
+        f(std::integral_constant<int, 8>{});
+    else if (num_topk <= 16)
+        f(std::integral_constant<int, 16>{});
+    else
+        f(std::integral_constant<int, 32>{});
+}
+
 // ---------------------------------------------------------------------------------------------
 // Routing layout
 // ---------------------------------------------------------------------------------------------
@@ -80,7 +96,7 @@ int layout_tokens_per_block(int64_t local_experts) {
 struct LayoutWorkspace {
     int32_t* block_counts;  // [NB][L+1]; column L counts tokens with any valid choice
     int32_t* block_status;  // [NB]
-    int32_t* local_rank;    // [T][K]
+    int32_t* packed_rank;   // [T][K]  (expert << 8) | in-block rank, or -1
     int32_t* local_row;     // [T]
     size_t bytes;
 };
@@ -95,7 +111,7 @@ LayoutWorkspace carve_layout_workspace(void* base, int64_t tokens, int topk, int
     offset = align_up(offset + static_cast<size_t>(blocks) * (local_experts + 1) * 4, 256);
     ws.block_status = reinterpret_cast<int32_t*>(cursor + offset);
     offset = align_up(offset + static_cast<size_t>(blocks) * 4, 256);
-    ws.local_rank = reinterpret_cast<int32_t*>(cursor + offset);
+    ws.packed_rank = reinterpret_cast<int32_t*>(cursor + offset);
     offset = align_up(offset + static_cast<size_t>(tokens) * topk * 4, 256);
     ws.local_row = reinterpret_cast<int32_t*>(cursor + offset);
     offset = align_up(offset + static_cast<size_t>(tokens) * 4, 256);
@@ -103,19 +119,28 @@ LayoutWorkspace carve_layout_workspace(void* base, int64_t tokens, int topk, int
     return ws;
 }
 
+// A (token, k) entry of the rank table packs (expert << kRankBits) | in-block rank; -1 marks a
+// masked choice.  A layout block never holds more than 256 tokens, so the rank fits 8 bits.
+constexpr int kRankBits = 8;
+constexpr int kRankMask = (1 << kRankBits) - 1;
+
 // One thread per token.  bits[e][w] has bit (token & 31) of word (token >> 5) set when the token
 // chose expert e; row L marks tokens with any valid choice.  Experts inside a token are distinct,
 // so the order of one expert's assignments is the token order and a popcount prefix is the rank.
-__global__ void layout_count_kernel(const int64_t* __restrict__ topk_idx,
-                                    int64_t num_tokens,
-                                    int num_topk,
-                                    int local_experts,
-                                    int words,
-                                    int64_t* __restrict__ snapshot,
-                                    int32_t* __restrict__ block_counts,
-                                    int32_t* __restrict__ block_status,
-                                    int32_t* __restrict__ local_rank,
-                                    int32_t* __restrict__ local_row) {
+// The token's routing ids are fetched in one batch of independent loads (kCap >= K of them, the
+// surplus re-reads id 0) and stay in registers for both passes over the bit matrix.
+template <int kCap>
+__global__ void __launch_bounds__(256) layout_count_kernel(const int64_t* __restrict__ topk_idx,
+                                                           int64_t num_tokens,
+                                                           int num_topk,
+                                                           int local_experts,
+                                                           int words,
+                                                           int threads,
+                                                           int64_t* __restrict__ snapshot,
+                                                           int32_t* __restrict__ block_counts,
+                                                           int32_t* __restrict__ block_status,
+                                                           int32_t* __restrict__ packed_rank,
+                                                           int32_t* __restrict__ local_row) {
     extern __shared__ uint32_t layout_lds[];
     const int rows = local_experts + 1;
     // bit rows are words + 1 apart: an odd stride spreads the experts a wavefront touches over the LDS banks
@@ -124,12 +149,6 @@ __global__ void layout_count_kernel(const int64_t* __restrict__ topk_idx,
     auto* prefix = reinterpret_cast<uint16_t*>(bits + static_cast<size_t>(rows) * stride);
     __shared__ int block_bad;
 
-    for (int i = threadIdx.x; i < rows * stride; i += blockDim.x)
-        bits[i] = 0;
-    if (threadIdx.x == 0)
-        block_bad = 0;
-    __syncthreads();
-
     const int tokens_per_block = words * 32;
     const int local_token = threadIdx.x;
     const int64_t token = static_cast<int64_t>(blockIdx.x) * tokens_per_block + local_token;
@@ -137,29 +156,50 @@ __global__ void layout_count_kernel(const int64_t* __restrict__ topk_idx,
     const int word = local_token >> 5;
     const uint32_t bit = 1u << (local_token & 31);
 
-    if (live) {
-        int bad = 0;
-        bool any = false;
-        for (int k = 0; k < num_topk; ++k) {
-            const int64_t expert = topk_idx[token * num_topk + k];
-            snapshot[token * num_topk + k] = expert;
-            if (expert >= 0 && expert < local_experts) {
-                const uint32_t old = atomicOr(&bits[static_cast<size_t>(expert) * stride + word], bit);
-                if (old & bit)
-                    bad |= NANOEP_ROUTING_DUPLICATE;
-                any = true;
-            } else if (expert != -1) {
-                bad |= NANOEP_ROUTING_BAD_EXPERT;
-            }
-        }
-        if (any)
-            atomicOr(&bits[static_cast<size_t>(local_experts) * stride + word], bit);
-        if (bad)
-            atomicOr(&block_bad, bad);
-    }
+    int64_t raw[kCap];
+    const int64_t* mine = topk_idx + (live ? token : 0) * num_topk;
+#pragma unroll
+    for (int k = 0; k < kCap; ++k)
+        raw[k] = mine[k < num_topk ? k : 0];
+
+    for (int i = threadIdx.x; i < rows * stride; i += threads)
+        bits[i] = 0;
+    if (threadIdx.x == 0)
+        block_bad = 0;
     __syncthreads();
 
-    for (int row = threadIdx.x; row < rows; row += blockDim.x) {
+    int ids[kCap];  // expert id, -1 masked, -2 out of range
+#pragma unroll
+    for (int k = 0; k < kCap; ++k) {
+        const int64_t expert = raw[k];
+        ids[k] = (expert >= 0 && expert < local_experts) ? static_cast<int>(expert) : (expert == -1 ? -1 : -2);
+        if (!live || k >= num_topk)
+            ids[k] = -1;
+        else
+            snapshot[token * num_topk + k] = expert;
+    }
+
+    int bad = 0;
+    bool any = false;
+#pragma unroll
+    for (int k = 0; k < kCap; ++k) {
+        const int id = ids[k];
+        if (id >= 0) {
+            const uint32_t old = atomicOr(&bits[static_cast<size_t>(id) * stride + word], bit);
+            if (old & bit)
+                bad |= NANOEP_ROUTING_DUPLICATE;
+            any = true;
+        } else if (id == -2) {
+            bad |= NANOEP_ROUTING_BAD_EXPERT;
+        }
+    }
+    if (any)
+        atomicOr(&bits[static_cast<size_t>(local_experts) * stride + word], bit);
+    if (bad)
+        atomicOr(&block_bad, bad);
+    __syncthreads();
+
+    for (int row = threadIdx.x; row < rows; row += threads) {
         int running = 0;
         for (int w = 0; w < words; ++w) {
             prefix[static_cast<size_t>(row) * words + w] = static_cast<uint16_t>(running);
@@ -173,14 +213,17 @@ __global__ void layout_count_kernel(const int64_t* __restrict__ topk_idx,
 
     if (live) {
         const uint32_t below = bit - 1;
-        for (int k = 0; k < num_topk; ++k) {
-            const int64_t expert = topk_idx[token * num_topk + k];
-            int rank = -1;
-            if (expert >= 0 && expert < local_experts) {
-                rank = prefix[static_cast<size_t>(expert) * words + word] +
-                       __popc(bits[static_cast<size_t>(expert) * stride + word] & below);
+#pragma unroll
+        for (int k = 0; k < kCap; ++k) {
+            const int id = ids[k];
+            int32_t packed = -1;
+            if (id >= 0) {
+                const int rank = prefix[static_cast<size_t>(id) * words + word] +
+                                 __popc(bits[static_cast<size_t>(id) * stride + word] & below);
+                packed = (id << kRankBits) | rank;
             }
-            local_rank[token * num_topk + k] = rank;
+            if (k < num_topk)
+                packed_rank[token * num_topk + k] = packed;
         }
         const uint32_t received = bits[static_cast<size_t>(local_experts) * stride + word];
         local_row[token] = (received & bit) ? prefix[static_cast<size_t>(local_experts) * words + word] + __popc(received & below) : -1;
@@ -188,7 +231,7 @@ __global__ void layout_count_kernel(const int64_t* __restrict__ topk_idx,
 }
 
 __device__ __forceinline__ int64_t round_up_to(int64_t value, int64_t alignment) {
-    return (value + alignment - 1) / alignment * alignment;
+    return alignment == 1 ? value : (value + alignment - 1) / alignment * alignment;
 }
 
 // Single workgroup.  Phase 1 turns every column of block_counts into its exclusive prefix over
@@ -294,25 +337,24 @@ __global__ void __launch_bounds__(kScanThreads) layout_scan_kernel(int32_t* __re
     }
 }
 
-__global__ void layout_assign_kernel(const int64_t* __restrict__ topk_idx,
-                                     int64_t num_tokens,
-                                     int num_topk,
-                                     int local_experts,
-                                     int tokens_per_block,
-                                     int expand,
-                                     const int32_t* __restrict__ block_base,
-                                     const int32_t* __restrict__ local_rank,
-                                     const int32_t* __restrict__ local_row,
-                                     const int64_t* __restrict__ expert_offsets,
-                                     int32_t* __restrict__ recv_metadata,
-                                     int64_t* __restrict__ dst_slots,
-                                     int32_t* __restrict__ token_slots) {
-    const int64_t token = static_cast<int64_t>(blockIdx.x) * tokens_per_block + threadIdx.x;
-    if (static_cast<int>(threadIdx.x) >= tokens_per_block || token >= num_tokens)
-        return;
-    const int rows = local_experts + 1;
-    const int32_t* base = block_base + static_cast<int64_t>(blockIdx.x) * rows;
-    const int row_in_block = local_row[token];
+// Writes one token's part of the handle.  `slot_base[e]` is the first slot of this block's
+// assignments to expert e, less `expert_offsets[e]` when that pointer is given.
+template <int kCap>
+__device__ __forceinline__ void assign_token_slots(int64_t token,
+                                                   int num_topk,
+                                                   int expand,
+                                                   int row_in_block,
+                                                   int64_t row_base,
+                                                   const int32_t* slot_base,
+                                                   const int64_t* expert_offsets,
+                                                   const int32_t* __restrict__ packed_rank,
+                                                   int32_t* __restrict__ recv_metadata,
+                                                   int64_t* __restrict__ dst_slots,
+                                                   int32_t* __restrict__ token_slots) {
+    int32_t packed[kCap];
+#pragma unroll
+    for (int k = 0; k < kCap; ++k)
+        packed[k] = packed_rank[token * num_topk + (k < num_topk ? k : 0)];
     if (row_in_block < 0) {
         dst_slots[token] = -1;
         if (token_slots != nullptr)
@@ -320,21 +362,195 @@ __global__ void layout_assign_kernel(const int64_t* __restrict__ topk_idx,
                 token_slots[token * num_topk + k] = -1;
         return;
     }
-    const int64_t row = static_cast<int64_t>(base[local_experts]) + row_in_block;
+    const int64_t row = row_base + row_in_block;
     dst_slots[token] = row;
     int32_t* out = recv_metadata + row * (num_topk + 2);
     out[0] = 0;
     out[1] = static_cast<int32_t>(token);
-    for (int k = 0; k < num_topk; ++k) {
-        const int64_t expert = topk_idx[token * num_topk + k];
+#pragma unroll
+    for (int k = 0; k < kCap; ++k) {
+        if (k >= num_topk)
+            break;
         int32_t value = -1;
-        if (expert >= 0 && expert < local_experts)
-            value = expand ? static_cast<int32_t>(expert_offsets[expert] + base[expert] + local_rank[token * num_topk + k])
-                           : static_cast<int32_t>(expert);
+        if (packed[k] >= 0) {
+            const int expert = packed[k] >> kRankBits;
+            if (expand) {
+                int64_t slot = static_cast<int64_t>(slot_base[expert]) + (packed[k] & kRankMask);
+                if (expert_offsets != nullptr)
+                    slot += expert_offsets[expert];
+                value = static_cast<int32_t>(slot);
+            } else {
+                value = expert;
+            }
+        }
         out[2 + k] = value;
         if (token_slots != nullptr)
             token_slots[token * num_topk + k] = value;
     }
+}
+
+template <int kCap>
+__global__ void __launch_bounds__(256) layout_assign_kernel(int64_t num_tokens,
+                                                            int num_topk,
+                                                            int local_experts,
+                                                            int tokens_per_block,
+                                                            int expand,
+                                                            const int32_t* __restrict__ block_base,
+                                                            const int32_t* __restrict__ packed_rank,
+                                                            const int32_t* __restrict__ local_row,
+                                                            const int64_t* __restrict__ expert_offsets,
+                                                            int32_t* __restrict__ recv_metadata,
+                                                            int64_t* __restrict__ dst_slots,
+                                                            int32_t* __restrict__ token_slots) {
+    const int64_t token = static_cast<int64_t>(blockIdx.x) * tokens_per_block + threadIdx.x;
+    if (static_cast<int>(threadIdx.x) >= tokens_per_block || token >= num_tokens)
+        return;
+    const int32_t* base = block_base + static_cast<int64_t>(blockIdx.x) * (local_experts + 1);
+    assign_token_slots<kCap>(token, num_topk, expand, local_row[token], base[local_experts], base, expert_offsets,
+                             packed_rank, recv_metadata, dst_slots, token_slots);
+}
+
+__device__ __forceinline__ int64_t wave_inclusive_scan(int64_t value) {
+    const int lane = threadIdx.x & (kWave - 1);
+#pragma unroll
+    for (int distance = 1; distance < kWave; distance *= 2) {
+        const int64_t other = __shfl_up(value, distance, kWave);
+        if (lane >= distance)
+            value += other;
+    }
+    return value;
+}
+
+// Scan and assignment in one launch, for batches with few layout blocks.  Every workgroup sums
+// the block histograms itself (they sit in L2): per column the total over all blocks and the
+// part from the blocks before its own, then the aligned exclusive scan over experts, all in LDS,
+// and finally the slots of its own tokens.  Workgroup 0 also writes the per-expert outputs and
+// the host mailbox (word 0 last).
+template <int kCap>
+__global__ void __launch_bounds__(256) layout_scan_assign_kernel(const int32_t* __restrict__ block_counts,
+                                                                 const int32_t* __restrict__ block_status,
+                                                                 int num_blocks,
+                                                                 int64_t num_tokens,
+                                                                 int num_topk,
+                                                                 int local_experts,
+                                                                 int tokens_per_block,
+                                                                 int threads,
+                                                                 int expand,
+                                                                 int64_t alignment,
+                                                                 const int32_t* __restrict__ packed_rank,
+                                                                 const int32_t* __restrict__ local_row,
+                                                                 int64_t* __restrict__ expert_counts,
+                                                                 int64_t* __restrict__ expert_offsets,
+                                                                 int64_t* __restrict__ send_counts,
+                                                                 int64_t* __restrict__ recv_rank_prefix,
+                                                                 int64_t* host_counts,
+                                                                 int32_t* __restrict__ recv_metadata,
+                                                                 int64_t* __restrict__ dst_slots,
+                                                                 int32_t* __restrict__ token_slots) {
+    extern __shared__ int32_t scan_lds[];
+    __shared__ int64_t wave_padded[kWavesPerBlock];
+    __shared__ int64_t wave_assigned[kWavesPerBlock];
+    __shared__ int status_bits;
+    const int rows = local_experts + 1;
+    int32_t* column_total = scan_lds;          // [L+1]
+    int32_t* column_before = scan_lds + rows;  // [L+1], turns into the block's first slot per expert
+
+    const int tid = threadIdx.x;
+    const int block = blockIdx.x;
+    const int64_t token = static_cast<int64_t>(block) * tokens_per_block + tid;
+    const bool live = tid < tokens_per_block && token < num_tokens;
+    const int row_in_block = live ? local_row[token] : -1;
+
+    for (int i = tid; i < 2 * rows; i += threads)
+        scan_lds[i] = 0;
+    if (tid == 0)
+        status_bits = 0;
+    __syncthreads();
+
+    const int columns_per_pass = rows < threads ? rows : threads;
+    const int segments = threads / columns_per_pass;
+    const int blocks_per_segment = (num_blocks + segments - 1) / segments;
+    const int column_local = tid % columns_per_pass;
+    const int segment = tid / columns_per_pass;
+    const int begin = segment * blocks_per_segment;
+    const int end = begin + blocks_per_segment < num_blocks ? begin + blocks_per_segment : num_blocks;
+    for (int column0 = 0; column0 < rows; column0 += columns_per_pass) {
+        const int column = column0 + column_local;
+        if (segment < segments && column < rows) {
+            int total = 0, before = 0;
+#pragma unroll 8
+            for (int b = begin; b < end; ++b) {
+                const int count = block_counts[static_cast<int64_t>(b) * rows + column];
+                total += count;
+                before += b < block ? count : 0;
+            }
+            if (segments == 1) {
+                column_total[column] = total;
+                column_before[column] = before;
+            } else {
+                atomicAdd(&column_total[column], total);
+                atomicAdd(&column_before[column], before);
+            }
+        }
+    }
+    if (block == 0) {
+        int bad = 0;
+        for (int b = tid; b < num_blocks; b += threads)
+            bad |= block_status[b];
+        if (bad)
+            atomicOr(&status_bits, bad);
+    }
+    __syncthreads();
+
+    const int per_thread = (local_experts + threads - 1) / threads;
+    const int first = tid * per_thread < local_experts ? tid * per_thread : local_experts;
+    const int last = first + per_thread < local_experts ? first + per_thread : local_experts;
+    int64_t padded_sum = 0, count_sum = 0;
+    for (int e = first; e < last; ++e) {
+        const int64_t count = column_total[e];
+        count_sum += count;
+        padded_sum += round_up_to(count, alignment);
+    }
+    const int64_t padded_scan = wave_inclusive_scan(padded_sum);
+    const int64_t assigned_scan = wave_inclusive_scan(count_sum);
+    const int wave = tid / kWave;
+    const int waves = threads / kWave;
+    if ((tid & (kWave - 1)) == kWave - 1) {
+        wave_padded[wave] = padded_scan;
+        wave_assigned[wave] = assigned_scan;
+    }
+    __syncthreads();
+    int64_t running = padded_scan - padded_sum;
+    int64_t capacity = 0, assigned = 0;
+    for (int w = 0; w < waves; ++w) {
+        running += w < wave ? wave_padded[w] : 0;
+        capacity += wave_padded[w];
+        assigned += wave_assigned[w];
+    }
+    for (int e = first; e < last; ++e) {
+        const int64_t count = column_total[e];
+        if (block == 0) {
+            expert_counts[e] = count;
+            expert_offsets[e] = running;
+        }
+        column_before[e] += static_cast<int32_t>(running);
+        running += round_up_to(count, alignment);
+    }
+    if (block == 0 && tid == 0) {
+        const int64_t received = column_total[local_experts];
+        expert_offsets[local_experts] = capacity;
+        send_counts[0] = received;
+        recv_rank_prefix[0] = received;
+        host_counts[1] = capacity;
+        host_counts[2] = assigned;
+        host_counts[3] = status_bits;
+        __threadfence_system();
+        __hip_atomic_store(&host_counts[0], received, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_SYSTEM);
+    }
+    __syncthreads();
+    if (live)
+        assign_token_slots<kCap>(token, num_topk, expand, row_in_block, column_before[local_experts], column_before,
+                                 nullptr, packed_rank, recv_metadata, dst_slots, token_slots);
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -772,7 +988,7 @@ int nanoep_layout(const int64_t* topk_idx, int64_t num_tokens, int num_topk, int
                   int64_t* recv_rank_prefix, int32_t* token_slots, void* workspace, size_t workspace_bytes,
                   int64_t* host_counts, void* stream_handle) {
     if (num_tokens < 0 || num_tokens > INT32_MAX || num_topk <= 0 || num_topk > kMaxTopk || num_local_experts <= 0 ||
-        num_local_experts > INT32_MAX - 1 || alignment <= 0 || alignment > (int64_t{1} << 31))
+        num_local_experts >= (int64_t{1} << (31 - kRankBits)) || alignment <= 0 || alignment > (int64_t{1} << 31))
         return NANOEP_ERR_INVALID_ARGUMENT;
     if (expert_counts == nullptr || expert_offsets == nullptr || send_counts == nullptr || recv_rank_prefix == nullptr ||
         host_counts == nullptr || workspace == nullptr)
@@ -793,24 +1009,46 @@ int nanoep_layout(const int64_t* topk_idx, int64_t num_tokens, int num_topk, int
 
     __atomic_store_n(&host_counts[0], int64_t{-1}, __ATOMIC_RELEASE);
     const int count_threads = tokens_per_block < kWave ? kWave : tokens_per_block;
-    if (blocks > 0) {
-        const size_t lds = static_cast<size_t>(experts + 1) * (words * 6 + 4);
-        layout_count_kernel<<<blocks, count_threads, lds, stream>>>(topk_idx, num_tokens, num_topk, experts, words,
-                                                                     topk_snapshot, ws.block_counts, ws.block_status,
-                                                                     ws.local_rank, ws.local_row);
-        NANOEP_HIP_TRY(hipGetLastError());
-    }
-    layout_scan_kernel<<<1, kScanThreads, static_cast<size_t>(experts + 1) * 4, stream>>>(
-        ws.block_counts, ws.block_status, blocks, experts, alignment, expert_counts, expert_offsets, send_counts,
-        recv_rank_prefix, host_counts);
-    NANOEP_HIP_TRY(hipGetLastError());
-    if (blocks > 0) {
-        layout_assign_kernel<<<blocks, count_threads, 0, stream>>>(topk_idx, num_tokens, num_topk, experts,
-                                                                    tokens_per_block, expand, ws.block_counts,
-                                                                    ws.local_rank, ws.local_row, expert_offsets,
-                                                                    recv_metadata, dst_slots, token_slots);
-        NANOEP_HIP_TRY(hipGetLastError());
-    }
+    // Two launches when every block can afford to sum the block histograms itself
+    // (blocks x (L+1) loads spread over the workgroup), three with a single-workgroup scan otherwise.
+    bool fused_scan = blocks > 0 && static_cast<int64_t>(blocks) * (experts + 1) <= int64_t{32} * count_threads;
+    const int forced_launches = env_int("NANOEP_LAYOUT_LAUNCHES", 0);
+    if (forced_launches == 3)
+        fused_scan = false;
+    else if (forced_launches == 2 && blocks > 0)
+        fused_scan = true;
+    hipError_t launch_status = hipSuccess;
+    with_topk_cap(num_topk, [&](auto cap) {
+        constexpr int kCap = decltype(cap)::value;
+        if (blocks > 0) {
+            const size_t lds = static_cast<size_t>(experts + 1) * (words * 6 + 4);
+            layout_count_kernel<kCap><<<blocks, count_threads, lds, stream>>>(
+                topk_idx, num_tokens, num_topk, experts, words, count_threads, topk_snapshot, ws.block_counts,
+                ws.block_status, ws.packed_rank, ws.local_row);
+            if ((launch_status = hipGetLastError()) != hipSuccess)
+                return;
+        }
+        if (fused_scan) {
+            layout_scan_assign_kernel<kCap><<<blocks, count_threads, static_cast<size_t>(experts + 1) * 8, stream>>>(
+                ws.block_counts, ws.block_status, blocks, num_tokens, num_topk, experts, tokens_per_block, count_threads,
+                expand, alignment, ws.packed_rank, ws.local_row, expert_counts, expert_offsets, send_counts,
+                recv_rank_prefix, host_counts, recv_metadata, dst_slots, token_slots);
+            launch_status = hipGetLastError();
+            return;
+        }
+        layout_scan_kernel<<<1, kScanThreads, static_cast<size_t>(experts + 1) * 4, stream>>>(
+            ws.block_counts, ws.block_status, blocks, experts, alignment, expert_counts, expert_offsets, send_counts,
+            recv_rank_prefix, host_counts);
+        if ((launch_status = hipGetLastError()) != hipSuccess)
+            return;
+        if (blocks > 0) {
+            layout_assign_kernel<kCap><<<blocks, count_threads, 0, stream>>>(
+                num_tokens, num_topk, experts, tokens_per_block, expand, ws.block_counts, ws.packed_rank, ws.local_row,
+                expert_offsets, recv_metadata, dst_slots, token_slots);
+            launch_status = hipGetLastError();
+        }
+    });
+    NANOEP_HIP_TRY(launch_status);
     return NANOEP_OK;
 }
 

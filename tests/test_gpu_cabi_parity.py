@@ -204,6 +204,21 @@ def test_topk_range(device, topk, experts, hidden, expand):
     run_dispatch_combine(device, idx, hidden, experts, 8, expand, expand, True, seed=topk)
 
 
+@pytest.mark.parametrize("launches", ["2", "3"], ids=["scan-in-assign", "separate-scan"])
+@pytest.mark.parametrize(
+    "tokens,experts,topk,kind,alignment",
+    [(1000, 16, 4, "mixed", 8), (4096, 256, 8, "dropout", 1), (700, 1500, 9, "sparse", 3), (2049, 8, 2, "skew", 128), (5000, 40, 17, "random", 1)],
+)
+@pytest.mark.parametrize("expand", [False, True], ids=["compact", "expanded"])
+def test_both_layout_launch_plans(device, monkeypatch, launches, tokens, experts, topk, kind, alignment, expand):
+    """The layout runs as two launches (every block scans the block histograms itself) or three
+    (single-workgroup scan), chosen by size; both plans must give the oracle's handle."""
+    monkeypatch.setenv("NANOEP_LAYOUT_LAUNCHES", launches)
+    idx = cases.routing(kind, tokens, experts, topk, seed=5)
+    metadata, counts = cabi.layout(idx.to(device), experts, alignment, expand)
+    assert_layout(metadata, counts, oracle.layout(idx, experts, alignment), expand)
+
+
 def test_empty_inputs(device):
     for expand in (False, True):
         idx = torch.empty((0, 4), dtype=torch.int64)
