@@ -52,8 +52,63 @@ def measured_traffic(kernel: str, workload: str):
     return float(match.group(1)) if match else None
 
 
-def cpu_baseline(workload, x, idx, weights, budget_seconds):
-    """The vectorised torch-CPU oracle on the same batch: dispatch + combine, bounded in time."""
+def layout_gpu_us(workload, idx, iterations=50):
+    """GPU time of the routing-layout launches alone (no host wait), through the C ABI."""
+    import ctypes
+
+    import torch
+
+    library = ctypes.CDLL(str(ROOT / "nanoep_amd" / "libnanoep_hip.so"))
+    p, i64 = ctypes.c_void_p, ctypes.c_int64
+    library.nanoep_layout_workspace_bytes.restype = ctypes.c_size_t
+    library.nanoep_layout_workspace_bytes.argtypes = [i64, ctypes.c_int, i64]
+    library.nanoep_slot_order_entries.restype = i64
+    library.nanoep_slot_order_entries.argtypes = [i64, ctypes.c_int, i64]
+    library.nanoep_layout.argtypes = [p, i64, ctypes.c_int, i64, i64, ctypes.c_int, p, p, p, p, p, p, p, p, p, p, ctypes.c_size_t, p, p]
+    tokens, topk, experts = workload.tokens, workload.topk, workload.experts
+    device = idx.device
+    nbytes = library.nanoep_layout_workspace_bytes(tokens, topk, experts)
+    workspace = torch.empty(nbytes, dtype=torch.uint8, device=device)
+    metadata = torch.empty((tokens, topk + 2), dtype=torch.int32, device=device)
+    table = torch.empty((tokens, topk), dtype=torch.int32, device=device)
+    order = torch.empty(library.nanoep_slot_order_entries(tokens, topk, experts), dtype=torch.int64, device=device)
+    snapshot = torch.empty_like(idx)
+    dst_slots = torch.empty((tokens, 1), dtype=torch.int64, device=device)
+    counts = torch.empty(experts, dtype=torch.int64, device=device)
+    offsets = torch.empty(experts + 1, dtype=torch.int64, device=device)
+    sent = torch.empty(1, dtype=torch.int64, device=device)
+    prefix = torch.empty(1, dtype=torch.int64, device=device)
+    mailbox = torch.empty(4, dtype=torch.int64, pin_memory=True)
+    stream = torch.cuda.current_stream()
+
+    def launch():
+        status = library.nanoep_layout(idx.data_ptr(), tokens, topk, experts, workload.alignment, int(workload.expand),
+                                       metadata.data_ptr(), counts.data_ptr(), offsets.data_ptr(), dst_slots.data_ptr(),
+                                       sent.data_ptr(), snapshot.data_ptr(), prefix.data_ptr(),
+                                       table.data_ptr() if workload.expand else None,
+                                       order.data_ptr() if workload.expand else None, workspace.data_ptr(), nbytes,
+                                       mailbox.data_ptr(), stream.cuda_stream)
+        if status != 0:
+            raise RuntimeError(f"nanoep_layout failed with status {status}")
+
+    for _ in range(10):
+        launch()
+    begin, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    torch.cuda.synchronize()
+    begin.record(stream)
+    for _ in range(iterations):
+        launch()
+    end.record(stream)
+    torch.cuda.synchronize()
+    return begin.elapsed_time(end) * 1e3 / iterations
+
+
+def cpu_baseline(workload, x, idx, weights, budget_seconds, gpu_dispatched=None, gpu_combined=None):
+    """The vectorised torch-CPU oracle on the same batch: dispatch + combine, bounded in time.
+
+    When the GPU results of the same batch are given, they are compared bit for bit with the
+    oracle's (NaN-free synthetic data, so plain bit equality is the bar) and the verdict is returned.
+    """
     import torch
 
     from nanoep_amd import workloads
@@ -72,25 +127,41 @@ def cpu_baseline(workload, x, idx, weights, budget_seconds):
                                          alignment=workload.alignment, lay=layout)
         oracle.combine(out_x, metadata, layout.dst_slots, do_expand=workload.expand)
 
-    step()  # warm caches and the allocator
-    times = []
-    started = time.perf_counter()
-    while True:
-        t0 = time.perf_counter()
-        step()
-        times.append(time.perf_counter() - t0)
-        if time.perf_counter() - started > budget_seconds or len(times) >= 20:
-            break
-    seconds = statistics.median(times)
+    parity = None
+    if gpu_dispatched is not None:
+        want_x, _, want_w, _ = oracle.dispatch(x, idx, workload.experts, weights, do_expand=workload.expand,
+                                               alignment=workload.alignment, lay=layout)
+        want_combined, _ = oracle.combine(want_x, metadata, layout.dst_slots, do_expand=workload.expand)
+        parity = bool(torch.equal(gpu_dispatched.view(torch.int16), want_x.view(torch.int16))
+                      and torch.equal(gpu_combined.view(torch.int16), want_combined.view(torch.int16)))
+        del want_x, want_combined
+
+    def sample(limit_seconds, limit_steps):
+        step()  # warm caches and the allocator
+        times = []
+        started = time.perf_counter()
+        while True:
+            t0 = time.perf_counter()
+            step()
+            times.append(time.perf_counter() - t0)
+            if time.perf_counter() - started > limit_seconds or len(times) >= limit_steps:
+                break
+        return statistics.median(times), len(times)
+
+    seconds, count = sample(budget_seconds, 20)
+    torch.set_num_threads(1)
+    single_seconds, single_count = sample(budget_seconds / 2, 5)
+    torch.set_num_threads(cores)
     return {
         "value": round(nbytes / seconds / 1e9, 3),
         "unit": "GB/s",
         "cores": cores,
         "kind": "port",
         "us_per_step": round(seconds * 1e6, 1),
-        "sample": f"{len(times)} timed steps (cached-layout dispatch + combine) of the full {workload.name} batch "
-                  f"with the vectorised torch-CPU oracle, {cores} threads",
-    }
+        "value_1_thread": round(nbytes / single_seconds / 1e9, 3),
+        "sample": f"{count} timed steps (cached-layout dispatch + combine) of the full {workload.name} batch "
+                  f"with the vectorised torch-CPU oracle, {cores} threads; {single_count} steps with 1 thread",
+    }, parity
 
 
 def main():
@@ -110,7 +181,7 @@ def main():
     device = torch.device("cuda", 0)
     torch.cuda.set_device(device)
 
-    rotation = 4
+    rotation = 8  # 8 x 58.7 MB of sources: more than the 256 MB last-level cache
     batches = [workloads.make_inputs(workload, seed=seed) for seed in range(rotation)]
     x_cpu, idx_cpu, w_cpu = batches[0]
     xs = [batch[0].to(device) for batch in batches]
@@ -130,7 +201,12 @@ def main():
                                        alignment=workload.alignment, zero_padding=workload.zero_padding)
             torch.cuda.synchronize()
             fresh_times.append(time.perf_counter() - t0)
+        layout_us = layout_gpu_us(workload, idx)
         handle = received.handle
+        check_combined = buffer.combine(received.x, handle).x
+        torch.cuda.synchronize()
+        gpu_dispatched, gpu_combined = received.x.cpu(), check_combined.cpu()
+        del check_combined
         n_recv, capacity = handle.layout.recv_count, handle.layout.expanded_capacity
         assignments = int(handle.layout.expert_counts.sum().item())
         d_bytes = workloads.dispatch_bytes(workload, n_recv, assignments, capacity)
@@ -211,6 +287,7 @@ def main():
             "combine_us": round(c_us, 2),
             "combine_GBps": round(c_bytes / c_us / 1e3, 1),
             "fresh_dispatch_us_host": round(statistics.median(fresh_times) * 1e6, 1),
+            "layout_us_gpu_no_host_wait": round(layout_us, 2),
             "dispatch_bytes": d_bytes,
             "combine_bytes": c_bytes,
             "roofline": {
@@ -257,7 +334,12 @@ def main():
     del xs, ring
     torch.cuda.empty_cache()
     if args.cpu_seconds > 0:
-        result["cpu_baseline"] = cpu_baseline(workload, x_cpu, idx_cpu, w_cpu, args.cpu_seconds)
+        result["cpu_baseline"], result["bit_exact_vs_oracle"] = cpu_baseline(
+            workload, x_cpu, idx_cpu, w_cpu, args.cpu_seconds, gpu_dispatched, gpu_combined)
+        if not result["bit_exact_vs_oracle"]:
+            log("ERROR: GPU results of the timed configuration differ from the oracle")
+            print(json.dumps(result), flush=True)
+            return 1
     print(json.dumps(result), flush=True)
     return 0
 

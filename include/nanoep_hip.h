@@ -60,6 +60,15 @@ int nanoep_window_layout(int ranks, int64_t max_tokens, int hidden, int topk, in
 /* Device scratch needed by nanoep_layout for (T, K, L). */
 size_t nanoep_layout_workspace_bytes(int64_t num_tokens, int num_topk, int64_t num_local_experts);
 
+/* Tokens per block of the routing layout for L local experts (0: L is not supported).  The
+ * slot-order list is ordered block of consecutive tokens by block. */
+int nanoep_layout_block_tokens(int64_t num_local_experts);
+
+/* Number of int64 words nanoep_layout writes to the slot-order list for (T, K, L): the block
+ * count times block_tokens * K entries (an upper bound of the A that carry assignments), then one
+ * word holding A. */
+int64_t nanoep_slot_order_entries(int64_t num_tokens, int num_topk, int64_t num_local_experts);
+
 /*
  * Routing layout: histogram + device-wide exclusive scan + stable token-order slot assignment.
  * Replaces count_and_notify / finalize_receive_counts (csrc/dispatch_main.cuh:116-210, :70-114),
@@ -71,6 +80,12 @@ size_t nanoep_layout_workspace_bytes(int64_t num_tokens, int num_topk, int64_t n
  * token_slots (optional, int32 [T, K]) receives slot[t,k] (or the local id when !expand), -1 when
  * masked: the same information as dst_slots + recv_metadata in one lookup.  It is not one of the
  * reference's handle tensors; nanoep_dispatch / nanoep_combine run a little faster when given it.
+ * slot_order (optional, expanded only, T*K < 2^31, int64 [nanoep_slot_order_entries]) lists the A
+ * valid assignments as (slot << 32) | (t * K + k), token block by token block and in ascending slot
+ * (that is expert-major) order inside a block; the entries from A on are -1 and the last word of
+ * the buffer holds A.  Walking it makes a
+ * dispatch write runs of consecutive destination rows while a block's source rows stay cache
+ * resident.  Like token_slots it is private to this library.
  * host_counts is pinned, device-visible host memory of NANOEP_HOST_COUNT_WORDS int64:
  * the call sets word 0 to -1, the device later stores {N, C, A (total assignments), status}
  * with word 0 last, so a host that sees word 0 >= 0 may read the rest.
@@ -78,8 +93,8 @@ size_t nanoep_layout_workspace_bytes(int64_t num_tokens, int num_topk, int64_t n
 int nanoep_layout(const int64_t* topk_idx, int64_t num_tokens, int num_topk, int64_t num_local_experts,
                   int64_t alignment, int expand, int32_t* recv_metadata, int64_t* expert_counts,
                   int64_t* expert_offsets, int64_t* dst_slots, int64_t* send_counts, int64_t* topk_snapshot,
-                  int64_t* recv_rank_prefix, int32_t* token_slots, void* workspace, size_t workspace_bytes,
-                  int64_t* host_counts, void* stream);
+                  int64_t* recv_rank_prefix, int32_t* token_slots, int64_t* slot_order, void* workspace,
+                  size_t workspace_bytes, int64_t* host_counts, void* stream);
 
 /* Spin on the mailbox until the layout enqueued on `stream` has published its counts
  * (the reference's wait_dispatch_counts, csrc/peer.cu:198-227).  out = {N, C, A, status}. */
@@ -95,14 +110,19 @@ int nanoep_wait_counts(int64_t* host_counts, void* stream, double timeout_second
  *             [offsets[e]+counts[e], offsets[e+1]) and their weights are zero-filled.
  * Work is walked in source-token order: dst_slots[t] names the receive row whose metadata holds
  * the token's slots (token_slots, when not NULL and expanded, replaces that two-step lookup).
+ * When slot_order is given for an expanded dispatch, the work is walked in that order instead and
+ * neither of the other lookups is read for the payload.  slot_order_entries is A when the caller
+ * knows it (the list may then be just its first A entries); a caller that enqueues the dispatch
+ * before it has read the counts passes -1 with the full buffer, and the kernel takes A from the
+ * buffer's last word.
  * x / recv_x are bf16, 16-byte aligned, H % 8 == 0.  weights / recv_weights / recv_topk_idx may be
  * NULL (recv_topk_idx must be NULL when expanded).  num_cus is the reference's SM budget
  * (0 = whole device): it is range-checked against the device's compute-unit count and otherwise
  * ignored, because these kernels are sized by the work, not by a cooperative grid.
  */
 int nanoep_dispatch(const void* x, const float* weights, const int32_t* recv_metadata, const int64_t* dst_slots,
-                    const int32_t* token_slots, const int64_t* expert_counts, const int64_t* expert_offsets,
-                    int64_t recv_count, int64_t expanded_capacity, int64_t num_tokens, int hidden, int num_topk,
+                    const int32_t* token_slots, const int64_t* slot_order, int64_t slot_order_entries,
+                    const int64_t* expert_counts, const int64_t* expert_offsets, int64_t recv_count, int64_t expanded_capacity, int64_t num_tokens, int hidden, int num_topk,
                     int64_t num_local_experts, int64_t alignment, int expand, int zero_padding, void* recv_x,
                     int64_t* recv_topk_idx, float* recv_weights, int num_cus, void* stream);
 

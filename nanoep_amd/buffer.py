@@ -54,6 +54,10 @@ class NativeHandle:
     # int32 [T, K] slot of every (token, k), -1 when masked: the same mapping as dst_slots +
     # recv_metadata in one lookup.  Only expanded handles made by this package carry it.
     token_slots: torch.Tensor | None = None
+    # int64 list of every valid assignment as (slot << 32) | (t * K + k), one segment per block of
+    # consecutive tokens, ascending slot inside a segment, -1 in unused entries: the order in which
+    # a replayed dispatch walks its work.  Only expanded handles made by this package carry it.
+    slot_order: torch.Tensor | None = None
 
 
 @dataclass
@@ -95,6 +99,8 @@ def _handle_metadata(handle: NativeHandle) -> list[torch.Tensor]:
     ]
     if getattr(handle, "token_slots", None) is not None:
         metadata.append(handle.token_slots)
+        if getattr(handle, "slot_order", None) is not None:
+            metadata.append(handle.slot_order)
     return metadata
 
 
@@ -268,6 +274,7 @@ class CudaBuffer:
                 x_dtype=x.dtype,
                 num_sms=main_sms,
                 token_slots=metadata[7] if len(metadata) > 7 else None,
+                slot_order=metadata[8] if len(metadata) > 8 else None,
             )
 
         event = CudaEvent(completed, keepalive=(self, x, routing, weights, handle)) if async_op else None

@@ -85,6 +85,8 @@ void with_topk_cap(int num_topk, F&& f) {
 // Tokens handled by one layout workgroup: the LDS bit matrix has (L+1) rows of tokens/32 words
 // plus a 16-bit prefix per word, so the block shrinks as the expert count grows.
 int layout_tokens_per_block(int64_t local_experts) {
+    if (static_cast<size_t>(local_experts + 1) * 12 > kLayoutLdsBudget)  // three int32 arrays of the assignment kernel
+        return 0;
     for (int tokens = 256; tokens >= 32; tokens /= 2) {
         const size_t words = static_cast<size_t>(tokens / 32);
         if (static_cast<size_t>(local_experts + 1) * (words * 6 + 4) <= kLayoutLdsBudget)
@@ -98,6 +100,7 @@ struct LayoutWorkspace {
     int32_t* block_status;  // [NB]
     int32_t* packed_rank;   // [T][K]  (expert << 8) | in-block rank, or -1
     int32_t* local_row;     // [T]
+    int64_t* totals;        // [1] total assignments, handed from the scan kernel to the assignment kernel
     size_t bytes;
 };
 
@@ -115,6 +118,8 @@ LayoutWorkspace carve_layout_workspace(void* base, int64_t tokens, int topk, int
     offset = align_up(offset + static_cast<size_t>(tokens) * topk * 4, 256);
     ws.local_row = reinterpret_cast<int32_t*>(cursor + offset);
     offset = align_up(offset + static_cast<size_t>(tokens) * 4, 256);
+    ws.totals = reinterpret_cast<int64_t*>(cursor + offset);
+    offset = align_up(offset + 8, 256);
     ws.bytes = offset + 256;
     return ws;
 }
@@ -246,6 +251,7 @@ __global__ void __launch_bounds__(kScanThreads) layout_scan_kernel(int32_t* __re
                                                                   int64_t* __restrict__ expert_offsets,
                                                                   int64_t* __restrict__ send_counts,
                                                                   int64_t* __restrict__ recv_rank_prefix,
+                                                                  int64_t* __restrict__ totals,
                                                                   int64_t* host_counts) {
     extern __shared__ int32_t column_total[];  // [L+1]
     __shared__ int32_t partial[kScanThreads];
@@ -329,6 +335,7 @@ __global__ void __launch_bounds__(kScanThreads) layout_scan_kernel(int32_t* __re
         expert_offsets[local_experts] = capacity;
         send_counts[0] = received;
         recv_rank_prefix[0] = received;
+        totals[0] = assignments[kScanThreads - 1];
         host_counts[1] = capacity;
         host_counts[2] = assignments[kScanThreads - 1];
         host_counts[3] = status_bits;
@@ -338,7 +345,8 @@ __global__ void __launch_bounds__(kScanThreads) layout_scan_kernel(int32_t* __re
 }
 
 // Writes one token's part of the handle.  `slot_base[e]` is the first slot of this block's
-// assignments to expert e, less `expert_offsets[e]` when that pointer is given.
+// assignments to expert e; `order_base[e]` is where expert e's run starts in the block's segment
+// of the slot-order list (`order` points at that segment, or is null).
 template <int kCap>
 __device__ __forceinline__ void assign_token_slots(int64_t token,
                                                    int num_topk,
@@ -346,11 +354,12 @@ __device__ __forceinline__ void assign_token_slots(int64_t token,
                                                    int row_in_block,
                                                    int64_t row_base,
                                                    const int32_t* slot_base,
-                                                   const int64_t* expert_offsets,
+                                                   const int32_t* order_base,
                                                    const int32_t* __restrict__ packed_rank,
                                                    int32_t* __restrict__ recv_metadata,
                                                    int64_t* __restrict__ dst_slots,
-                                                   int32_t* __restrict__ token_slots) {
+                                                   int32_t* __restrict__ token_slots,
+                                                   int64_t* __restrict__ order) {
     int32_t packed[kCap];
 #pragma unroll
     for (int k = 0; k < kCap; ++k)
@@ -374,40 +383,17 @@ __device__ __forceinline__ void assign_token_slots(int64_t token,
         int32_t value = -1;
         if (packed[k] >= 0) {
             const int expert = packed[k] >> kRankBits;
-            if (expand) {
-                int64_t slot = static_cast<int64_t>(slot_base[expert]) + (packed[k] & kRankMask);
-                if (expert_offsets != nullptr)
-                    slot += expert_offsets[expert];
-                value = static_cast<int32_t>(slot);
-            } else {
-                value = expert;
+            const int rank = packed[k] & kRankMask;
+            value = expand ? slot_base[expert] + rank : expert;
+            if (order != nullptr) {
+                const uint32_t source = static_cast<uint32_t>(token * num_topk + k);
+                order[order_base[expert] + rank] = (static_cast<int64_t>(value) << 32) | source;
             }
         }
         out[2 + k] = value;
         if (token_slots != nullptr)
             token_slots[token * num_topk + k] = value;
     }
-}
-
-template <int kCap>
-__global__ void __launch_bounds__(256) layout_assign_kernel(int64_t num_tokens,
-                                                            int num_topk,
-                                                            int local_experts,
-                                                            int tokens_per_block,
-                                                            int expand,
-                                                            const int32_t* __restrict__ block_base,
-                                                            const int32_t* __restrict__ packed_rank,
-                                                            const int32_t* __restrict__ local_row,
-                                                            const int64_t* __restrict__ expert_offsets,
-                                                            int32_t* __restrict__ recv_metadata,
-                                                            int64_t* __restrict__ dst_slots,
-                                                            int32_t* __restrict__ token_slots) {
-    const int64_t token = static_cast<int64_t>(blockIdx.x) * tokens_per_block + threadIdx.x;
-    if (static_cast<int>(threadIdx.x) >= tokens_per_block || token >= num_tokens)
-        return;
-    const int32_t* base = block_base + static_cast<int64_t>(blockIdx.x) * (local_experts + 1);
-    assign_token_slots<kCap>(token, num_topk, expand, local_row[token], base[local_experts], base, expert_offsets,
-                             packed_rank, recv_metadata, dst_slots, token_slots);
 }
 
 __device__ __forceinline__ int64_t wave_inclusive_scan(int64_t value) {
@@ -421,39 +407,50 @@ __device__ __forceinline__ int64_t wave_inclusive_scan(int64_t value) {
     return value;
 }
 
-// Scan and assignment in one launch, for batches with few layout blocks.  Every workgroup sums
-// the block histograms itself (they sit in L2): per column the total over all blocks and the
-// part from the blocks before its own, then the aligned exclusive scan over experts, all in LDS,
-// and finally the slots of its own tokens.  Workgroup 0 also writes the per-expert outputs and
-// the host mailbox (word 0 last).
-template <int kCap>
-__global__ void __launch_bounds__(256) layout_scan_assign_kernel(const int32_t* __restrict__ block_counts,
-                                                                 const int32_t* __restrict__ block_status,
-                                                                 int num_blocks,
-                                                                 int64_t num_tokens,
-                                                                 int num_topk,
-                                                                 int local_experts,
-                                                                 int tokens_per_block,
-                                                                 int threads,
-                                                                 int expand,
-                                                                 int64_t alignment,
-                                                                 const int32_t* __restrict__ packed_rank,
-                                                                 const int32_t* __restrict__ local_row,
-                                                                 int64_t* __restrict__ expert_counts,
-                                                                 int64_t* __restrict__ expert_offsets,
-                                                                 int64_t* __restrict__ send_counts,
-                                                                 int64_t* __restrict__ recv_rank_prefix,
-                                                                 int64_t* host_counts,
-                                                                 int32_t* __restrict__ recv_metadata,
-                                                                 int64_t* __restrict__ dst_slots,
-                                                                 int32_t* __restrict__ token_slots) {
-    extern __shared__ int32_t scan_lds[];
+// Slot assignment, one workgroup per block of tokens (the blocks of layout_count_kernel).
+//
+// kFusedScan: `block_counts` holds the raw block histograms and every workgroup sums them itself
+// (they sit in L2): per column the total over all blocks and the part from the blocks before its
+// own, then the aligned exclusive scan over experts, all in LDS; workgroup 0 also writes the
+// per-expert outputs and the host mailbox (word 0 last).  Otherwise layout_scan_kernel has done
+// that and `block_counts` holds each block's exclusive prefixes.
+//
+// Either way the workgroup also scans its own histogram over experts: that places every
+// assignment of the block in expert-major order inside the block's run of `slot_order`; the runs
+// of consecutive blocks follow each other without gaps and the unused tail of the list is -1.
+template <int kCap, bool kFusedScan>
+__global__ void __launch_bounds__(256) layout_assign_kernel(const int32_t* __restrict__ block_counts,
+                                                            const int32_t* __restrict__ block_status,
+                                                            int num_blocks,
+                                                            int64_t num_tokens,
+                                                            int num_topk,
+                                                            int local_experts,
+                                                            int tokens_per_block,
+                                                            int threads,
+                                                            int expand,
+                                                            int64_t alignment,
+                                                            const int32_t* __restrict__ packed_rank,
+                                                            const int32_t* __restrict__ local_row,
+                                                            int64_t* expert_counts,
+                                                            int64_t* expert_offsets,
+                                                            int64_t* send_counts,
+                                                            int64_t* __restrict__ recv_rank_prefix,
+                                                            const int64_t* __restrict__ totals,
+                                                            int64_t* host_counts,
+                                                            int32_t* __restrict__ recv_metadata,
+                                                            int64_t* __restrict__ dst_slots,
+                                                            int32_t* __restrict__ token_slots,
+                                                            int64_t* __restrict__ slot_order) {
+    extern __shared__ int32_t assign_lds[];
     __shared__ int64_t wave_padded[kWavesPerBlock];
     __shared__ int64_t wave_assigned[kWavesPerBlock];
+    __shared__ int32_t wave_own[kWavesPerBlock];
+    __shared__ int32_t wave_before[kWavesPerBlock];
     __shared__ int status_bits;
     const int rows = local_experts + 1;
-    int32_t* column_total = scan_lds;          // [L+1]
-    int32_t* column_before = scan_lds + rows;  // [L+1], turns into the block's first slot per expert
+    int32_t* column_total = assign_lds;         // [L+1] totals over all blocks (fused scan only)
+    int32_t* slot_base = assign_lds + rows;     // [L+1] assignments before this block -> first slot per expert
+    int32_t* order_base = assign_lds + 2 * rows;  // [L+1] this block's histogram -> its exclusive scan
 
     const int tid = threadIdx.x;
     const int block = blockIdx.x;
@@ -461,44 +458,62 @@ __global__ void __launch_bounds__(256) layout_scan_assign_kernel(const int32_t* 
     const bool live = tid < tokens_per_block && token < num_tokens;
     const int row_in_block = live ? local_row[token] : -1;
 
-    for (int i = tid; i < 2 * rows; i += threads)
-        scan_lds[i] = 0;
-    if (tid == 0)
-        status_bits = 0;
-    __syncthreads();
+    if (kFusedScan) {
+        for (int i = tid; i < 2 * rows; i += threads)
+            assign_lds[i] = 0;
+        if (tid == 0)
+            status_bits = 0;
+        __syncthreads();
 
-    const int columns_per_pass = rows < threads ? rows : threads;
-    const int segments = threads / columns_per_pass;
-    const int blocks_per_segment = (num_blocks + segments - 1) / segments;
-    const int column_local = tid % columns_per_pass;
-    const int segment = tid / columns_per_pass;
-    const int begin = segment * blocks_per_segment;
-    const int end = begin + blocks_per_segment < num_blocks ? begin + blocks_per_segment : num_blocks;
-    for (int column0 = 0; column0 < rows; column0 += columns_per_pass) {
-        const int column = column0 + column_local;
-        if (segment < segments && column < rows) {
-            int total = 0, before = 0;
+        const int columns_per_pass = rows < threads ? rows : threads;
+        const int segments = threads / columns_per_pass;
+        const int blocks_per_segment = (num_blocks + segments - 1) / segments;
+        const int column_local = tid % columns_per_pass;
+        const int segment = tid / columns_per_pass;
+        const int begin = segment * blocks_per_segment;
+        const int end = begin + blocks_per_segment < num_blocks ? begin + blocks_per_segment : num_blocks;
+        for (int column0 = 0; column0 < rows; column0 += columns_per_pass) {
+            const int column = column0 + column_local;
+            if (segment < segments && column < rows) {
+                int total = 0, before = 0, own = 0;
 #pragma unroll 8
-            for (int b = begin; b < end; ++b) {
-                const int count = block_counts[static_cast<int64_t>(b) * rows + column];
-                total += count;
-                before += b < block ? count : 0;
-            }
-            if (segments == 1) {
-                column_total[column] = total;
-                column_before[column] = before;
-            } else {
-                atomicAdd(&column_total[column], total);
-                atomicAdd(&column_before[column], before);
+                for (int b = begin; b < end; ++b) {
+                    const int count = block_counts[static_cast<int64_t>(b) * rows + column];
+                    total += count;
+                    before += b < block ? count : 0;
+                    own = b == block ? count : own;
+                }
+                if (segments == 1) {
+                    column_total[column] = total;
+                    slot_base[column] = before;
+                } else {
+                    atomicAdd(&column_total[column], total);
+                    atomicAdd(&slot_base[column], before);
+                }
+                if (block >= begin && block < end)
+                    order_base[column] = own;
             }
         }
-    }
-    if (block == 0) {
-        int bad = 0;
-        for (int b = tid; b < num_blocks; b += threads)
-            bad |= block_status[b];
-        if (bad)
-            atomicOr(&status_bits, bad);
+        if (block == 0) {
+            int bad = 0;
+            for (int b = tid; b < num_blocks; b += threads)
+                bad |= block_status[b];
+            if (bad)
+                atomicOr(&status_bits, bad);
+        }
+    } else {
+        const int32_t* mine = block_counts + static_cast<int64_t>(block) * rows;
+        const bool last_block = block + 1 >= num_blocks;
+        for (int column = tid; column < rows; column += threads) {
+            const int32_t before = mine[column];
+            int32_t next;
+            if (!last_block)
+                next = mine[rows + column];
+            else
+                next = static_cast<int32_t>(column < local_experts ? expert_counts[column] : send_counts[0]);
+            order_base[column] = next - before;
+            slot_base[column] = before;
+        }
     }
     __syncthreads();
 
@@ -506,37 +521,60 @@ __global__ void __launch_bounds__(256) layout_scan_assign_kernel(const int32_t* 
     const int first = tid * per_thread < local_experts ? tid * per_thread : local_experts;
     const int last = first + per_thread < local_experts ? first + per_thread : local_experts;
     int64_t padded_sum = 0, count_sum = 0;
+    int own_sum = 0, before_sum = 0;
     for (int e = first; e < last; ++e) {
-        const int64_t count = column_total[e];
-        count_sum += count;
-        padded_sum += round_up_to(count, alignment);
+        if (kFusedScan) {
+            const int64_t count = column_total[e];
+            count_sum += count;
+            padded_sum += round_up_to(count, alignment);
+        }
+        own_sum += order_base[e];
+        before_sum += slot_base[e];
     }
-    const int64_t padded_scan = wave_inclusive_scan(padded_sum);
-    const int64_t assigned_scan = wave_inclusive_scan(count_sum);
+    const int64_t padded_scan = kFusedScan ? wave_inclusive_scan(padded_sum) : 0;
+    const int64_t assigned_scan = kFusedScan ? wave_inclusive_scan(count_sum) : 0;
+    const int own_scan = static_cast<int>(wave_inclusive_scan(own_sum));
+    const int before_scan = static_cast<int>(wave_inclusive_scan(before_sum));
     const int wave = tid / kWave;
     const int waves = threads / kWave;
     if ((tid & (kWave - 1)) == kWave - 1) {
         wave_padded[wave] = padded_scan;
         wave_assigned[wave] = assigned_scan;
+        wave_own[wave] = own_scan;
+        wave_before[wave] = before_scan;
     }
     __syncthreads();
     int64_t running = padded_scan - padded_sum;
+    int running_own = own_scan - own_sum;
     int64_t capacity = 0, assigned = 0;
+    int own_total = 0, assigned_before = 0;  // this block's assignments, and those of the blocks before it
     for (int w = 0; w < waves; ++w) {
         running += w < wave ? wave_padded[w] : 0;
+        running_own += w < wave ? wave_own[w] : 0;
         capacity += wave_padded[w];
         assigned += wave_assigned[w];
+        own_total += wave_own[w];
+        assigned_before += wave_before[w];
     }
+    if (!kFusedScan)
+        assigned = totals[0];
     for (int e = first; e < last; ++e) {
-        const int64_t count = column_total[e];
-        if (block == 0) {
-            expert_counts[e] = count;
-            expert_offsets[e] = running;
+        if (kFusedScan) {
+            const int64_t count = column_total[e];
+            if (block == 0) {
+                expert_counts[e] = count;
+                expert_offsets[e] = running;
+            }
+            slot_base[e] += static_cast<int32_t>(running);
+            running += round_up_to(count, alignment);
+        } else {
+            slot_base[e] += static_cast<int32_t>(expert_offsets[e]);
         }
-        column_before[e] += static_cast<int32_t>(running);
-        running += round_up_to(count, alignment);
+        const int own = order_base[e];
+        order_base[e] = running_own;
+        running_own += own;
     }
-    if (block == 0 && tid == 0) {
+    if (kFusedScan && block == 0 && tid == 0) {
         const int64_t received = column_total[local_experts];
         expert_offsets[local_experts] = capacity;
         send_counts[0] = received;
@@ -548,9 +586,22 @@ __global__ void __launch_bounds__(256) layout_scan_assign_kernel(const int32_t* 
         __hip_atomic_store(&host_counts[0], received, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_SYSTEM);
     }
     __syncthreads();
+    // The list is dense: this block's run starts where the earlier blocks' assignments end.  Every
+    // block also clears as many entries of the unused tail [A, entries) as it has masked choices.
+    int64_t* order = nullptr;
+    if (slot_order != nullptr) {
+        order = slot_order + assigned_before;
+        const int64_t block_entries = static_cast<int64_t>(tokens_per_block) * num_topk;
+        int64_t* tail = slot_order + assigned + (block * block_entries - assigned_before);
+        const int holes = static_cast<int>(block_entries) - own_total;
+        for (int i = tid; i < holes; i += threads)
+            tail[i] = -1;
+        if (block == 0 && tid == 0)
+            slot_order[num_blocks * block_entries] = assigned;  // count word behind the list
+    }
     if (live)
-        assign_token_slots<kCap>(token, num_topk, expand, row_in_block, column_before[local_experts], column_before,
-                                 nullptr, packed_rank, recv_metadata, dst_slots, token_slots);
+        assign_token_slots<kCap>(token, num_topk, expand, row_in_block, slot_base[local_experts], slot_base, order_base,
+                                 packed_rank, recv_metadata, dst_slots, token_slots, order);
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -590,6 +641,31 @@ __device__ __forceinline__ uint32_t xcd_contiguous_block(uint32_t blocks_per_xcd
     return (blockIdx.x % kNumXcds) * blocks_per_xcd + blockIdx.x / kNumXcds;
 }
 
+// n / d for n < 2^31 as one 64-bit multiply and shift: magic = ceil(2^shift / d), shift = 31 + ceil(log2 d).
+struct FastDivisor {
+    uint32_t magic;
+    uint32_t shift;
+};
+
+FastDivisor make_fast_divisor(uint32_t divisor) {
+    uint32_t log2_ceil = 0;
+    while ((uint64_t{1} << log2_ceil) < divisor)
+        ++log2_ceil;
+    const uint32_t shift = 31 + log2_ceil;
+    const uint64_t power = uint64_t{1} << shift;
+    return {static_cast<uint32_t>((power + divisor - 1) / divisor), shift};
+}
+
+__device__ __forceinline__ uint32_t fast_divide(uint32_t n, uint32_t magic, uint32_t shift) {
+    return static_cast<uint32_t>((static_cast<uint64_t>(n) * magic) >> shift);
+}
+
+// Kernel arguments are fetched with scalar loads where they are first used, which strings several
+// dependent round trips along a short wavefront's life.  Naming them in an empty asm statement at
+// the top of the kernel makes the compiler fetch them all in one batch.
+#define NANOEP_FETCH_ARGS_2(a, b) asm volatile("" ::"s"(a), "s"(b))
+#define NANOEP_FETCH_ARGS_4(a, b, c, d) asm volatile("" ::"s"(a), "s"(b), "s"(c), "s"(d))
+
 // One wavefront moves one 1 KiB chunk (64 lanes x 16 bytes) of one destination row with exactly
 // one 128-bit load and one nontemporal 128-bit store per lane: on this part a wavefront that issues
 // a single store and retires sustains more HBM write bandwidth than one that issues several.
@@ -605,12 +681,21 @@ __device__ __forceinline__ uint32_t xcd_contiguous_block(uint32_t blocks_per_xcd
 //
 // Workgroups past copy_blocks zero-fill the alignment gaps: workgroup (e, g) owns gap candidates
 // j = g * waves .. of expert e, row offsets[e] + counts[e] + j while that is below offsets[e+1].
-template <bool kDirectSlots>
+// How a dispatch wavefront finds its (source token, k, destination row).
+enum DispatchLookup {
+    kLookupMetadata = 0,  // candidate = (token, k) in token order; dst_slots -> recv_metadata row -> field k
+    kLookupTable = 1,     // candidate = (token, k) in token order; token_slots[token][k]
+    kLookupOrder = 2,     // candidate = entry of the slot-order list: (slot << 32) | (token * K + k), or -1
+};
+
+template <int kLookup>
 __global__ void __launch_bounds__(1024) dispatch_rows_kernel(const u32x4* __restrict__ x,                // [T][vectors]
                                                              const float* __restrict__ weights,         // [T][K] or null
                                                              const int32_t* __restrict__ recv_metadata,  // [N][K+2]
                                                              const int64_t* __restrict__ dst_slots,     // [T]
                                                              const int32_t* __restrict__ token_slots,   // [T][K] or null
+                                                             const int64_t* __restrict__ slot_order,    // [copy_candidates] or null
+                                                             const int64_t* __restrict__ live_count,    // device count of list entries, or null
                                                              const int64_t* __restrict__ expert_counts,
                                                              const int64_t* __restrict__ expert_offsets,
                                                              u32x4* __restrict__ recv_x,                // [C or N][vectors]
@@ -618,11 +703,15 @@ __global__ void __launch_bounds__(1024) dispatch_rows_kernel(const u32x4* __rest
                                                              float* __restrict__ recv_weights,          // [C] / [N][K] or null
                                                              int64_t recv_count,
                                                              int64_t out_rows,
-                                                             uint32_t copy_candidates,  // T*K expanded, T compact
+                                                             uint32_t copy_candidates,  // T*K expanded, T compact, list entries when ordered
+                                                             uint32_t source_limit,     // T*K
                                                              uint32_t copy_blocks,
                                                              uint32_t total_blocks,
                                                              uint32_t blocks_per_xcd,
+                                                             uint32_t pad_blocks,
                                                              uint32_t parts,            // workgroups per candidate group (rows longer than 16 chunks)
+                                                             uint32_t parts_magic,      // fast divisor by parts
+                                                             uint32_t parts_shift,
                                                              uint32_t chunks_per_block,  // == blockDim.y
                                                              uint32_t rows_per_block,    // == blockDim.z
                                                              uint32_t pad_per_expert,
@@ -632,19 +721,33 @@ __global__ void __launch_bounds__(1024) dispatch_rows_kernel(const u32x4* __rest
                                                              int num_topk,
                                                              int topk_shift,  // log2(K) when K is a power of two, else -1
                                                              int expand) {
+    NANOEP_FETCH_ARGS_4(x, weights, recv_x, recv_weights);
+    NANOEP_FETCH_ARGS_4(token_slots, slot_order, dst_slots, recv_metadata);
+    NANOEP_FETCH_ARGS_4(out_rows, recv_count, copy_candidates, source_limit);
+    NANOEP_FETCH_ARGS_4(parts_magic, parts_shift, vectors, chunks);
+    NANOEP_FETCH_ARGS_4(num_topk, topk_shift, expand, chunks_per_block);
+    if (kLookup == kLookupOrder && live_count != nullptr) {
+        // The list length was not known when the grid was sized: shrink the walk to the entries in
+        // use, so that the per-XCD ranges split the real work and not its unused tail.
+        const int64_t live = uniform_load(live_count);
+        if (live >= 0 && live < static_cast<int64_t>(copy_candidates)) {
+            copy_candidates = static_cast<uint32_t>(live);
+            copy_blocks = (rows_per_block == 1 ? copy_candidates : (copy_candidates + rows_per_block - 1) / rows_per_block) * parts;
+            total_blocks = copy_blocks + pad_blocks;
+            blocks_per_xcd = (total_blocks + kNumXcds - 1) / kNumXcds;
+        }
+    }
+    // (a grid sized for more blocks than the shrunken walk has must not spill into the next XCD's range)
     const uint32_t block = xcd_contiguous_block(blocks_per_xcd);
-    if (block >= total_blocks)
+    if (block >= total_blocks || blockIdx.x / kNumXcds >= blocks_per_xcd)
         return;
     const int lane = threadIdx.x;
     const uint32_t wave_y = __builtin_amdgcn_readfirstlane(threadIdx.y);
     const uint32_t wave_z = __builtin_amdgcn_readfirstlane(threadIdx.z);
 
     if (block < copy_blocks) {
-        uint32_t group = block, part = 0;
-        if (parts > 1) {
-            group = block / parts;
-            part = block - group * parts;
-        }
+        const uint32_t group = fast_divide(block, parts_magic, parts_shift);
+        const uint32_t part = block - group * parts;
         const uint32_t candidate = group * rows_per_block + wave_z;
         const int chunk = static_cast<int>(part * chunks_per_block + wave_y);
         if (candidate >= copy_candidates || chunk >= chunks)
@@ -653,25 +756,38 @@ __global__ void __launch_bounds__(1024) dispatch_rows_kernel(const u32x4* __rest
         const bool in_row = vector < vectors;
         uint32_t token = candidate;
         int k = 0;
-        if (expand) {
-            token = topk_shift >= 0 ? candidate >> topk_shift : candidate / static_cast<uint32_t>(num_topk);
-            k = static_cast<int>(candidate - token * num_topk);
-        }
-        token = __builtin_amdgcn_readfirstlane(token);
-        k = __builtin_amdgcn_readfirstlane(k);
-        // lanes past the end of a short row re-read vector 0 instead of branching around the load
-        const u32x4 data = x[static_cast<int64_t>(token) * vectors + (in_row ? vector : 0)];
-
         int64_t out_row;
         const int32_t* fields = nullptr;
-        if (kDirectSlots && expand) {
-            out_row = uniform_load(token_slots + static_cast<int64_t>(token) * num_topk + k);
-        } else {
-            const int64_t row = uniform_load(dst_slots + token);
-            if (row < 0 || row >= recv_count)
+        u32x4 data;
+        if (kLookup == kLookupOrder) {
+            const int64_t entry = uniform_load(slot_order + candidate);
+            if (entry < 0)
                 return;
-            fields = recv_metadata + row * (num_topk + 2);
-            out_row = expand ? static_cast<int64_t>(uniform_load(fields + 2 + k)) : row;
+            const uint32_t source = static_cast<uint32_t>(entry);
+            if (source >= source_limit)
+                return;
+            out_row = entry >> 32;
+            token = topk_shift >= 0 ? source >> topk_shift : source / static_cast<uint32_t>(num_topk);
+            k = static_cast<int>(source - token * num_topk);
+            data = x[static_cast<int64_t>(token) * vectors + (in_row ? vector : 0)];
+        } else {
+            if (expand) {
+                token = topk_shift >= 0 ? candidate >> topk_shift : candidate / static_cast<uint32_t>(num_topk);
+                k = static_cast<int>(candidate - token * num_topk);
+            }
+            token = __builtin_amdgcn_readfirstlane(token);
+            k = __builtin_amdgcn_readfirstlane(k);
+            // lanes past the end of a short row re-read vector 0 instead of branching around the load
+            data = x[static_cast<int64_t>(token) * vectors + (in_row ? vector : 0)];
+            if (kLookup == kLookupTable && expand) {
+                out_row = uniform_load(token_slots + static_cast<int64_t>(token) * num_topk + k);
+            } else {
+                const int64_t row = uniform_load(dst_slots + token);
+                if (row < 0 || row >= recv_count)
+                    return;
+                fields = recv_metadata + row * (num_topk + 2);
+                out_row = expand ? static_cast<int64_t>(uniform_load(fields + 2 + k)) : row;
+            }
         }
         if (out_row < 0 || out_row >= out_rows)
             return;
@@ -754,6 +870,8 @@ __global__ void __launch_bounds__(1024) combine_rows_kernel(const u32x4* __restr
                                                             int64_t y_rows,
                                                             uint32_t num_tokens,
                                                             uint32_t parts,
+                                                            uint32_t parts_magic,  // fast divisor by parts
+                                                            uint32_t parts_shift,
                                                             uint32_t chunks_per_block,  // == blockDim.y
                                                             uint32_t tokens_per_block,  // == blockDim.z
                                                             int vectors,
@@ -761,14 +879,16 @@ __global__ void __launch_bounds__(1024) combine_rows_kernel(const u32x4* __restr
                                                             int num_topk,
                                                             int expand,
                                                             int multiple_reduction) {
+    NANOEP_FETCH_ARGS_4(y, weights, bias, out_x);
+    NANOEP_FETCH_ARGS_4(recv_metadata, dst_slots, token_slots, out_weights);
+    NANOEP_FETCH_ARGS_4(recv_count, y_rows, num_tokens, parts);
+    NANOEP_FETCH_ARGS_4(parts_magic, parts_shift, chunks_per_block, tokens_per_block);
+    NANOEP_FETCH_ARGS_4(vectors, chunks, num_topk, expand);
     const int lane = threadIdx.x;
     const uint32_t wave_y = __builtin_amdgcn_readfirstlane(threadIdx.y);
     const uint32_t wave_z = __builtin_amdgcn_readfirstlane(threadIdx.z);
-    uint32_t group = blockIdx.x, part = 0;
-    if (parts > 1) {
-        group = blockIdx.x / parts;
-        part = blockIdx.x - group * parts;
-    }
+    const uint32_t group = fast_divide(blockIdx.x, parts_magic, parts_shift);
+    const uint32_t part = blockIdx.x - group * parts;
     const uint32_t token = __builtin_amdgcn_readfirstlane(group * tokens_per_block + wave_z);
     const int chunk = static_cast<int>(part * chunks_per_block + wave_y);
     if (token >= num_tokens || chunk >= chunks)
@@ -869,13 +989,19 @@ struct RowBlocking {
     unsigned parts;
 };
 
-RowBlocking pick_row_blocking(int chunks) {
+RowBlocking pick_row_blocking(int chunks, bool ordered = false) {
     RowBlocking blocking{};
-    // Two-wavefront workgroups measured best or within noise of best on every shape tried
-    // (rows of 4 to 14 chunks, expanded and compact); they retire and refill quickest.
+    // Token-order walks: two-wavefront workgroups measured best or within noise of best on every
+    // shape tried (rows of 4 to 14 chunks, expanded and compact); they retire and refill quickest.
+    // Slot-order walks do better with the row split evenly over workgroups of up to 8 wavefronts.
     int per_block = env_int("NANOEP_CHUNKS_PER_BLOCK", 0);
-    if (per_block < 1 || per_block > kMaxWavesPerBlock)
+    if (per_block < 1 || per_block > kMaxWavesPerBlock) {
         per_block = kDefaultChunksPerBlock;
+        if (ordered) {
+            const int pieces = (chunks + 7) / 8;
+            per_block = (chunks + pieces - 1) / pieces;
+        }
+    }
     if (per_block > chunks)
         per_block = chunks;
     blocking.chunks_per_block = static_cast<unsigned>(per_block);
@@ -915,7 +1041,7 @@ bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) ==
 
 extern "C" {
 
-int nanoep_abi_version(void) { return 1; }
+int nanoep_abi_version(void) { return 2; }
 
 const char* nanoep_status_string(int status) {
     switch (status) {
@@ -982,11 +1108,24 @@ size_t nanoep_layout_workspace_bytes(int64_t num_tokens, int num_topk, int64_t n
     return carve_layout_workspace(nullptr, num_tokens, num_topk, num_local_experts).bytes;
 }
 
+int nanoep_layout_block_tokens(int64_t num_local_experts) {
+    return num_local_experts <= 0 ? 0 : layout_tokens_per_block(num_local_experts);
+}
+
+int64_t nanoep_slot_order_entries(int64_t num_tokens, int num_topk, int64_t num_local_experts) {
+    if (num_tokens < 0 || num_topk <= 0 || num_local_experts <= 0)
+        return 0;
+    const int per_block = layout_tokens_per_block(num_local_experts);
+    if (per_block == 0 || num_tokens == 0)
+        return 0;
+    return (num_tokens + per_block - 1) / per_block * per_block * num_topk + 1;
+}
+
 int nanoep_layout(const int64_t* topk_idx, int64_t num_tokens, int num_topk, int64_t num_local_experts,
                   int64_t alignment, int expand, int32_t* recv_metadata, int64_t* expert_counts,
                   int64_t* expert_offsets, int64_t* dst_slots, int64_t* send_counts, int64_t* topk_snapshot,
-                  int64_t* recv_rank_prefix, int32_t* token_slots, void* workspace, size_t workspace_bytes,
-                  int64_t* host_counts, void* stream_handle) {
+                  int64_t* recv_rank_prefix, int32_t* token_slots, int64_t* slot_order, void* workspace,
+                  size_t workspace_bytes, int64_t* host_counts, void* stream_handle) {
     if (num_tokens < 0 || num_tokens > INT32_MAX || num_topk <= 0 || num_topk > kMaxTopk || num_local_experts <= 0 ||
         num_local_experts >= (int64_t{1} << (31 - kRankBits)) || alignment <= 0 || alignment > (int64_t{1} << 31))
         return NANOEP_ERR_INVALID_ARGUMENT;
@@ -994,6 +1133,9 @@ int nanoep_layout(const int64_t* topk_idx, int64_t num_tokens, int num_topk, int
         host_counts == nullptr || workspace == nullptr)
         return NANOEP_ERR_INVALID_ARGUMENT;
     if (num_tokens > 0 && (topk_idx == nullptr || recv_metadata == nullptr || dst_slots == nullptr || topk_snapshot == nullptr))
+        return NANOEP_ERR_INVALID_ARGUMENT;
+    // the slot-order list packs token * K + k into 32 bits and only exists for the expanded layout
+    if (slot_order != nullptr && (!expand || num_tokens * num_topk >= (int64_t{1} << 31)))
         return NANOEP_ERR_INVALID_ARGUMENT;
     const int tokens_per_block = layout_tokens_per_block(num_local_experts);
     if (tokens_per_block == 0)
@@ -1028,23 +1170,25 @@ int nanoep_layout(const int64_t* topk_idx, int64_t num_tokens, int num_topk, int
             if ((launch_status = hipGetLastError()) != hipSuccess)
                 return;
         }
+        const size_t assign_lds = static_cast<size_t>(experts + 1) * 12;
         if (fused_scan) {
-            layout_scan_assign_kernel<kCap><<<blocks, count_threads, static_cast<size_t>(experts + 1) * 8, stream>>>(
+            layout_assign_kernel<kCap, true><<<blocks, count_threads, assign_lds, stream>>>(
                 ws.block_counts, ws.block_status, blocks, num_tokens, num_topk, experts, tokens_per_block, count_threads,
                 expand, alignment, ws.packed_rank, ws.local_row, expert_counts, expert_offsets, send_counts,
-                recv_rank_prefix, host_counts, recv_metadata, dst_slots, token_slots);
+                recv_rank_prefix, ws.totals, host_counts, recv_metadata, dst_slots, token_slots, slot_order);
             launch_status = hipGetLastError();
             return;
         }
         layout_scan_kernel<<<1, kScanThreads, static_cast<size_t>(experts + 1) * 4, stream>>>(
             ws.block_counts, ws.block_status, blocks, experts, alignment, expert_counts, expert_offsets, send_counts,
-            recv_rank_prefix, host_counts);
+            recv_rank_prefix, ws.totals, host_counts);
         if ((launch_status = hipGetLastError()) != hipSuccess)
             return;
         if (blocks > 0) {
-            layout_assign_kernel<kCap><<<blocks, count_threads, 0, stream>>>(
-                num_tokens, num_topk, experts, tokens_per_block, expand, ws.block_counts, ws.packed_rank, ws.local_row,
-                expert_offsets, recv_metadata, dst_slots, token_slots);
+            layout_assign_kernel<kCap, false><<<blocks, count_threads, assign_lds, stream>>>(
+                ws.block_counts, ws.block_status, blocks, num_tokens, num_topk, experts, tokens_per_block, count_threads,
+                expand, alignment, ws.packed_rank, ws.local_row, expert_counts, expert_offsets, send_counts,
+                recv_rank_prefix, ws.totals, host_counts, recv_metadata, dst_slots, token_slots, slot_order);
             launch_status = hipGetLastError();
         }
     });
@@ -1089,7 +1233,8 @@ int nanoep_wait_counts(int64_t* host_counts, void* stream_handle, double timeout
 }
 
 int nanoep_dispatch(const void* x, const float* weights, const int32_t* recv_metadata, const int64_t* dst_slots,
-                    const int32_t* token_slots, const int64_t* expert_counts, const int64_t* expert_offsets,
+                    const int32_t* token_slots, const int64_t* slot_order, int64_t slot_order_entries,
+                    const int64_t* expert_counts, const int64_t* expert_offsets,
                     int64_t recv_count, int64_t expanded_capacity, int64_t num_tokens, int hidden, int num_topk,
                     int64_t num_local_experts, int64_t alignment, int expand, int zero_padding, void* recv_x,
                     int64_t* recv_topk_idx, float* recv_weights, int num_cus, void* stream_handle) {
@@ -1116,11 +1261,21 @@ int nanoep_dispatch(const void* x, const float* weights, const int32_t* recv_met
     if (pad && (expert_counts == nullptr || expert_offsets == nullptr))
         return NANOEP_ERR_INVALID_ARGUMENT;
 
+    // full list length without its trailing count word
+    const int64_t order_bound = nanoep_slot_order_entries(num_tokens, num_topk, num_local_experts) - 1;
+    const bool ordered = expand && slot_order != nullptr && order_bound > 0 && env_int("NANOEP_DISPATCH_ORDER", 1) != 0;
+    if (ordered && (slot_order_entries > order_bound || num_tokens * num_topk >= (int64_t{1} << 31)))
+        return NANOEP_ERR_INVALID_ARGUMENT;
+    // a negative entry count defers to the count word the layout stored behind the list
+    const int64_t* live_count = ordered && slot_order_entries < 0 ? slot_order + order_bound : nullptr;
+    if (live_count != nullptr)
+        slot_order_entries = order_bound;
+
     const int vectors = hidden / 8;
     const int chunks = (vectors + kWave - 1) / kWave;
-    const RowBlocking blocking = pick_row_blocking(chunks);
+    const RowBlocking blocking = pick_row_blocking(chunks, ordered);
     const int64_t waves = static_cast<int64_t>(blocking.chunks_per_block) * blocking.rows_per_block;
-    const int64_t copy_candidates = expand ? num_tokens * num_topk : num_tokens;
+    const int64_t copy_candidates = ordered ? slot_order_entries : expand ? num_tokens * num_topk : num_tokens;
     const int64_t copy_blocks = (copy_candidates + blocking.rows_per_block - 1) / blocking.rows_per_block * blocking.parts;
     // No expert's gap exceeds alignment-1 rows, and all gaps together stay below C.
     const int64_t pad_per_expert = !pad ? 0 : (alignment - 1 < expanded_capacity ? alignment - 1 : expanded_capacity);
@@ -1136,20 +1291,25 @@ int nanoep_dispatch(const void* x, const float* weights, const int32_t* recv_met
 
     const dim3 grid(blocks_per_xcd * kNumXcds);
     const dim3 block(kWave, blocking.chunks_per_block, blocking.rows_per_block);
+    const FastDivisor parts_divisor = make_fast_divisor(blocking.parts);
     auto stream = static_cast<hipStream_t>(stream_handle);
-#define NANOEP_LAUNCH_DISPATCH(DIRECT)                                                                               \
-    dispatch_rows_kernel<DIRECT><<<grid, block, 0, stream>>>(                                                        \
-        static_cast<const u32x4*>(x), weights, recv_metadata, dst_slots, token_slots, expert_counts, expert_offsets, \
-        static_cast<u32x4*>(recv_x), recv_topk_idx, recv_weights, recv_count, out_rows,                              \
-        static_cast<uint32_t>(copy_candidates), static_cast<uint32_t>(copy_blocks), static_cast<uint32_t>(total_blocks), \
-        blocks_per_xcd, blocking.parts, blocking.chunks_per_block, blocking.rows_per_block,                          \
-        static_cast<uint32_t>(pad_per_expert),                                                                       \
+#define NANOEP_LAUNCH_DISPATCH(LOOKUP)                                                                               \
+    dispatch_rows_kernel<LOOKUP><<<grid, block, 0, stream>>>(                                                        \
+        static_cast<const u32x4*>(x), weights, recv_metadata, dst_slots, token_slots, slot_order, live_count,        \
+        expert_counts,                                                                                               \
+        expert_offsets, static_cast<u32x4*>(recv_x), recv_topk_idx, recv_weights, recv_count, out_rows,              \
+        static_cast<uint32_t>(copy_candidates), static_cast<uint32_t>(num_tokens * num_topk),                        \
+        static_cast<uint32_t>(copy_blocks), static_cast<uint32_t>(total_blocks), blocks_per_xcd,                     \
+        static_cast<uint32_t>(total_blocks - copy_blocks), blocking.parts, parts_divisor.magic, parts_divisor.shift, blocking.chunks_per_block,         \
+        blocking.rows_per_block, static_cast<uint32_t>(pad_per_expert),                                              \
         static_cast<uint32_t>(pad_groups_per_expert > 0 ? pad_groups_per_expert : 1), vectors, chunks, num_topk,     \
         topk_shift, expand ? 1 : 0)
-    if (token_slots != nullptr && expand)
-        NANOEP_LAUNCH_DISPATCH(true);
+    if (ordered)
+        NANOEP_LAUNCH_DISPATCH(kLookupOrder);
+    else if (token_slots != nullptr && expand)
+        NANOEP_LAUNCH_DISPATCH(kLookupTable);
     else
-        NANOEP_LAUNCH_DISPATCH(false);
+        NANOEP_LAUNCH_DISPATCH(kLookupMetadata);
 #undef NANOEP_LAUNCH_DISPATCH
     NANOEP_HIP_TRY(hipGetLastError());
     return NANOEP_OK;
@@ -1191,11 +1351,13 @@ int nanoep_combine(const void* y, const float* weights, const void* bias, const 
     const int gathered = expand ? num_topk : 1;
     // the slot table only helps the expanded layout, and only when something was received
     const bool direct = token_slots != nullptr && expand && recv_count > 0;
+    const FastDivisor parts_divisor = make_fast_divisor(blocking.parts);
 #define NANOEP_LAUNCH_COMBINE(GROUP, DIRECT)                                                                       \
     combine_rows_kernel<GROUP, DIRECT><<<grid, block, 0, stream>>>(                                                \
         static_cast<const u32x4*>(y), weights, static_cast<const u32x4*>(bias), recv_metadata, dst_slots,          \
         token_slots, static_cast<u32x4*>(out_x), out_weights, recv_count, y_rows, static_cast<uint32_t>(num_tokens), \
-        blocking.parts, blocking.chunks_per_block, blocking.rows_per_block, vectors, chunks, num_topk, expand ? 1 : 0, \
+        blocking.parts, parts_divisor.magic, parts_divisor.shift, blocking.chunks_per_block, blocking.rows_per_block,  \
+        vectors, chunks, num_topk, expand ? 1 : 0,                                                                   \
         multiple_reduction ? 1 : 0)
 #define NANOEP_LAUNCH_COMBINE_GROUP(GROUP)    \
     do {                                     \

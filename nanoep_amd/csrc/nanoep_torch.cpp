@@ -240,6 +240,22 @@ const int32_t* slot_table(const std::vector<torch::Tensor>& metadata, int64_t to
     return table.numel() == 0 ? nullptr : table.data_ptr<int32_t>();
 }
 
+// The optional ninth handle tensor: int64 slot-order list written by the layout kernels.
+const int64_t* slot_order_list(const std::vector<torch::Tensor>& metadata, int64_t tokens, int64_t topk, int64_t local_experts,
+                               bool expand, int64_t* entries) {
+    *entries = 0;
+    if (!expand || metadata.size() < 9 || !metadata[8].defined())
+        return nullptr;
+    const auto& order = metadata[8];
+    TORCH_CHECK(order.device() == metadata[0].device() && order.scalar_type() == torch::kInt64 && order.is_contiguous() &&
+                    order.dim() == 1 && order.size(0) <= nanoep_slot_order_entries(tokens, static_cast<int>(topk), local_experts),
+                "cached slot-order list has invalid CUDA storage or shape");
+    // the whole buffer (list + count word) defers to the count on the device
+    const bool whole = order.numel() > 0 && order.numel() == nanoep_slot_order_entries(tokens, static_cast<int>(topk), local_experts);
+    *entries = whole ? -1 : order.numel();
+    return order.numel() == 0 ? nullptr : order.data_ptr<int64_t>();
+}
+
 // Communication stream waits for the producer of the inputs: the caller's stream, an explicit
 // event, or both (csrc/pipeline.cu:364-377 in the reference).
 // An external-stream wrapper never compares equal to a pool stream object, so identity is decided
@@ -295,8 +311,8 @@ DispatchResult dispatch(PeerRuntime& runtime,
                         int64_t previous_event,
                         bool async_op) {
     const bool cached = !cached_metadata.empty();
-    TORCH_CHECK(!cached || cached_metadata.size() == 7 || cached_metadata.size() == 8,
-                "cached metadata must contain the seven prepared tensors from dispatch (plus the optional slot table)");
+    TORCH_CHECK(!cached || (cached_metadata.size() >= 7 && cached_metadata.size() <= 9),
+                "cached metadata must contain the seven prepared tensors from dispatch (plus the optional slot table and slot-order list)");
     const auto& routing = cached ? cached_metadata[5] : indices;
     int64_t* host_counts = runtime.host_counts();
     check_payload_inputs(x, routing, weights, runtime.device(), num_experts, max_tokens);
@@ -337,11 +353,17 @@ DispatchResult dispatch(PeerRuntime& runtime,
             return 0;
         });
     };
-    const auto launch_permute = [&](const std::vector<torch::Tensor>& handle, int64_t received, int64_t capacity) {
+    // count_on_device: the handle carries the whole slot-order buffer and the number of entries in
+    // use is not known on the host yet, so the kernel reads it from the buffer's last word
+    const auto launch_permute = [&](const std::vector<torch::Tensor>& handle, int64_t received, int64_t capacity,
+                                    bool count_on_device = false) {
+        int64_t order_entries = 0;
+        const int64_t* order = slot_order_list(handle, tokens, topk, local_experts, expand, &order_entries);
+        TORCH_CHECK(!count_on_device || order == nullptr || order_entries == -1, "slot-order buffer is incomplete");
         check_status(
             nanoep_dispatch(x.data_ptr(), weights.has_value() ? weights->data_ptr<float>() : nullptr, handle[0].data_ptr<int32_t>(),
-                            handle[3].data_ptr<int64_t>(), slot_table(handle, tokens, topk, expand), handle[1].data_ptr<int64_t>(),
-                            handle[2].data_ptr<int64_t>(), received, capacity, tokens, static_cast<int>(hidden),
+                            handle[3].data_ptr<int64_t>(), slot_table(handle, tokens, topk, expand), order, order_entries,
+                            handle[1].data_ptr<int64_t>(), handle[2].data_ptr<int64_t>(), received, capacity, tokens, static_cast<int>(hidden),
                             static_cast<int>(topk), local_experts, alignment, expand ? 1 : 0, zero_padding ? 1 : 0, out_x.data_ptr(),
                             expand ? nullptr : out_indices.data_ptr<int64_t>(),
                             weights.has_value() ? out_weights.data_ptr<float>() : nullptr, cu_budget, comm.stream()),
@@ -368,7 +390,9 @@ DispatchResult dispatch(PeerRuntime& runtime,
         TORCH_CHECK(capture == hipStreamCaptureStatusNone, "Fresh dispatch with host count polling cannot be captured in a HIP graph");
 
         const auto int64_options = routing.options();
-        torch::Tensor recv_metadata, expert_counts, expert_offsets, dst_slots, send_counts, snapshot, prefix, token_slots;
+        torch::Tensor recv_metadata, expert_counts, expert_offsets, dst_slots, send_counts, snapshot, prefix, token_slots, slot_order;
+        // the slot-order list packs token * K + k into 32 bits
+        const bool ordered = expand && tokens * topk < (int64_t{1} << 31);
         allocate_for_consumer([&] {
             recv_metadata = torch::empty({tokens, topk + 2}, int64_options.dtype(torch::kInt32));
             expert_counts = torch::empty({local_experts}, int64_options);
@@ -379,11 +403,15 @@ DispatchResult dispatch(PeerRuntime& runtime,
             prefix = torch::empty({1}, int64_options);
             if (expand)
                 token_slots = torch::empty({tokens, topk}, int64_options.dtype(torch::kInt32));
+            if (ordered)
+                slot_order = torch::empty({nanoep_slot_order_entries(tokens, static_cast<int>(topk), local_experts)}, int64_options);
             return 0;
         });
         metadata = {recv_metadata, expert_counts, expert_offsets, dst_slots, send_counts, snapshot, prefix};
         if (expand)
             metadata.push_back(token_slots);  // private eighth entry: slot[t,k] in one lookup
+        if (ordered)
+            metadata.push_back(slot_order);  // private ninth entry: assignments in block-wise slot order
         const size_t workspace_bytes = nanoep_layout_workspace_bytes(tokens, static_cast<int>(topk), local_experts);
         TORCH_CHECK(workspace_bytes > 0, "unsupported routing geometry for the layout kernels");
         auto workspace = torch::empty({static_cast<int64_t>(workspace_bytes)}, int64_options.dtype(torch::kUInt8));
@@ -391,7 +419,9 @@ DispatchResult dispatch(PeerRuntime& runtime,
                                    recv_metadata.data_ptr<int32_t>(), expert_counts.data_ptr<int64_t>(),
                                    expert_offsets.data_ptr<int64_t>(), dst_slots.data_ptr<int64_t>(), send_counts.data_ptr<int64_t>(),
                                    snapshot.data_ptr<int64_t>(), prefix.data_ptr<int64_t>(),
-                                   expand ? token_slots.data_ptr<int32_t>() : nullptr, workspace.data_ptr(), workspace_bytes,
+                                   expand ? token_slots.data_ptr<int32_t>() : nullptr,
+                                   ordered && slot_order.numel() > 0 ? slot_order.data_ptr<int64_t>() : nullptr, workspace.data_ptr(),
+                                   workspace_bytes,
                                    host_counts, comm.stream()),
                      "layout");
 
@@ -406,7 +436,7 @@ DispatchResult dispatch(PeerRuntime& runtime,
         const bool speculative = tokens > 0 && gap_bound <= tokens * topk / 4 + 1024 && row_bound <= std::numeric_limits<int32_t>::max();
         if (speculative) {
             allocate_outputs(row_bound, tokens);
-            launch_permute(metadata, tokens, row_bound);
+            launch_permute(metadata, tokens, row_bound, /*count_on_device=*/true);
         }
 
         int64_t counts[NANOEP_HOST_COUNT_WORDS] = {0, 0, 0, 0};
@@ -423,6 +453,10 @@ DispatchResult dispatch(PeerRuntime& runtime,
         TORCH_CHECK(!expand || expanded_capacity <= std::numeric_limits<int32_t>::max(),
                     "expanded capacity exceeds int32 metadata range");
         metadata[0] = recv_metadata.narrow(0, 0, recv_count);
+        if (ordered) {
+            TORCH_CHECK(counts[2] >= 0 && counts[2] <= slot_order.size(0), "assignment count exceeds the slot-order list");
+            metadata[8] = slot_order.narrow(0, 0, counts[2]);  // replays walk the A assignments only
+        }
         if (speculative) {
             TORCH_CHECK(!expand || expanded_capacity <= row_bound, "expanded capacity exceeds its upper bound");
             out_x = out_x.narrow(0, 0, expand ? expanded_capacity : recv_count);
@@ -472,7 +506,7 @@ CombineResult combine(PeerRuntime& runtime,
                       int64_t comm_stream,
                       int64_t previous_event,
                       bool async_op) {
-    TORCH_CHECK((metadata.size() == 7 || metadata.size() == 8) && x.dim() == 2 && metadata[5].dim() == 2,
+    TORCH_CHECK(metadata.size() >= 7 && metadata.size() <= 9 && x.dim() == 2 && metadata[5].dim() == 2,
                 "combine requires a 2D payload and seven prepared metadata tensors");
     (void)runtime.host_counts();  // rejects a closed runtime
     const auto device = static_cast<c10::DeviceIndex>(runtime.device());

@@ -40,9 +40,13 @@ def lib() -> ctypes.CDLL:
         handle.nanoep_window_layout.argtypes = [i, i64, i, i, i64, i, ctypes.POINTER(i64)]
         handle.nanoep_layout_workspace_bytes.restype = sz
         handle.nanoep_layout_workspace_bytes.argtypes = [i64, i, i64]
-        handle.nanoep_layout.argtypes = [p, i64, i, i64, i64, i, p, p, p, p, p, p, p, p, p, sz, p, p]
+        handle.nanoep_layout_block_tokens.restype = i
+        handle.nanoep_layout_block_tokens.argtypes = [i64]
+        handle.nanoep_slot_order_entries.restype = i64
+        handle.nanoep_slot_order_entries.argtypes = [i64, i, i64]
+        handle.nanoep_layout.argtypes = [p, i64, i, i64, i64, i, p, p, p, p, p, p, p, p, p, p, sz, p, p]
         handle.nanoep_wait_counts.argtypes = [p, p, dbl, ctypes.POINTER(i64)]
-        handle.nanoep_dispatch.argtypes = [p, p, p, p, p, p, p, i64, i64, i64, i, i, i64, i64, i, i, p, p, p, i, p]
+        handle.nanoep_dispatch.argtypes = [p, p, p, p, p, p, i64, p, p, i64, i64, i64, i, i, i64, i64, i, i, p, p, p, i, p]
         handle.nanoep_combine.argtypes = [p, p, p, p, p, p, i64, i64, i64, i, i, i, i, p, p, i, p]
         handle.nanoep_copy_bytes.argtypes = [p, p, sz, p]
         _lib = handle
@@ -76,7 +80,7 @@ def window_layout(ranks, tokens, hidden, topk, experts, multi=False) -> list[int
 
 
 def layout(topk_idx: torch.Tensor, num_local_experts: int, alignment: int, expand: bool, *, raise_on_routing=True):
-    """Runs the layout kernels and returns (metadata list of 7, (N, C, A, status))."""
+    """Runs the layout kernels and returns (metadata list of 7, or 9 when expanded, (N, C, A, status))."""
     device = topk_idx.device
     tokens, topk = topk_idx.shape
     i64 = dict(dtype=torch.int64, device=device)
@@ -88,6 +92,10 @@ def layout(topk_idx: torch.Tensor, num_local_experts: int, alignment: int, expan
     snapshot = torch.empty_like(topk_idx)
     prefix = torch.empty(1, **i64)
     token_slots = torch.empty((tokens, topk), dtype=torch.int32, device=device) if expand else None
+    slot_order = None
+    if expand:
+        entries = lib().nanoep_slot_order_entries(tokens, topk, num_local_experts)
+        slot_order = torch.full((entries,), -7, dtype=torch.int64, device=device)
     ws_bytes = lib().nanoep_layout_workspace_bytes(tokens, topk, num_local_experts)
     workspace = torch.empty(ws_bytes, dtype=torch.uint8, device=device)
     mailbox = torch.empty(HOST_COUNT_WORDS, dtype=torch.int64, pin_memory=True)
@@ -95,7 +103,7 @@ def layout(topk_idx: torch.Tensor, num_local_experts: int, alignment: int, expan
         lib().nanoep_layout(
             ptr(topk_idx), tokens, topk, num_local_experts, alignment, int(expand), ptr(recv_metadata),
             ptr(expert_counts), ptr(expert_offsets), ptr(dst_slots), ptr(send_counts), ptr(snapshot), ptr(prefix),
-            ptr(token_slots), ptr(workspace), ws_bytes, mailbox.data_ptr(), stream_handle(),
+            ptr(token_slots), ptr(slot_order), ptr(workspace), ws_bytes, mailbox.data_ptr(), stream_handle(),
         )
     )
     out = (ctypes.c_int64 * HOST_COUNT_WORDS)()
@@ -107,6 +115,7 @@ def layout(topk_idx: torch.Tensor, num_local_experts: int, alignment: int, expan
     metadata = [recv_metadata[: counts[0]], expert_counts, expert_offsets, dst_slots, send_counts, snapshot, prefix]
     if token_slots is not None:
         metadata.append(token_slots)  # private eighth entry: the one-lookup slot table
+        metadata.append(slot_order)  # private ninth entry: assignments in block-wise slot order
     return metadata, counts
 
 
@@ -114,8 +123,12 @@ def token_slots_of(metadata, use_table=True):
     return metadata[7] if use_table and len(metadata) > 7 else None
 
 
+def slot_order_of(metadata, use_order=True):
+    return metadata[8] if use_order and len(metadata) > 8 else None
+
+
 def dispatch(x, weights, metadata, counts, num_local_experts, alignment, expand, zero_padding, *, num_cus=0, poison=None,
-             use_table=True):
+             use_table=True, use_order=True, order_count="exact"):
     """Returns (recv_x, recv_topk_idx | None, recv_weights | None) through nanoep_dispatch."""
     recv_metadata, expert_counts, expert_offsets, dst_slots = metadata[0], metadata[1], metadata[2], metadata[3]
     received, capacity = counts[0], counts[1]
@@ -133,10 +146,13 @@ def dispatch(x, weights, metadata, counts, num_local_experts, alignment, expand,
     recv_x = new((rows, hidden), torch.bfloat16)
     recv_idx = None if expand else new((rows, topk), torch.int64)
     recv_w = None if weights is None else new((rows,) if expand else (rows, topk), torch.float32)
+    order = slot_order_of(metadata, use_order)
+    # exact count A, or -1: the kernel reads A from the word behind the list
+    order_entries = 0 if order is None else (counts[2] if order_count == "exact" else -1)
     check(
         lib().nanoep_dispatch(
-            ptr(x), ptr(weights), ptr(recv_metadata), ptr(dst_slots), ptr(token_slots_of(metadata, use_table)), ptr(expert_counts),
-            ptr(expert_offsets), received, capacity,
+            ptr(x), ptr(weights), ptr(recv_metadata), ptr(dst_slots), ptr(token_slots_of(metadata, use_table)),
+            ptr(order), order_entries, ptr(expert_counts), ptr(expert_offsets), received, capacity,
             tokens, hidden, topk, num_local_experts, alignment, int(expand), int(zero_padding), ptr(recv_x),
             ptr(recv_idx), ptr(recv_w), num_cus, stream_handle(),
         )

@@ -12,7 +12,8 @@ from oracle import nanoep_oracle as oracle
 def test_every_declared_symbol_is_exported():
     declared = cabi.declared_symbols()
     assert {"nanoep_layout", "nanoep_dispatch", "nanoep_combine", "nanoep_wait_counts", "nanoep_window_layout",
-            "nanoep_layout_workspace_bytes", "nanoep_copy_bytes", "nanoep_abi_version"} <= set(declared)
+            "nanoep_layout_workspace_bytes", "nanoep_copy_bytes", "nanoep_abi_version",
+            "nanoep_slot_order_entries", "nanoep_layout_block_tokens"} <= set(declared)
     library = cabi.lib()
     for name in declared:
         assert hasattr(library, name), f"{name} is declared in include/nanoep_hip.h but not exported"
@@ -20,7 +21,7 @@ def test_every_declared_symbol_is_exported():
 
 def test_version_and_status_strings():
     library = cabi.lib()
-    assert library.nanoep_abi_version() == 1
+    assert library.nanoep_abi_version() == 2
     texts = [library.nanoep_status_string(code).decode() for code in range(0, 7)]
     assert texts[0] == "ok" and len(set(texts[:6])) == 6 and texts[6] == "unknown status"
     assert library.nanoep_last_hip_error().decode() == ""
@@ -54,14 +55,19 @@ def test_argument_checks_come_before_any_device_work():
     library = cabi.lib()
     null = None
     # hidden not a multiple of 8, top-k out of range, negative counts, unaligned pointers
-    assert library.nanoep_dispatch(null, null, null, null, null, null, null, 0, 0, 0, 7, 2, 4, 1, 0, 0, null, null, null, 0, null) == 1
-    assert library.nanoep_dispatch(null, null, null, null, null, null, null, 0, 0, 0, 256, 33, 4, 1, 0, 0, null, null, null, 0, null) == 1
-    assert library.nanoep_dispatch(null, null, null, null, null, null, null, 5, 0, 4, 256, 2, 4, 1, 0, 0, null, null, null, 0, null) == 1
-    assert library.nanoep_dispatch(8, null, null, null, null, null, null, 0, 0, 0, 256, 2, 4, 1, 0, 0, null, null, null, 0, null) == 1
+    assert library.nanoep_dispatch(null, null, null, null, null, null, 0, null, null, 0, 0, 0, 7, 2, 4, 1, 0, 0, null, null, null, 0, null) == 1
+    assert library.nanoep_dispatch(null, null, null, null, null, null, 0, null, null, 0, 0, 0, 256, 33, 4, 1, 0, 0, null, null, null, 0, null) == 1
+    assert library.nanoep_dispatch(null, null, null, null, null, null, 0, null, null, 5, 0, 4, 256, 2, 4, 1, 0, 0, null, null, null, 0, null) == 1
+    assert library.nanoep_dispatch(8, null, null, null, null, null, 0, null, null, 0, 0, 0, 256, 2, 4, 1, 0, 0, null, null, null, 0, null) == 1
     assert library.nanoep_combine(null, null, null, null, null, null, 0, 0, 0, 250, 2, 1, 0, null, null, 0, null) == 1
     assert library.nanoep_combine(null, null, null, null, null, null, 3, 0, 2, 256, 2, 1, 0, null, null, 0, null) == 1
     assert library.nanoep_copy_bytes(null, null, 24, null) == 1
-    assert library.nanoep_layout(null, -1, 2, 4, 1, 0, null, null, null, null, null, null, null, null, null, 0, null, null) == 1
-    assert library.nanoep_layout(null, 4, 2, 4, 0, 0, null, null, null, null, null, null, null, null, null, 0, null, null) == 1
+    assert library.nanoep_layout(null, -1, 2, 4, 1, 0, null, null, null, null, null, null, null, null, null, null, 0, null, null) == 1
+    assert library.nanoep_layout(null, 4, 2, 4, 0, 0, null, null, null, null, null, null, null, null, null, null, 0, null, null) == 1
+    # a slot-order list only exists for the expanded layout
+    assert library.nanoep_layout(null, 4, 2, 4, 1, 0, null, 8, 8, null, 8, null, 8, null, 8, 8, 0, 8, null) == 1
+    assert library.nanoep_slot_order_entries(4096, 8, 256) == 4096 * 8 + 1 and library.nanoep_layout_block_tokens(256) == 256
+    assert library.nanoep_slot_order_entries(100, 3, 8) == 256 * 3 + 1 and library.nanoep_slot_order_entries(0, 3, 8) == 0
+    assert library.nanoep_layout_block_tokens(6000) == 0 and library.nanoep_layout_block_tokens(0) == 0
     out = (ctypes.c_int64 * 4)()
     assert library.nanoep_wait_counts(null, null, 0.0, out) == 1

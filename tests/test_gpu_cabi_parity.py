@@ -44,6 +44,22 @@ def assert_layout(metadata, counts, expected: oracle.Layout, expand):
         table = torch.full(expected.topk_idx.shape, -1, dtype=torch.int32)
         table[expected.src_tokens] = expected.expanded_slots.to(torch.int32)
         assert torch.equal(metadata[7].cpu(), table), "token_slots"
+        # private slot-order list: block of consecutive tokens by block, the valid assignments as
+        # (slot << 32) | (t * K + k) in ascending slot order, without gaps; -1 from entry A on
+        tokens, topk = expected.topk_idx.shape
+        block_tokens = cabi.lib().nanoep_layout_block_tokens(expected.expert_counts.numel())
+        flat = table.flatten().to(torch.int64)
+        packed = (flat << 32) | torch.arange(flat.numel(), dtype=torch.int64)
+        want = []
+        for first in range(0, tokens, block_tokens):
+            part = packed[first * topk : (first + block_tokens) * topk]
+            want.append(part[flat[first * topk : (first + block_tokens) * topk] >= 0].sort().values)
+        entries = cabi.lib().nanoep_slot_order_entries(tokens, topk, expected.expert_counts.numel())
+        if entries:
+            want.append(torch.full((entries - 1 - counts[2],), -1, dtype=torch.int64))
+            want.append(torch.tensor([counts[2]], dtype=torch.int64))  # count word behind the list
+        want = torch.cat(want) if want else torch.empty(0, dtype=torch.int64)
+        assert torch.equal(metadata[8].cpu(), want), "slot_order"
 
 
 def run_dispatch_combine(device, idx, hidden, experts, alignment, expand, zero_padding, weighted, *, seed=0, num_cus=0):
@@ -63,10 +79,24 @@ def run_dispatch_combine(device, idx, hidden, experts, alignment, expand, zero_p
         # the same handle without the private slot table must give the same bytes
         plain_x, _, plain_w = cabi.dispatch(
             x.to(device), None if w is None else w.to(device), metadata, counts, experts, alignment, expand, zero_padding,
-            num_cus=num_cus, poison=POISON, use_table=False,
+            num_cus=num_cus, poison=POISON, use_table=False, use_order=False,
         )
         assert torch.equal(plain_x.view(torch.int16), got_x.view(torch.int16))
         assert plain_w is None or torch.equal(plain_w.view(torch.int32), got_w.view(torch.int32))
+        # ... so must the slot-order walk that reads its entry count on the device
+        device_x, _, device_w = cabi.dispatch(
+            x.to(device), None if w is None else w.to(device), metadata, counts, experts, alignment, expand, zero_padding,
+            num_cus=num_cus, poison=POISON, order_count="device",
+        )
+        assert torch.equal(device_x.view(torch.int16), got_x.view(torch.int16))
+        assert device_w is None or torch.equal(device_w.view(torch.int32), got_w.view(torch.int32))
+        # ... and so must the token-order walk with the slot table
+        table_x, _, table_w = cabi.dispatch(
+            x.to(device), None if w is None else w.to(device), metadata, counts, experts, alignment, expand, zero_padding,
+            num_cus=num_cus, poison=POISON, use_order=False,
+        )
+        assert torch.equal(table_x.view(torch.int16), got_x.view(torch.int16))
+        assert table_w is None or torch.equal(table_w.view(torch.int32), got_w.view(torch.int32))
         assert got_idx is None
         live = torch.zeros(counts[1], dtype=torch.bool)
         live[expected_layout.expanded_slots[expected_layout.expanded_slots >= 0]] = True
