@@ -632,14 +632,8 @@ __device__ __forceinline__ T uniform_load(const T* p) {
     return *(const __attribute__((address_space(4))) T*)(p);
 }
 
-// Workgroups are handed to the 8 XCDs round-robin by their linear id, and every XCD has its own
-// L2.  Giving XCD i the contiguous logical range [i * blocks_per_xcd, (i+1) * blocks_per_xcd)
-// keeps neighbouring work items (which share their source row) behind one L2.
+// Workgroups are handed to the 8 XCDs round-robin by their linear id, and every XCD has its own L2.
 constexpr int kNumXcds = 8;
-
-__device__ __forceinline__ uint32_t xcd_contiguous_block(uint32_t blocks_per_xcd) {
-    return (blockIdx.x % kNumXcds) * blocks_per_xcd + blockIdx.x / kNumXcds;
-}
 
 // n / d for n < 2^31 as one 64-bit multiply and shift: magic = ceil(2^shift / d), shift = 31 + ceil(log2 d).
 struct FastDivisor {
@@ -706,9 +700,9 @@ __global__ void __launch_bounds__(1024) dispatch_rows_kernel(const u32x4* __rest
                                                              uint32_t copy_candidates,  // T*K expanded, T compact, list entries when ordered
                                                              uint32_t source_limit,     // T*K
                                                              uint32_t copy_blocks,
-                                                             uint32_t total_blocks,
-                                                             uint32_t blocks_per_xcd,
+                                                             uint32_t copy_per_xcd,  // ceil(copy_blocks / 8)
                                                              uint32_t pad_blocks,
+                                                             uint32_t pad_per_xcd,   // ceil(pad_blocks / 8)
                                                              uint32_t parts,            // workgroups per candidate group (rows longer than 16 chunks)
                                                              uint32_t parts_magic,      // fast divisor by parts
                                                              uint32_t parts_shift,
@@ -733,19 +727,23 @@ __global__ void __launch_bounds__(1024) dispatch_rows_kernel(const u32x4* __rest
         if (live >= 0 && live < static_cast<int64_t>(copy_candidates)) {
             copy_candidates = static_cast<uint32_t>(live);
             copy_blocks = (rows_per_block == 1 ? copy_candidates : (copy_candidates + rows_per_block - 1) / rows_per_block) * parts;
-            total_blocks = copy_blocks + pad_blocks;
-            blocks_per_xcd = (total_blocks + kNumXcds - 1) / kNumXcds;
+            copy_per_xcd = (copy_blocks + kNumXcds - 1) / kNumXcds;
         }
     }
-    // (a grid sized for more blocks than the shrunken walk has must not spill into the next XCD's range)
-    const uint32_t block = xcd_contiguous_block(blocks_per_xcd);
-    if (block >= total_blocks || blockIdx.x / kNumXcds >= blocks_per_xcd)
+    // Workgroups are handed to the XCDs round-robin.  Each XCD takes one contiguous range of the
+    // copy work followed by one contiguous range of the zero-fill work, so neighbouring work items
+    // (which share their source rows) stay behind one L2 and every XCD gets its share of both.
+    const uint32_t xcd = blockIdx.x % kNumXcds;
+    const uint32_t index_in_xcd = blockIdx.x / kNumXcds;
+    const bool copy_work = index_in_xcd < copy_per_xcd;
+    const uint32_t block = copy_work ? xcd * copy_per_xcd + index_in_xcd : xcd * pad_per_xcd + (index_in_xcd - copy_per_xcd);
+    if (copy_work ? block >= copy_blocks : (index_in_xcd - copy_per_xcd >= pad_per_xcd || block >= pad_blocks))
         return;
     const int lane = threadIdx.x;
     const uint32_t wave_y = __builtin_amdgcn_readfirstlane(threadIdx.y);
     const uint32_t wave_z = __builtin_amdgcn_readfirstlane(threadIdx.z);
 
-    if (block < copy_blocks) {
+    if (copy_work) {
         const uint32_t group = fast_divide(block, parts_magic, parts_shift);
         const uint32_t part = block - group * parts;
         const uint32_t candidate = group * rows_per_block + wave_z;
@@ -805,9 +803,8 @@ __global__ void __launch_bounds__(1024) dispatch_rows_kernel(const u32x4* __rest
                 recv_weights[out_row * num_topk + lane] = weights[static_cast<int64_t>(token) * num_topk + lane];
         }
     } else {
-        const uint32_t pad_block = block - copy_blocks;
-        const uint32_t expert = pad_block / pad_groups_per_expert;
-        const uint32_t group = pad_block - expert * pad_groups_per_expert;
+        const uint32_t expert = block / pad_groups_per_expert;
+        const uint32_t group = block - expert * pad_groups_per_expert;
         const uint32_t waves = chunks_per_block * rows_per_block;
         const uint32_t j = group * waves + wave_z * chunks_per_block + wave_y;
         if (j >= pad_per_expert)
@@ -1280,16 +1277,17 @@ int nanoep_dispatch(const void* x, const float* weights, const int32_t* recv_met
     // No expert's gap exceeds alignment-1 rows, and all gaps together stay below C.
     const int64_t pad_per_expert = !pad ? 0 : (alignment - 1 < expanded_capacity ? alignment - 1 : expanded_capacity);
     const int64_t pad_groups_per_expert = (pad_per_expert + waves - 1) / waves;
-    const int64_t total_blocks = copy_blocks + num_local_experts * pad_groups_per_expert;
-    if (copy_candidates >= (int64_t{1} << 31) || total_blocks >= (int64_t{1} << 31) - kNumXcds)
+    const int64_t pad_blocks = num_local_experts * pad_groups_per_expert;
+    if (copy_candidates >= (int64_t{1} << 31) || copy_blocks + pad_blocks >= (int64_t{1} << 31) - 2 * kNumXcds)
         return NANOEP_ERR_INVALID_ARGUMENT;
-    const uint32_t blocks_per_xcd = static_cast<uint32_t>((total_blocks + kNumXcds - 1) / kNumXcds);
+    const uint32_t copy_per_xcd = static_cast<uint32_t>((copy_blocks + kNumXcds - 1) / kNumXcds);
+    const uint32_t pad_per_xcd = static_cast<uint32_t>((pad_blocks + kNumXcds - 1) / kNumXcds);
     int topk_shift = -1;
     if ((num_topk & (num_topk - 1)) == 0)
         for (topk_shift = 0; (1 << topk_shift) < num_topk; ++topk_shift) {
         }
 
-    const dim3 grid(blocks_per_xcd * kNumXcds);
+    const dim3 grid((copy_per_xcd + pad_per_xcd) * kNumXcds);
     const dim3 block(kWave, blocking.chunks_per_block, blocking.rows_per_block);
     const FastDivisor parts_divisor = make_fast_divisor(blocking.parts);
     auto stream = static_cast<hipStream_t>(stream_handle);
@@ -1299,8 +1297,8 @@ int nanoep_dispatch(const void* x, const float* weights, const int32_t* recv_met
         expert_counts,                                                                                               \
         expert_offsets, static_cast<u32x4*>(recv_x), recv_topk_idx, recv_weights, recv_count, out_rows,              \
         static_cast<uint32_t>(copy_candidates), static_cast<uint32_t>(num_tokens * num_topk),                        \
-        static_cast<uint32_t>(copy_blocks), static_cast<uint32_t>(total_blocks), blocks_per_xcd,                     \
-        static_cast<uint32_t>(total_blocks - copy_blocks), blocking.parts, parts_divisor.magic, parts_divisor.shift, blocking.chunks_per_block,         \
+        static_cast<uint32_t>(copy_blocks), copy_per_xcd, static_cast<uint32_t>(pad_blocks), pad_per_xcd,            \
+        blocking.parts, parts_divisor.magic, parts_divisor.shift, blocking.chunks_per_block,         \
         blocking.rows_per_block, static_cast<uint32_t>(pad_per_expert),                                              \
         static_cast<uint32_t>(pad_groups_per_expert > 0 ? pad_groups_per_expert : 1), vectors, chunks, num_topk,     \
         topk_shift, expand ? 1 : 0)
