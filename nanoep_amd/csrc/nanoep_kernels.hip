@@ -682,7 +682,7 @@ enum DispatchLookup {
     kLookupOrder = 2,     // candidate = entry of the slot-order list: (slot << 32) | (token * K + k), or -1
 };
 
-template <int kLookup>
+template <int kLookup, bool kZeroFill>
 __global__ void __launch_bounds__(1024) dispatch_rows_kernel(const u32x4* __restrict__ x,                // [T][vectors]
                                                              const float* __restrict__ weights,         // [T][K] or null
                                                              const int32_t* __restrict__ recv_metadata,  // [N][K+2]
@@ -733,11 +733,16 @@ __global__ void __launch_bounds__(1024) dispatch_rows_kernel(const u32x4* __rest
     // Workgroups are handed to the XCDs round-robin.  Each XCD takes one contiguous range of the
     // copy work followed by one contiguous range of the zero-fill work, so neighbouring work items
     // (which share their source rows) stay behind one L2 and every XCD gets its share of both.
+    // (kZeroFill is false when the launch has no zero-fill work: the copy path then carries none of
+    // its bookkeeping, which shows in a wavefront that lives about a microsecond)
     const uint32_t xcd = blockIdx.x % kNumXcds;
     const uint32_t index_in_xcd = blockIdx.x / kNumXcds;
-    const bool copy_work = index_in_xcd < copy_per_xcd;
-    const uint32_t block = copy_work ? xcd * copy_per_xcd + index_in_xcd : xcd * pad_per_xcd + (index_in_xcd - copy_per_xcd);
-    if (copy_work ? block >= copy_blocks : (index_in_xcd - copy_per_xcd >= pad_per_xcd || block >= pad_blocks))
+    const bool copy_work = !kZeroFill || index_in_xcd < copy_per_xcd;
+    uint32_t block = xcd * copy_per_xcd + index_in_xcd;
+    if (kZeroFill && !copy_work)
+        block = xcd * pad_per_xcd + (index_in_xcd - copy_per_xcd);
+    if (copy_work ? (index_in_xcd >= copy_per_xcd || block >= copy_blocks)
+                  : (index_in_xcd - copy_per_xcd >= pad_per_xcd || block >= pad_blocks))
         return;
     const int lane = threadIdx.x;
     const uint32_t wave_y = __builtin_amdgcn_readfirstlane(threadIdx.y);
@@ -819,6 +824,70 @@ __global__ void __launch_bounds__(1024) dispatch_rows_kernel(const u32x4* __rest
         if (lane == 0 && recv_weights != nullptr)
             recv_weights[out_row] = 0.0f;
     }
+}
+
+// The slot-order walk without zero-fill work, stripped to what its wavefronts need: a wavefront
+// lives about a microsecond, most of it waiting in a chain of scalar work -> list entry -> source
+// load -> store, so every scalar instruction and branch ahead of the source load is throughput.
+// Validity is folded into one flag and the load is issued unconditionally (row 0 stands in).
+template <bool kDeviceCount>
+__global__ void __launch_bounds__(1024) dispatch_ordered_kernel(const u32x4* __restrict__ x,              // [T][vectors]
+                                                                const float* __restrict__ weights,       // [T][K] or null
+                                                                const int64_t* __restrict__ slot_order,  // [entries]
+                                                                const int64_t* __restrict__ live_count,  // device entry count (kDeviceCount)
+                                                                u32x4* __restrict__ recv_x,              // [C][vectors]
+                                                                float* __restrict__ recv_weights,        // [C] or null
+                                                                uint32_t entries,
+                                                                uint32_t source_limit,  // T*K
+                                                                uint32_t out_rows,
+                                                                uint32_t copy_blocks,
+                                                                uint32_t copy_per_xcd,
+                                                                uint32_t parts,
+                                                                uint32_t parts_magic,
+                                                                uint32_t parts_shift,
+                                                                uint32_t chunks_per_block,  // == blockDim.y
+                                                                uint32_t rows_per_block,    // == blockDim.z
+                                                                uint32_t vectors,
+                                                                uint32_t chunks,
+                                                                uint32_t topk_magic,  // fast divisor by K
+                                                                uint32_t topk_shift) {
+    NANOEP_FETCH_ARGS_4(x, weights, recv_x, recv_weights);
+    NANOEP_FETCH_ARGS_4(slot_order, entries, source_limit, out_rows);
+    NANOEP_FETCH_ARGS_4(copy_blocks, copy_per_xcd, parts, parts_magic);
+    NANOEP_FETCH_ARGS_4(parts_shift, chunks_per_block, rows_per_block, vectors);
+    NANOEP_FETCH_ARGS_4(chunks, topk_magic, topk_shift, live_count);
+    if (kDeviceCount) {
+        const int64_t live = uniform_load(live_count);
+        if (live >= 0 && live < static_cast<int64_t>(entries)) {
+            entries = static_cast<uint32_t>(live);
+            copy_blocks = (rows_per_block == 1 ? entries : (entries + rows_per_block - 1) / rows_per_block) * parts;
+            copy_per_xcd = (copy_blocks + kNumXcds - 1) / kNumXcds;
+        }
+    }
+    const uint32_t index_in_xcd = blockIdx.x / kNumXcds;
+    const uint32_t block = (blockIdx.x % kNumXcds) * copy_per_xcd + index_in_xcd;
+    if (index_in_xcd >= copy_per_xcd || block >= copy_blocks)
+        return;
+    const uint32_t group = fast_divide(block, parts_magic, parts_shift);
+    const uint32_t part = block - group * parts;
+    const uint32_t candidate = group * rows_per_block + __builtin_amdgcn_readfirstlane(threadIdx.z);
+    const uint32_t chunk = part * chunks_per_block + __builtin_amdgcn_readfirstlane(threadIdx.y);
+    if (candidate >= entries || chunk >= chunks)
+        return;
+    const int64_t entry = uniform_load(slot_order + candidate);
+    const uint32_t source = static_cast<uint32_t>(entry);
+    const uint32_t out_row = static_cast<uint32_t>(static_cast<uint64_t>(entry) >> 32);
+    const bool valid = entry >= 0 && source < source_limit && out_row < out_rows;
+    const uint32_t token = valid ? fast_divide(source, topk_magic, topk_shift) : 0u;
+    const uint32_t vector = chunk * kWave + threadIdx.x;
+    const bool in_row = vector < vectors;
+    const u32x4 data = x[static_cast<uint64_t>(token) * vectors + (in_row ? vector : 0u)];
+    if (!valid)
+        return;
+    if (in_row)
+        store_vec<true>(recv_x + static_cast<uint64_t>(out_row) * vectors + vector, data);
+    if (chunk == 0 && threadIdx.x == 0 && recv_weights != nullptr)
+        recv_weights[out_row] = weights[source];
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -1291,8 +1360,15 @@ int nanoep_dispatch(const void* x, const float* weights, const int32_t* recv_met
     const dim3 block(kWave, blocking.chunks_per_block, blocking.rows_per_block);
     const FastDivisor parts_divisor = make_fast_divisor(blocking.parts);
     auto stream = static_cast<hipStream_t>(stream_handle);
-#define NANOEP_LAUNCH_DISPATCH(LOOKUP)                                                                               \
-    dispatch_rows_kernel<LOOKUP><<<grid, block, 0, stream>>>(                                                        \
+#define NANOEP_LAUNCH_DISPATCH(LOOKUP)                   \
+    do {                                                 \
+        if (pad_blocks > 0)                              \
+            NANOEP_LAUNCH_DISPATCH_AS(LOOKUP, true);     \
+        else                                             \
+            NANOEP_LAUNCH_DISPATCH_AS(LOOKUP, false);    \
+    } while (0)
+#define NANOEP_LAUNCH_DISPATCH_AS(LOOKUP, ZERO_FILL)                                                                 \
+    dispatch_rows_kernel<LOOKUP, ZERO_FILL><<<grid, block, 0, stream>>>(                                             \
         static_cast<const u32x4*>(x), weights, recv_metadata, dst_slots, token_slots, slot_order, live_count,        \
         expert_counts,                                                                                               \
         expert_offsets, static_cast<u32x4*>(recv_x), recv_topk_idx, recv_weights, recv_count, out_rows,              \
@@ -1302,13 +1378,28 @@ int nanoep_dispatch(const void* x, const float* weights, const int32_t* recv_met
         blocking.rows_per_block, static_cast<uint32_t>(pad_per_expert),                                              \
         static_cast<uint32_t>(pad_groups_per_expert > 0 ? pad_groups_per_expert : 1), vectors, chunks, num_topk,     \
         topk_shift, expand ? 1 : 0)
-    if (ordered)
+    if (ordered && pad_blocks == 0) {
+        const FastDivisor topk_divisor = make_fast_divisor(static_cast<uint32_t>(num_topk));
+#define NANOEP_LAUNCH_ORDERED(DEVICE_COUNT)                                                                           \
+    dispatch_ordered_kernel<DEVICE_COUNT><<<grid, block, 0, stream>>>(                                               \
+        static_cast<const u32x4*>(x), weights, slot_order, live_count, static_cast<u32x4*>(recv_x), recv_weights,    \
+        static_cast<uint32_t>(copy_candidates), static_cast<uint32_t>(num_tokens * num_topk),                        \
+        static_cast<uint32_t>(out_rows), static_cast<uint32_t>(copy_blocks), copy_per_xcd, blocking.parts,           \
+        parts_divisor.magic, parts_divisor.shift, blocking.chunks_per_block, blocking.rows_per_block,                \
+        static_cast<uint32_t>(vectors), static_cast<uint32_t>(chunks), topk_divisor.magic, topk_divisor.shift)
+        if (live_count != nullptr)
+            NANOEP_LAUNCH_ORDERED(true);
+        else
+            NANOEP_LAUNCH_ORDERED(false);
+#undef NANOEP_LAUNCH_ORDERED
+    } else if (ordered)
         NANOEP_LAUNCH_DISPATCH(kLookupOrder);
     else if (token_slots != nullptr && expand)
         NANOEP_LAUNCH_DISPATCH(kLookupTable);
     else
         NANOEP_LAUNCH_DISPATCH(kLookupMetadata);
 #undef NANOEP_LAUNCH_DISPATCH
+#undef NANOEP_LAUNCH_DISPATCH_AS
     NANOEP_HIP_TRY(hipGetLastError());
     return NANOEP_OK;
 }
