@@ -308,13 +308,13 @@ def main():
             "dispatch_bytes": d_bytes,
             "combine_bytes": c_bytes,
             "roofline": {
-                "kernel": "dispatch_rows_kernel",
+                "kernel": "dispatch_ordered_kernel",
                 "bound": "hbm",
                 "achieved": round(d_bytes / d_us / 1e3, 1),
                 "peak": HBM_PEAK_GBS,
                 "unit": "GB/s",
                 "frac": round(d_bytes / d_us / 1e3 / HBM_PEAK_GBS, 4),
-                "traffic": measured_traffic("dispatch_rows_kernel", workload.name),
+                "traffic": measured_traffic("dispatch_ordered_kernel", workload.name),
                 "algorithmic_bytes": d_bytes,
                 "avg_us": round(d_us, 2),
             },
