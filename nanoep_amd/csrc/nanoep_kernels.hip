@@ -16,9 +16,13 @@
 //                          workgroup 0 publishes N, C to the host mailbox.
 //   layout_scan_kernel + layout_assign_kernel : (many blocks) the same in two launches, with one
 //                          workgroup doing the scans: slot = offset[e] + block_base[b][e] + rank.
-//   dispatch_rows_kernel : one wavefront per (receive row, row chunk): 128-bit loads of the source
-//                          row held in registers, stored to every destination row; extra work items
-//                          zero-fill the alignment gaps.
+//   dispatch_ordered_kernel : expanded layouts with the layout's slot-order list: one wavefront per
+//                          (list entry, row chunk), token block by token block and expert-major
+//                          inside a block, so a block's source rows stay in one XCD's L2 and every
+//                          expert receives runs of consecutive rows; one 128-bit load and one
+//                          nontemporal 128-bit store per lane.
+//   dispatch_rows_kernel : the same work item walked in source-token order (compact layouts, handles
+//                          without the list); extra work items zero-fill the alignment gaps.
 //   combine_rows_kernel  : one wavefront per (source token, row chunk): gathers the token's rows in
 //                          ascending k, fp32 accumulate, one round-to-nearest-even bf16 store.
 //
@@ -673,14 +677,47 @@ __device__ __forceinline__ uint32_t fast_divide(uint32_t n, uint32_t magic, uint
 // (token_slots[t][k], or dst_slots[t] -> recv_metadata[row][2+k] for a handle without that table)
 // resolve the destination row.
 //
-// Workgroups past copy_blocks zero-fill the alignment gaps: workgroup (e, g) owns gap candidates
+// Zero-fill workgroups clear the alignment gaps: workgroup (e, g) owns gap candidates
 // j = g * waves .. of expert e, row offsets[e] + counts[e] + j while that is below offsets[e+1].
-// How a dispatch wavefront finds its (source token, k, destination row).
+// Every XCD takes one contiguous range of the copy work followed by one contiguous range of the
+// zero-fill work, so it gets its share of both.
+
+// How a token-order dispatch wavefront finds its destination row.
 enum DispatchLookup {
-    kLookupMetadata = 0,  // candidate = (token, k) in token order; dst_slots -> recv_metadata row -> field k
-    kLookupTable = 1,     // candidate = (token, k) in token order; token_slots[token][k]
-    kLookupOrder = 2,     // candidate = entry of the slot-order list: (slot << 32) | (token * K + k), or -1
+    kLookupMetadata = 0,  // dst_slots -> recv_metadata row -> field k
+    kLookupTable = 1,     // token_slots[token][k]
 };
+
+// One zero-fill workgroup: each wavefront clears one whole gap row (and its weight).
+__device__ __forceinline__ void zero_fill_gap_rows(uint32_t block,
+                                                   uint32_t pad_per_expert,
+                                                   uint32_t pad_groups_per_expert,
+                                                   uint32_t chunks_per_block,
+                                                   uint32_t rows_per_block,
+                                                   const int64_t* __restrict__ expert_counts,
+                                                   const int64_t* __restrict__ expert_offsets,
+                                                   u32x4* __restrict__ recv_x,
+                                                   float* __restrict__ recv_weights,
+                                                   int64_t out_rows,
+                                                   int vectors) {
+    const uint32_t wave_y = __builtin_amdgcn_readfirstlane(threadIdx.y);
+    const uint32_t wave_z = __builtin_amdgcn_readfirstlane(threadIdx.z);
+    const uint32_t expert = block / pad_groups_per_expert;
+    const uint32_t group = block - expert * pad_groups_per_expert;
+    const uint32_t waves = chunks_per_block * rows_per_block;
+    const uint32_t j = group * waves + wave_z * chunks_per_block + wave_y;
+    if (j >= pad_per_expert)
+        return;
+    const int64_t out_row = uniform_load(expert_offsets + expert) + uniform_load(expert_counts + expert) + j;
+    if (out_row >= uniform_load(expert_offsets + expert + 1) || out_row >= out_rows)
+        return;
+    const u32x4 zero = {0u, 0u, 0u, 0u};
+    u32x4* dst = recv_x + out_row * vectors;
+    for (int vector = threadIdx.x; vector < vectors; vector += kWave)
+        store_vec<true>(dst + vector, zero);
+    if (threadIdx.x == 0 && recv_weights != nullptr)
+        recv_weights[out_row] = 0.0f;
+}
 
 template <int kLookup, bool kZeroFill>
 __global__ void __launch_bounds__(1024) dispatch_rows_kernel(const u32x4* __restrict__ x,                // [T][vectors]
@@ -688,8 +725,6 @@ __global__ void __launch_bounds__(1024) dispatch_rows_kernel(const u32x4* __rest
                                                              const int32_t* __restrict__ recv_metadata,  // [N][K+2]
                                                              const int64_t* __restrict__ dst_slots,     // [T]
                                                              const int32_t* __restrict__ token_slots,   // [T][K] or null
-                                                             const int64_t* __restrict__ slot_order,    // [copy_candidates] or null
-                                                             const int64_t* __restrict__ live_count,    // device count of list entries, or null
                                                              const int64_t* __restrict__ expert_counts,
                                                              const int64_t* __restrict__ expert_offsets,
                                                              u32x4* __restrict__ recv_x,                // [C or N][vectors]
@@ -697,8 +732,7 @@ __global__ void __launch_bounds__(1024) dispatch_rows_kernel(const u32x4* __rest
                                                              float* __restrict__ recv_weights,          // [C] / [N][K] or null
                                                              int64_t recv_count,
                                                              int64_t out_rows,
-                                                             uint32_t copy_candidates,  // T*K expanded, T compact, list entries when ordered
-                                                             uint32_t source_limit,     // T*K
+                                                             uint32_t copy_candidates,  // T*K expanded, T compact
                                                              uint32_t copy_blocks,
                                                              uint32_t copy_per_xcd,  // ceil(copy_blocks / 8)
                                                              uint32_t pad_blocks,
@@ -716,20 +750,10 @@ __global__ void __launch_bounds__(1024) dispatch_rows_kernel(const u32x4* __rest
                                                              int topk_shift,  // log2(K) when K is a power of two, else -1
                                                              int expand) {
     NANOEP_FETCH_ARGS_4(x, weights, recv_x, recv_weights);
-    NANOEP_FETCH_ARGS_4(token_slots, slot_order, dst_slots, recv_metadata);
-    NANOEP_FETCH_ARGS_4(out_rows, recv_count, copy_candidates, source_limit);
+    NANOEP_FETCH_ARGS_4(token_slots, copy_blocks, dst_slots, recv_metadata);
+    NANOEP_FETCH_ARGS_4(out_rows, recv_count, copy_candidates, copy_per_xcd);
     NANOEP_FETCH_ARGS_4(parts_magic, parts_shift, vectors, chunks);
     NANOEP_FETCH_ARGS_4(num_topk, topk_shift, expand, chunks_per_block);
-    if (kLookup == kLookupOrder && live_count != nullptr) {
-        // The list length was not known when the grid was sized: shrink the walk to the entries in
-        // use, so that the per-XCD ranges split the real work and not its unused tail.
-        const int64_t live = uniform_load(live_count);
-        if (live >= 0 && live < static_cast<int64_t>(copy_candidates)) {
-            copy_candidates = static_cast<uint32_t>(live);
-            copy_blocks = (rows_per_block == 1 ? copy_candidates : (copy_candidates + rows_per_block - 1) / rows_per_block) * parts;
-            copy_per_xcd = (copy_blocks + kNumXcds - 1) / kNumXcds;
-        }
-    }
     // Workgroups are handed to the XCDs round-robin.  Each XCD takes one contiguous range of the
     // copy work followed by one contiguous range of the zero-fill work, so neighbouring work items
     // (which share their source rows) stay behind one L2 and every XCD gets its share of both.
@@ -761,36 +785,22 @@ __global__ void __launch_bounds__(1024) dispatch_rows_kernel(const u32x4* __rest
         int k = 0;
         int64_t out_row;
         const int32_t* fields = nullptr;
-        u32x4 data;
-        if (kLookup == kLookupOrder) {
-            const int64_t entry = uniform_load(slot_order + candidate);
-            if (entry < 0)
-                return;
-            const uint32_t source = static_cast<uint32_t>(entry);
-            if (source >= source_limit)
-                return;
-            out_row = entry >> 32;
-            token = topk_shift >= 0 ? source >> topk_shift : source / static_cast<uint32_t>(num_topk);
-            k = static_cast<int>(source - token * num_topk);
-            data = x[static_cast<int64_t>(token) * vectors + (in_row ? vector : 0)];
+        if (expand) {
+            token = topk_shift >= 0 ? candidate >> topk_shift : candidate / static_cast<uint32_t>(num_topk);
+            k = static_cast<int>(candidate - token * num_topk);
+        }
+        token = __builtin_amdgcn_readfirstlane(token);
+        k = __builtin_amdgcn_readfirstlane(k);
+        // lanes past the end of a short row re-read vector 0 instead of branching around the load
+        const u32x4 data = x[static_cast<int64_t>(token) * vectors + (in_row ? vector : 0)];
+        if (kLookup == kLookupTable && expand) {
+            out_row = uniform_load(token_slots + static_cast<int64_t>(token) * num_topk + k);
         } else {
-            if (expand) {
-                token = topk_shift >= 0 ? candidate >> topk_shift : candidate / static_cast<uint32_t>(num_topk);
-                k = static_cast<int>(candidate - token * num_topk);
-            }
-            token = __builtin_amdgcn_readfirstlane(token);
-            k = __builtin_amdgcn_readfirstlane(k);
-            // lanes past the end of a short row re-read vector 0 instead of branching around the load
-            data = x[static_cast<int64_t>(token) * vectors + (in_row ? vector : 0)];
-            if (kLookup == kLookupTable && expand) {
-                out_row = uniform_load(token_slots + static_cast<int64_t>(token) * num_topk + k);
-            } else {
-                const int64_t row = uniform_load(dst_slots + token);
-                if (row < 0 || row >= recv_count)
-                    return;
-                fields = recv_metadata + row * (num_topk + 2);
-                out_row = expand ? static_cast<int64_t>(uniform_load(fields + 2 + k)) : row;
-            }
+            const int64_t row = uniform_load(dst_slots + token);
+            if (row < 0 || row >= recv_count)
+                return;
+            fields = recv_metadata + row * (num_topk + 2);
+            out_row = expand ? static_cast<int64_t>(uniform_load(fields + 2 + k)) : row;
         }
         if (out_row < 0 || out_row >= out_rows)
             return;
@@ -808,40 +818,34 @@ __global__ void __launch_bounds__(1024) dispatch_rows_kernel(const u32x4* __rest
                 recv_weights[out_row * num_topk + lane] = weights[static_cast<int64_t>(token) * num_topk + lane];
         }
     } else {
-        const uint32_t expert = block / pad_groups_per_expert;
-        const uint32_t group = block - expert * pad_groups_per_expert;
-        const uint32_t waves = chunks_per_block * rows_per_block;
-        const uint32_t j = group * waves + wave_z * chunks_per_block + wave_y;
-        if (j >= pad_per_expert)
-            return;
-        const int64_t out_row = uniform_load(expert_offsets + expert) + uniform_load(expert_counts + expert) + j;
-        if (out_row >= uniform_load(expert_offsets + expert + 1) || out_row >= out_rows)
-            return;
-        const u32x4 zero = {0u, 0u, 0u, 0u};
-        u32x4* dst = recv_x + out_row * vectors;
-        for (int vector = lane; vector < vectors; vector += kWave)
-            store_vec<true>(dst + vector, zero);
-        if (lane == 0 && recv_weights != nullptr)
-            recv_weights[out_row] = 0.0f;
+        zero_fill_gap_rows(block, pad_per_expert, pad_groups_per_expert, chunks_per_block, rows_per_block, expert_counts,
+                           expert_offsets, recv_x, recv_weights, out_rows, vectors);
     }
 }
 
-// The slot-order walk without zero-fill work, stripped to what its wavefronts need: a wavefront
-// lives about a microsecond, most of it waiting in a chain of scalar work -> list entry -> source
-// load -> store, so every scalar instruction and branch ahead of the source load is throughput.
-// Validity is folded into one flag and the load is issued unconditionally (row 0 stands in).
-template <bool kDeviceCount>
+// The slot-order walk, stripped to what its wavefronts need: a wavefront lives about a microsecond,
+// most of it waiting in a chain of scalar work -> list entry -> source load -> store, so every
+// scalar instruction and branch ahead of the source load is throughput.  Validity is folded into
+// one flag and the load is issued unconditionally (row 0 stands in).  kZeroFill is false when the
+// launch has no gap rows to clear: the copy path then carries none of that bookkeeping.
+template <bool kDeviceCount, bool kZeroFill>
 __global__ void __launch_bounds__(1024) dispatch_ordered_kernel(const u32x4* __restrict__ x,              // [T][vectors]
                                                                 const float* __restrict__ weights,       // [T][K] or null
                                                                 const int64_t* __restrict__ slot_order,  // [entries]
                                                                 const int64_t* __restrict__ live_count,  // device entry count (kDeviceCount)
-                                                                u32x4* __restrict__ recv_x,              // [C][vectors]
-                                                                float* __restrict__ recv_weights,        // [C] or null
+                                                                const int64_t* __restrict__ expert_counts,
+                                                                const int64_t* __restrict__ expert_offsets,
+                                                                u32x4* __restrict__ recv_x,        // [C][vectors]
+                                                                float* __restrict__ recv_weights,  // [C] or null
                                                                 uint32_t entries,
                                                                 uint32_t source_limit,  // T*K
                                                                 uint32_t out_rows,
                                                                 uint32_t copy_blocks,
                                                                 uint32_t copy_per_xcd,
+                                                                uint32_t pad_blocks,
+                                                                uint32_t pad_per_xcd,
+                                                                uint32_t pad_per_expert,
+                                                                uint32_t pad_groups_per_expert,
                                                                 uint32_t parts,
                                                                 uint32_t parts_magic,
                                                                 uint32_t parts_shift,
@@ -857,6 +861,8 @@ __global__ void __launch_bounds__(1024) dispatch_ordered_kernel(const u32x4* __r
     NANOEP_FETCH_ARGS_4(parts_shift, chunks_per_block, rows_per_block, vectors);
     NANOEP_FETCH_ARGS_4(chunks, topk_magic, topk_shift, live_count);
     if (kDeviceCount) {
+        // The list length was not known when the grid was sized: shrink the walk to the entries in
+        // use, so that the per-XCD ranges split the real work and not its unused tail.
         const int64_t live = uniform_load(live_count);
         if (live >= 0 && live < static_cast<int64_t>(entries)) {
             entries = static_cast<uint32_t>(live);
@@ -865,6 +871,14 @@ __global__ void __launch_bounds__(1024) dispatch_ordered_kernel(const u32x4* __r
         }
     }
     const uint32_t index_in_xcd = blockIdx.x / kNumXcds;
+    if (kZeroFill && index_in_xcd >= copy_per_xcd) {
+        const uint32_t pad_index = index_in_xcd - copy_per_xcd;
+        const uint32_t pad_block = (blockIdx.x % kNumXcds) * pad_per_xcd + pad_index;
+        if (pad_index < pad_per_xcd && pad_block < pad_blocks)
+            zero_fill_gap_rows(pad_block, pad_per_expert, pad_groups_per_expert, chunks_per_block, rows_per_block,
+                               expert_counts, expert_offsets, recv_x, recv_weights, out_rows, static_cast<int>(vectors));
+        return;
+    }
     const uint32_t block = (blockIdx.x % kNumXcds) * copy_per_xcd + index_in_xcd;
     if (index_in_xcd >= copy_per_xcd || block >= copy_blocks)
         return;
@@ -1360,46 +1374,48 @@ int nanoep_dispatch(const void* x, const float* weights, const int32_t* recv_met
     const dim3 block(kWave, blocking.chunks_per_block, blocking.rows_per_block);
     const FastDivisor parts_divisor = make_fast_divisor(blocking.parts);
     auto stream = static_cast<hipStream_t>(stream_handle);
-#define NANOEP_LAUNCH_DISPATCH(LOOKUP)                   \
-    do {                                                 \
-        if (pad_blocks > 0)                              \
-            NANOEP_LAUNCH_DISPATCH_AS(LOOKUP, true);     \
-        else                                             \
-            NANOEP_LAUNCH_DISPATCH_AS(LOOKUP, false);    \
-    } while (0)
-#define NANOEP_LAUNCH_DISPATCH_AS(LOOKUP, ZERO_FILL)                                                                 \
-    dispatch_rows_kernel<LOOKUP, ZERO_FILL><<<grid, block, 0, stream>>>(                                             \
-        static_cast<const u32x4*>(x), weights, recv_metadata, dst_slots, token_slots, slot_order, live_count,        \
-        expert_counts,                                                                                               \
-        expert_offsets, static_cast<u32x4*>(recv_x), recv_topk_idx, recv_weights, recv_count, out_rows,              \
-        static_cast<uint32_t>(copy_candidates), static_cast<uint32_t>(num_tokens * num_topk),                        \
-        static_cast<uint32_t>(copy_blocks), copy_per_xcd, static_cast<uint32_t>(pad_blocks), pad_per_xcd,            \
-        blocking.parts, parts_divisor.magic, parts_divisor.shift, blocking.chunks_per_block,         \
-        blocking.rows_per_block, static_cast<uint32_t>(pad_per_expert),                                              \
-        static_cast<uint32_t>(pad_groups_per_expert > 0 ? pad_groups_per_expert : 1), vectors, chunks, num_topk,     \
-        topk_shift, expand ? 1 : 0)
-    if (ordered && pad_blocks == 0) {
+    if (ordered) {
         const FastDivisor topk_divisor = make_fast_divisor(static_cast<uint32_t>(num_topk));
-#define NANOEP_LAUNCH_ORDERED(DEVICE_COUNT)                                                                           \
-    dispatch_ordered_kernel<DEVICE_COUNT><<<grid, block, 0, stream>>>(                                               \
-        static_cast<const u32x4*>(x), weights, slot_order, live_count, static_cast<u32x4*>(recv_x), recv_weights,    \
-        static_cast<uint32_t>(copy_candidates), static_cast<uint32_t>(num_tokens * num_topk),                        \
-        static_cast<uint32_t>(out_rows), static_cast<uint32_t>(copy_blocks), copy_per_xcd, blocking.parts,           \
+#define NANOEP_LAUNCH_ORDERED(DEVICE_COUNT, ZERO_FILL)                                                                \
+    dispatch_ordered_kernel<DEVICE_COUNT, ZERO_FILL><<<grid, block, 0, stream>>>(                                    \
+        static_cast<const u32x4*>(x), weights, slot_order, live_count, expert_counts, expert_offsets,                \
+        static_cast<u32x4*>(recv_x), recv_weights, static_cast<uint32_t>(copy_candidates),                           \
+        static_cast<uint32_t>(num_tokens * num_topk), static_cast<uint32_t>(out_rows),                               \
+        static_cast<uint32_t>(copy_blocks), copy_per_xcd, static_cast<uint32_t>(pad_blocks), pad_per_xcd,            \
+        static_cast<uint32_t>(pad_per_expert),                                                                       \
+        static_cast<uint32_t>(pad_groups_per_expert > 0 ? pad_groups_per_expert : 1), blocking.parts,                \
         parts_divisor.magic, parts_divisor.shift, blocking.chunks_per_block, blocking.rows_per_block,                \
         static_cast<uint32_t>(vectors), static_cast<uint32_t>(chunks), topk_divisor.magic, topk_divisor.shift)
-        if (live_count != nullptr)
-            NANOEP_LAUNCH_ORDERED(true);
+        if (live_count != nullptr && pad_blocks > 0)
+            NANOEP_LAUNCH_ORDERED(true, true);
+        else if (live_count != nullptr)
+            NANOEP_LAUNCH_ORDERED(true, false);
+        else if (pad_blocks > 0)
+            NANOEP_LAUNCH_ORDERED(false, true);
         else
-            NANOEP_LAUNCH_ORDERED(false);
+            NANOEP_LAUNCH_ORDERED(false, false);
 #undef NANOEP_LAUNCH_ORDERED
-    } else if (ordered)
-        NANOEP_LAUNCH_DISPATCH(kLookupOrder);
-    else if (token_slots != nullptr && expand)
-        NANOEP_LAUNCH_DISPATCH(kLookupTable);
-    else
-        NANOEP_LAUNCH_DISPATCH(kLookupMetadata);
-#undef NANOEP_LAUNCH_DISPATCH
-#undef NANOEP_LAUNCH_DISPATCH_AS
+    } else {
+#define NANOEP_LAUNCH_ROWS(LOOKUP, ZERO_FILL)                                                                         \
+    dispatch_rows_kernel<LOOKUP, ZERO_FILL><<<grid, block, 0, stream>>>(                                             \
+        static_cast<const u32x4*>(x), weights, recv_metadata, dst_slots, token_slots, expert_counts, expert_offsets, \
+        static_cast<u32x4*>(recv_x), recv_topk_idx, recv_weights, recv_count, out_rows,                              \
+        static_cast<uint32_t>(copy_candidates), static_cast<uint32_t>(copy_blocks), copy_per_xcd,                    \
+        static_cast<uint32_t>(pad_blocks), pad_per_xcd, blocking.parts, parts_divisor.magic, parts_divisor.shift,    \
+        blocking.chunks_per_block, blocking.rows_per_block, static_cast<uint32_t>(pad_per_expert),                   \
+        static_cast<uint32_t>(pad_groups_per_expert > 0 ? pad_groups_per_expert : 1), vectors, chunks, num_topk,     \
+        topk_shift, expand ? 1 : 0)
+        const bool table = token_slots != nullptr && expand;
+        if (table && pad_blocks > 0)
+            NANOEP_LAUNCH_ROWS(kLookupTable, true);
+        else if (table)
+            NANOEP_LAUNCH_ROWS(kLookupTable, false);
+        else if (pad_blocks > 0)
+            NANOEP_LAUNCH_ROWS(kLookupMetadata, true);
+        else
+            NANOEP_LAUNCH_ROWS(kLookupMetadata, false);
+#undef NANOEP_LAUNCH_ROWS
+    }
     NANOEP_HIP_TRY(hipGetLastError());
     return NANOEP_OK;
 }
