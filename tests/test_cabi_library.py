@@ -2,6 +2,8 @@
 or argument-checking entry points behave (no compute call is made here)."""
 
 import ctypes
+import shutil
+import subprocess
 
 import pytest
 
@@ -71,3 +73,20 @@ def test_argument_checks_come_before_any_device_work():
     assert library.nanoep_layout_block_tokens(6000) == 0 and library.nanoep_layout_block_tokens(0) == 0
     out = (ctypes.c_int64 * 4)()
     assert library.nanoep_wait_counts(null, null, 0.0, out) == 1
+
+
+@pytest.mark.skipif(shutil.which("gcc") is None, reason="no C compiler")
+def test_plain_c_client_compiles_links_and_runs(tmp_path):
+    """The header is C99 and the library links from C without HIP or torch on the include path."""
+    binary = tmp_path / "cabi_c_client"
+    source = cabi.ROOT / "tests" / "cabi_c_client.c"
+    library_dir = cabi.LIBRARY.parent
+    subprocess.run(
+        ["gcc", "-std=c99", "-Wall", "-Wextra", "-Werror", "-pedantic", f"-I{cabi.HEADER.parent}", str(source), "-o", str(binary),
+         f"-L{library_dir}", "-lnanoep_hip", f"-Wl,-rpath,{library_dir}"],
+        check=True, capture_output=True, text=True,
+    )
+    out = subprocess.run([str(binary)], check=True, capture_output=True, text=True, timeout=60).stdout.splitlines()
+    assert out[0] == "abi 2 status 0 window 0 96 160 160 9888"
+    assert out[1].startswith("invalid 1 '") and "invalid" in out[1].lower()
+    assert out[2] == "sizes 32769 256 1"
