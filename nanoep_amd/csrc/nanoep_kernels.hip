@@ -139,17 +139,17 @@ constexpr int kRankMask = (1 << kRankBits) - 1;
 // The token's routing ids are fetched in one batch of independent loads (kCap >= K of them, the
 // surplus re-reads id 0) and stay in registers for both passes over the bit matrix.
 template <int kCap>
-__global__ void __launch_bounds__(256) layout_count_kernel(const int64_t* __restrict__ topk_idx,
-                                                           int64_t num_tokens,
-                                                           int num_topk,
-                                                           int local_experts,
-                                                           int words,
-                                                           int threads,
-                                                           int64_t* __restrict__ snapshot,
-                                                           int32_t* __restrict__ block_counts,
-                                                           int32_t* __restrict__ block_status,
-                                                           int32_t* __restrict__ packed_rank,
-                                                           int32_t* __restrict__ local_row) {
+__device__ __forceinline__ void layout_count_block(const int64_t* __restrict__ topk_idx,
+                                                   int64_t num_tokens,
+                                                   int num_topk,
+                                                   int local_experts,
+                                                   int words,
+                                                   int threads,
+                                                   int64_t* __restrict__ snapshot,
+                                                   int32_t* block_counts,
+                                                   int32_t* block_status,
+                                                   int32_t* packed_rank,
+                                                   int32_t* local_row) {
     extern __shared__ uint32_t layout_lds[];
     const int rows = local_experts + 1;
     // bit rows are words + 1 apart: an odd stride spreads the experts a wavefront touches over the LDS banks
@@ -237,6 +237,22 @@ __global__ void __launch_bounds__(256) layout_count_kernel(const int64_t* __rest
         const uint32_t received = bits[static_cast<size_t>(local_experts) * stride + word];
         local_row[token] = (received & bit) ? prefix[static_cast<size_t>(local_experts) * words + word] + __popc(received & below) : -1;
     }
+}
+
+template <int kCap>
+__global__ void __launch_bounds__(256) layout_count_kernel(const int64_t* __restrict__ topk_idx,
+                                                           int64_t num_tokens,
+                                                           int num_topk,
+                                                           int local_experts,
+                                                           int words,
+                                                           int threads,
+                                                           int64_t* __restrict__ snapshot,
+                                                           int32_t* __restrict__ block_counts,
+                                                           int32_t* __restrict__ block_status,
+                                                           int32_t* __restrict__ packed_rank,
+                                                           int32_t* __restrict__ local_row) {
+    layout_count_block<kCap>(topk_idx, num_tokens, num_topk, local_experts, words, threads, snapshot, block_counts,
+                             block_status, packed_rank, local_row);
 }
 
 __device__ __forceinline__ int64_t round_up_to(int64_t value, int64_t alignment) {
@@ -423,28 +439,28 @@ __device__ __forceinline__ int64_t wave_inclusive_scan(int64_t value) {
 // assignment of the block in expert-major order inside the block's run of `slot_order`; the runs
 // of consecutive blocks follow each other without gaps and the unused tail of the list is -1.
 template <int kCap, bool kFusedScan>
-__global__ void __launch_bounds__(256) layout_assign_kernel(const int32_t* __restrict__ block_counts,
-                                                            const int32_t* __restrict__ block_status,
-                                                            int num_blocks,
-                                                            int64_t num_tokens,
-                                                            int num_topk,
-                                                            int local_experts,
-                                                            int tokens_per_block,
-                                                            int threads,
-                                                            int expand,
-                                                            int64_t alignment,
-                                                            const int32_t* __restrict__ packed_rank,
-                                                            const int32_t* __restrict__ local_row,
-                                                            int64_t* expert_counts,
-                                                            int64_t* expert_offsets,
-                                                            int64_t* send_counts,
-                                                            int64_t* __restrict__ recv_rank_prefix,
-                                                            const int64_t* __restrict__ totals,
-                                                            int64_t* host_counts,
-                                                            int32_t* __restrict__ recv_metadata,
-                                                            int64_t* __restrict__ dst_slots,
-                                                            int32_t* __restrict__ token_slots,
-                                                            int64_t* __restrict__ slot_order) {
+__device__ __forceinline__ void layout_assign_block(const int32_t* block_counts,
+                                                    const int32_t* block_status,
+                                                    int num_blocks,
+                                                    int64_t num_tokens,
+                                                    int num_topk,
+                                                    int local_experts,
+                                                    int tokens_per_block,
+                                                    int threads,
+                                                    int expand,
+                                                    int64_t alignment,
+                                                    const int32_t* packed_rank,
+                                                    const int32_t* local_row,
+                                                    int64_t* expert_counts,
+                                                    int64_t* expert_offsets,
+                                                    int64_t* send_counts,
+                                                    int64_t* __restrict__ recv_rank_prefix,
+                                                    const int64_t* totals,
+                                                    int64_t* host_counts,
+                                                    int32_t* __restrict__ recv_metadata,
+                                                    int64_t* __restrict__ dst_slots,
+                                                    int32_t* __restrict__ token_slots,
+                                                    int64_t* __restrict__ slot_order) {
     extern __shared__ int32_t assign_lds[];
     __shared__ int64_t wave_padded[kWavesPerBlock];
     __shared__ int64_t wave_assigned[kWavesPerBlock];
@@ -606,6 +622,69 @@ __global__ void __launch_bounds__(256) layout_assign_kernel(const int32_t* __res
     if (live)
         assign_token_slots<kCap>(token, num_topk, expand, row_in_block, slot_base[local_experts], slot_base, order_base,
                                  packed_rank, recv_metadata, dst_slots, token_slots, order);
+}
+
+template <int kCap, bool kFusedScan>
+__global__ void __launch_bounds__(256) layout_assign_kernel(const int32_t* __restrict__ block_counts,
+                                                            const int32_t* __restrict__ block_status,
+                                                            int num_blocks,
+                                                            int64_t num_tokens,
+                                                            int num_topk,
+                                                            int local_experts,
+                                                            int tokens_per_block,
+                                                            int threads,
+                                                            int expand,
+                                                            int64_t alignment,
+                                                            const int32_t* __restrict__ packed_rank,
+                                                            const int32_t* __restrict__ local_row,
+                                                            int64_t* expert_counts,
+                                                            int64_t* expert_offsets,
+                                                            int64_t* send_counts,
+                                                            int64_t* recv_rank_prefix,
+                                                            const int64_t* __restrict__ totals,
+                                                            int64_t* host_counts,
+                                                            int32_t* recv_metadata,
+                                                            int64_t* dst_slots,
+                                                            int32_t* token_slots,
+                                                            int64_t* slot_order) {
+    layout_assign_block<kCap, kFusedScan>(block_counts, block_status, num_blocks, num_tokens, num_topk, local_experts,
+                                          tokens_per_block, threads, expand, alignment, packed_rank, local_row, expert_counts,
+                                          expert_offsets, send_counts, recv_rank_prefix, totals, host_counts, recv_metadata,
+                                          dst_slots, token_slots, slot_order);
+}
+
+// Whole layout in one launch when all tokens fit one block: the count pass, then (its results are
+// this workgroup's own global writes, made visible by the fence and the barrier) the assignment pass.
+template <int kCap>
+__global__ void __launch_bounds__(256) layout_single_block_kernel(const int64_t* topk_idx,
+                                                                  int64_t num_tokens,
+                                                                  int num_topk,
+                                                                  int local_experts,
+                                                                  int words,
+                                                                  int threads,
+                                                                  int expand,
+                                                                  int64_t alignment,
+                                                                  int64_t* snapshot,
+                                                                  int32_t* block_counts,
+                                                                  int32_t* block_status,
+                                                                  int32_t* packed_rank,
+                                                                  int32_t* local_row,
+                                                                  int64_t* expert_counts,
+                                                                  int64_t* expert_offsets,
+                                                                  int64_t* send_counts,
+                                                                  int64_t* recv_rank_prefix,
+                                                                  int64_t* host_counts,
+                                                                  int32_t* recv_metadata,
+                                                                  int64_t* dst_slots,
+                                                                  int32_t* token_slots,
+                                                                  int64_t* slot_order) {
+    layout_count_block<kCap>(topk_idx, num_tokens, num_topk, local_experts, words, threads, snapshot, block_counts,
+                             block_status, packed_rank, local_row);
+    __threadfence();
+    __syncthreads();
+    layout_assign_block<kCap, true>(block_counts, block_status, 1, num_tokens, num_topk, local_experts, words * 32, threads,
+                                    expand, alignment, packed_rank, local_row, expert_counts, expert_offsets, send_counts,
+                                    recv_rank_prefix, nullptr, host_counts, recv_metadata, dst_slots, token_slots, slot_order);
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -1242,6 +1321,16 @@ int nanoep_layout(const int64_t* topk_idx, int64_t num_tokens, int num_topk, int
     hipError_t launch_status = hipSuccess;
     with_topk_cap(num_topk, [&](auto cap) {
         constexpr int kCap = decltype(cap)::value;
+        if (blocks == 1 && forced_launches == 0) {
+            const size_t count_lds = static_cast<size_t>(experts + 1) * (words * 6 + 4);
+            const size_t assign_lds = static_cast<size_t>(experts + 1) * 12;
+            layout_single_block_kernel<kCap><<<1, count_threads, count_lds > assign_lds ? count_lds : assign_lds, stream>>>(
+                topk_idx, num_tokens, num_topk, experts, words, count_threads, expand, alignment, topk_snapshot,
+                ws.block_counts, ws.block_status, ws.packed_rank, ws.local_row, expert_counts, expert_offsets, send_counts,
+                recv_rank_prefix, host_counts, recv_metadata, dst_slots, token_slots, slot_order);
+            launch_status = hipGetLastError();
+            return;
+        }
         if (blocks > 0) {
             const size_t lds = static_cast<size_t>(experts + 1) * (words * 6 + 4);
             layout_count_kernel<kCap><<<blocks, count_threads, lds, stream>>>(
