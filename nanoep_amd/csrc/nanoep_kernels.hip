@@ -11,10 +11,11 @@
 //   layout_count_kernel  : one workgroup per block of tokens; LDS bit matrix (expert x token) built
 //                          with LDS atomics, popcount prefixes give the in-block stable rank of
 //                          every (token,k) and the block's per-expert histogram.
-//   layout_scan_assign_kernel : (few blocks) every workgroup sums the block histograms into LDS,
-//                          scans the aligned expert totals and writes its tokens' part of the handle;
-//                          workgroup 0 publishes N, C to the host mailbox.
-//   layout_scan_kernel + layout_assign_kernel : (many blocks) the same in two launches, with one
+//   layout_assign_kernel<fused scan> : (few blocks) every workgroup sums the block histograms into
+//                          LDS, scans the aligned expert totals and writes its tokens' part of the
+//                          handle and of the slot-order list; workgroup 0 publishes N, C to the host.
+//   layout_single_block_kernel : (one block) count and assignment passes in a single launch.
+//   layout_scan_kernel + layout_assign_kernel<no scan> : (many blocks) the same in two launches, one
 //                          workgroup doing the scans: slot = offset[e] + block_base[b][e] + rank.
 //   dispatch_ordered_kernel : expanded layouts with the layout's slot-order list: one wavefront per
 //                          (list entry, row chunk), token block by token block and expert-major
