@@ -32,6 +32,8 @@ WORKLOADS = {
                         "4096 x 4096, 8 experts top-2 uniform distinct ids, expanded"),
     "deepseek-v3": Workload("deepseek-v3", 4096, 7168, 256, 8, "softmax-topk-dropout", True, 1, True,
                             "4096 x 7168, 256 experts top-8 of softmax(N(0,1)), 10% of choices masked, expanded + zero_padding"),
+    "deepseek-v3-a128": Workload("deepseek-v3-a128", 4096, 7168, 256, 8, "softmax-topk-dropout", True, 128, True,
+                                 "the deepseek-v3 batch with expert segments padded to multiples of 128 rows"),
     "ep8-share": Workload("ep8-share", 32768, 7168, 32, 8, "zipf", False, 1, False,
                           "32768 x 7168 (8 source segments x 4096), 32 local experts top-8 Zipf(1.2), compact, cached handle"),
     "qwen3-moe": Workload("qwen3-moe", 8192, 2048, 128, 8, "biased-topk", True, 128, True,
