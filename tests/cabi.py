@@ -4,6 +4,7 @@ every compute call goes through the C ABI of nanoep_amd/libnanoep_hip.so."""
 from __future__ import annotations
 
 import ctypes
+import os
 import re
 from pathlib import Path
 
@@ -128,8 +129,13 @@ def slot_order_of(metadata, use_order=True):
 
 
 def dispatch(x, weights, metadata, counts, num_local_experts, alignment, expand, zero_padding, *, num_cus=0, poison=None,
-             use_table=True, use_order=True, order_count="exact"):
-    """Returns (recv_x, recv_topk_idx | None, recv_weights | None) through nanoep_dispatch."""
+             use_table=True, use_order=True, order_count="exact", walk="forced"):
+    """Returns (recv_x, recv_topk_idx | None, recv_weights | None) through nanoep_dispatch.
+
+    The library picks the slot-order walk by itself only for batches of at least eight token
+    blocks; walk="forced" makes it walk whatever list it is given, so that small cases cover that
+    kernel too, walk="auto" leaves the choice to the library.
+    """
     recv_metadata, expert_counts, expert_offsets, dst_slots = metadata[0], metadata[1], metadata[2], metadata[3]
     received, capacity = counts[0], counts[1]
     tokens, hidden = x.shape
@@ -149,14 +155,21 @@ def dispatch(x, weights, metadata, counts, num_local_experts, alignment, expand,
     order = slot_order_of(metadata, use_order)
     # exact count A, or -1: the kernel reads A from the word behind the list
     order_entries = 0 if order is None else (counts[2] if order_count == "exact" else -1)
-    check(
-        lib().nanoep_dispatch(
+    previous = os.environ.pop("NANOEP_DISPATCH_ORDER", None)
+    if walk == "forced":
+        os.environ["NANOEP_DISPATCH_ORDER"] = "1"
+    try:
+        status = lib().nanoep_dispatch(
             ptr(x), ptr(weights), ptr(recv_metadata), ptr(dst_slots), ptr(token_slots_of(metadata, use_table)),
             ptr(order), order_entries, ptr(expert_counts), ptr(expert_offsets), received, capacity,
             tokens, hidden, topk, num_local_experts, alignment, int(expand), int(zero_padding), ptr(recv_x),
             ptr(recv_idx), ptr(recv_w), num_cus, stream_handle(),
         )
-    )
+    finally:
+        os.environ.pop("NANOEP_DISPATCH_ORDER", None)
+        if previous is not None:
+            os.environ["NANOEP_DISPATCH_ORDER"] = previous
+    check(status)
     return recv_x, recv_idx, recv_w
 
 
