@@ -200,14 +200,18 @@ def main():
     result = {}
     with torch.cuda.stream(stream):
         # fresh dispatch: layout kernels + host wait for N/C + permute, as seen by the caller
-        fresh_times = []
+        fresh_times, fresh_gpu_times = [], []
         for _ in range(10):
+            begin, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
             torch.cuda.synchronize()
             t0 = time.perf_counter()
+            begin.record(stream)
             received = buffer.dispatch(xs[0], topk_idx=idx, weights=weights, do_expand=workload.expand,
                                        alignment=workload.alignment, zero_padding=workload.zero_padding)
+            end.record(stream)
             torch.cuda.synchronize()
             fresh_times.append(time.perf_counter() - t0)
+            fresh_gpu_times.append(begin.elapsed_time(end) * 1e-3)
         layout_us = layout_gpu_us(workload, idx)
         handle = received.handle
         check_combined = buffer.combine(received.x, handle).x
@@ -304,6 +308,7 @@ def main():
             "combine_us": round(c_us, 2),
             "combine_GBps": round(c_bytes / c_us / 1e3, 1),
             "fresh_dispatch_us_host": round(statistics.median(fresh_times) * 1e6, 1),
+            "fresh_dispatch_us_gpu": round(statistics.median(fresh_gpu_times) * 1e6, 1),
             "layout_us_gpu_no_host_wait": round(layout_us, 2),
             "dispatch_bytes": d_bytes,
             "combine_bytes": c_bytes,
