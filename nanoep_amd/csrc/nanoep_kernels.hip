@@ -22,8 +22,10 @@
 //                          inside a block, so a block's source rows stay in one XCD's L2 and every
 //                          expert receives runs of consecutive rows; one 128-bit load and one
 //                          nontemporal 128-bit store per lane.
-//   dispatch_rows_kernel : the same work item walked in source-token order (compact layouts, handles
+//   dispatch_rows_kernel : the same work item walked in source-token order (small batches, handles
 //                          without the list); extra work items zero-fill the alignment gaps.
+//   dispatch_compact_kernel / combine_compact_kernel : compact layouts are row copies with holes;
+//                          plain launch order, single-wavefront workgroups, nothing but the copy.
 //   combine_rows_kernel  : one wavefront per (source token, row chunk): gathers the token's rows in
 //                          ascending k, fp32 accumulate, one round-to-nearest-even bf16 store.
 //
@@ -984,6 +986,53 @@ __global__ void __launch_bounds__(1024) dispatch_ordered_kernel(const u32x4* __r
         recv_weights[out_row] = weights[source];
 }
 
+// Compact layout: receive row r holds source token src_token(r), in token order, so the dispatch is
+// a row copy with holes.  Nothing is re-used, so workgroups walk the rows in plain launch order
+// (one linear stream over the whole device) and the kernel carries nothing but the copy.
+__global__ void __launch_bounds__(1024) dispatch_compact_kernel(const u32x4* __restrict__ x,                // [T][vectors]
+                                                                const float* __restrict__ weights,         // [T][K] or null
+                                                                const int32_t* __restrict__ recv_metadata,  // [N][K+2]
+                                                                const int64_t* __restrict__ dst_slots,     // [T]
+                                                                u32x4* __restrict__ recv_x,                // [N][vectors]
+                                                                int64_t* __restrict__ recv_topk_idx,       // [N][K] or null
+                                                                float* __restrict__ recv_weights,          // [N][K] or null
+                                                                uint32_t tokens,
+                                                                uint32_t recv_count,
+                                                                uint32_t parts,
+                                                                uint32_t parts_magic,
+                                                                uint32_t parts_shift,
+                                                                uint32_t chunks_per_block,  // == blockDim.y
+                                                                uint32_t rows_per_block,    // == blockDim.z
+                                                                uint32_t vectors,
+                                                                uint32_t chunks,
+                                                                uint32_t topk) {
+    NANOEP_FETCH_ARGS_4(x, dst_slots, recv_x, tokens);
+    NANOEP_FETCH_ARGS_4(recv_count, parts, parts_magic, parts_shift);
+    NANOEP_FETCH_ARGS_4(chunks_per_block, rows_per_block, vectors, chunks);
+    const uint32_t group = fast_divide(blockIdx.x, parts_magic, parts_shift);
+    const uint32_t part = blockIdx.x - group * parts;
+    const uint32_t token = group * rows_per_block + __builtin_amdgcn_readfirstlane(threadIdx.z);
+    const uint32_t chunk = part * chunks_per_block + __builtin_amdgcn_readfirstlane(threadIdx.y);
+    if (token >= tokens || chunk >= chunks)
+        return;
+    const uint32_t vector = chunk * kWave + threadIdx.x;
+    const bool in_row = vector < vectors;
+    // the source address depends on the block index alone: its load is in flight during the lookup
+    const u32x4 data = x[static_cast<uint64_t>(token) * vectors + (in_row ? vector : 0u)];
+    const int64_t row = uniform_load(dst_slots + token);
+    if (row < 0 || row >= static_cast<int64_t>(recv_count))
+        return;
+    if (in_row)
+        store_vec<true>(recv_x + static_cast<uint64_t>(row) * vectors + vector, data);
+    if (chunk == 0 && threadIdx.x < topk) {
+        const uint32_t lane = threadIdx.x;
+        if (recv_topk_idx != nullptr)
+            recv_topk_idx[row * topk + lane] = recv_metadata[row * (topk + 2) + 2 + lane];
+        if (recv_weights != nullptr)
+            recv_weights[row * topk + lane] = weights[static_cast<uint64_t>(token) * topk + lane];
+    }
+}
+
 // ---------------------------------------------------------------------------------------------
 // Combine gather-reduce
 // ---------------------------------------------------------------------------------------------
@@ -1137,6 +1186,64 @@ __global__ void __launch_bounds__(kBlockThreads) copy_vectors_kernel(const u32x4
 // Launch helpers
 // ---------------------------------------------------------------------------------------------
 
+// Compact layout: a token has one received row, so the combine is a row copy through fp32
+// (0.0f + x, which turns -0 into +0 and quiets NaNs, then the bias) with holes: tokens that were
+// not sent get 0 (+bias).  Plain launch order, nothing but the copy in the kernel.
+__global__ void __launch_bounds__(1024) combine_compact_kernel(const u32x4* __restrict__ y,                // [N][vectors]
+                                                               const float* __restrict__ weights,         // [N][K] or null
+                                                               const u32x4* __restrict__ bias,            // [T][vectors] or null
+                                                               const int32_t* __restrict__ recv_metadata,  // [N][K+2]
+                                                               const int64_t* __restrict__ dst_slots,     // [T]
+                                                               u32x4* __restrict__ out_x,                 // [T][vectors]
+                                                               float* __restrict__ out_weights,           // [T][K] or null
+                                                               uint32_t tokens,
+                                                               uint32_t recv_count,
+                                                               uint32_t parts,
+                                                               uint32_t parts_magic,
+                                                               uint32_t parts_shift,
+                                                               uint32_t chunks_per_block,  // == blockDim.y
+                                                               uint32_t rows_per_block,    // == blockDim.z
+                                                               uint32_t vectors,
+                                                               uint32_t chunks,
+                                                               uint32_t topk) {
+    NANOEP_FETCH_ARGS_4(y, dst_slots, out_x, bias);
+    NANOEP_FETCH_ARGS_4(tokens, recv_count, parts, parts_magic);
+    NANOEP_FETCH_ARGS_4(parts_shift, chunks_per_block, rows_per_block, vectors);
+    const uint32_t group = fast_divide(blockIdx.x, parts_magic, parts_shift);
+    const uint32_t part = blockIdx.x - group * parts;
+    const uint32_t token = group * rows_per_block + __builtin_amdgcn_readfirstlane(threadIdx.z);
+    const uint32_t chunk = part * chunks_per_block + __builtin_amdgcn_readfirstlane(threadIdx.y);
+    if (token >= tokens || chunk >= chunks)
+        return;
+    const uint32_t vector = chunk * kWave + threadIdx.x;
+    const bool in_row = vector < vectors;
+    const uint32_t load_vector = in_row ? vector : 0u;
+    const int64_t row = uniform_load(dst_slots + token);
+    const bool received = row >= 0 && row < static_cast<int64_t>(recv_count);
+    // a token that was not sent re-reads row 0 and drops it: the load stays unconditional
+    const u32x4 data = load_vec<true>(y + static_cast<uint64_t>(received ? row : 0) * vectors + load_vector);
+    float acc[8] = {0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f};
+    if (received)
+        accumulate(acc, data);
+    if (bias != nullptr)
+        accumulate(acc, load_vec<true>(bias + static_cast<uint64_t>(token) * vectors + load_vector));
+    if (in_row) {
+        u32x4 packed;
+        packed.x = bf16_round(acc[0]) | (bf16_round(acc[1]) << 16);
+        packed.y = bf16_round(acc[2]) | (bf16_round(acc[3]) << 16);
+        packed.z = bf16_round(acc[4]) | (bf16_round(acc[5]) << 16);
+        packed.w = bf16_round(acc[6]) | (bf16_round(acc[7]) << 16);
+        store_vec<true>(out_x + static_cast<uint64_t>(token) * vectors + vector, packed);
+    }
+    if (chunk == 0 && out_weights != nullptr && threadIdx.x < topk) {
+        const uint32_t lane = threadIdx.x;
+        float weight = 0.0f;
+        if (received && recv_metadata[row * (topk + 2) + 2 + lane] >= 0)
+            weight = weights[row * topk + lane];
+        out_weights[static_cast<uint64_t>(token) * topk + lane] = weight;
+    }
+}
+
 constexpr int kMaxWavesPerBlock = 16;
 constexpr int kDefaultChunksPerBlock = 2;
 
@@ -1149,17 +1256,22 @@ struct RowBlocking {
     unsigned parts;
 };
 
-RowBlocking pick_row_blocking(int chunks, bool ordered = false) {
+enum WalkShape {
+    kTokenOrderWalk,  // two-wavefront workgroups: best or within noise of best for the expanded token-order walks
+    kSlotOrderWalk,   // the row split evenly over workgroups of up to 8 wavefronts
+    kRowCopyWalk,     // compact layouts (plain row copies): single-wavefront workgroups
+};
+
+RowBlocking pick_row_blocking(int chunks, WalkShape shape) {
     RowBlocking blocking{};
-    // Token-order walks: two-wavefront workgroups measured best or within noise of best on every
-    // shape tried (rows of 4 to 14 chunks, expanded and compact); they retire and refill quickest.
-    // Slot-order walks do better with the row split evenly over workgroups of up to 8 wavefronts.
     int per_block = env_int("NANOEP_CHUNKS_PER_BLOCK", 0);
     if (per_block < 1 || per_block > kMaxWavesPerBlock) {
         per_block = kDefaultChunksPerBlock;
-        if (ordered) {
+        if (shape == kSlotOrderWalk) {
             const int pieces = (chunks + 7) / 8;
             per_block = (chunks + pieces - 1) / pieces;
+        } else if (shape == kRowCopyWalk) {
+            per_block = 1;
         }
     }
     if (per_block > chunks)
@@ -1449,7 +1561,7 @@ int nanoep_dispatch(const void* x, const float* weights, const int32_t* recv_met
 
     const int vectors = hidden / 8;
     const int chunks = (vectors + kWave - 1) / kWave;
-    const RowBlocking blocking = pick_row_blocking(chunks, ordered);
+    const RowBlocking blocking = pick_row_blocking(chunks, ordered ? kSlotOrderWalk : expand ? kTokenOrderWalk : kRowCopyWalk);
     const int64_t waves = static_cast<int64_t>(blocking.chunks_per_block) * blocking.rows_per_block;
     const int64_t copy_candidates = ordered ? slot_order_entries : expand ? num_tokens * num_topk : num_tokens;
     const int64_t copy_blocks = (copy_candidates + blocking.rows_per_block - 1) / blocking.rows_per_block * blocking.parts;
@@ -1491,6 +1603,13 @@ int nanoep_dispatch(const void* x, const float* weights, const int32_t* recv_met
         else
             NANOEP_LAUNCH_ORDERED(false, false);
 #undef NANOEP_LAUNCH_ORDERED
+    } else if (!expand) {
+        const int64_t blocks = (num_tokens + blocking.rows_per_block - 1) / blocking.rows_per_block * blocking.parts;
+        dispatch_compact_kernel<<<dim3(static_cast<unsigned>(blocks)), block, 0, stream>>>(
+            static_cast<const u32x4*>(x), weights, recv_metadata, dst_slots, static_cast<u32x4*>(recv_x), recv_topk_idx,
+            recv_weights, static_cast<uint32_t>(num_tokens), static_cast<uint32_t>(recv_count), blocking.parts,
+            parts_divisor.magic, parts_divisor.shift, blocking.chunks_per_block, blocking.rows_per_block,
+            static_cast<uint32_t>(vectors), static_cast<uint32_t>(chunks), static_cast<uint32_t>(num_topk));
     } else {
 #define NANOEP_LAUNCH_ROWS(LOOKUP, ZERO_FILL)                                                                         \
     dispatch_rows_kernel<LOOKUP, ZERO_FILL><<<grid, block, 0, stream>>>(                                             \
@@ -1542,7 +1661,7 @@ int nanoep_combine(const void* y, const float* weights, const void* bias, const 
 
     const int vectors = hidden / 8;
     const int chunks = (vectors + kWave - 1) / kWave;
-    const RowBlocking blocking = pick_row_blocking(chunks);
+    const RowBlocking blocking = pick_row_blocking(chunks, expand ? kTokenOrderWalk : kRowCopyWalk);
     const int64_t blocks = (num_tokens + blocking.rows_per_block - 1) / blocking.rows_per_block * blocking.parts;
     if (blocks >= (int64_t{1} << 31))
         return NANOEP_ERR_INVALID_ARGUMENT;
@@ -1553,6 +1672,17 @@ int nanoep_combine(const void* y, const float* weights, const void* bias, const 
     // the slot table only helps the expanded layout, and only when something was received
     const bool direct = token_slots != nullptr && expand && recv_count > 0;
     const FastDivisor parts_divisor = make_fast_divisor(blocking.parts);
+    if (!expand) {
+        // y may be a null pointer when nothing was received: every token then takes the hole path
+        combine_compact_kernel<<<grid, block, 0, stream>>>(
+            static_cast<const u32x4*>(recv_count > 0 ? y : out_x), weights, static_cast<const u32x4*>(bias), recv_metadata,
+            dst_slots, static_cast<u32x4*>(out_x), out_weights, static_cast<uint32_t>(num_tokens),
+            static_cast<uint32_t>(recv_count), blocking.parts, parts_divisor.magic, parts_divisor.shift,
+            blocking.chunks_per_block, blocking.rows_per_block, static_cast<uint32_t>(vectors), static_cast<uint32_t>(chunks),
+            static_cast<uint32_t>(num_topk));
+        NANOEP_HIP_TRY(hipGetLastError());
+        return NANOEP_OK;
+    }
 #define NANOEP_LAUNCH_COMBINE(GROUP, DIRECT)                                                                       \
     combine_rows_kernel<GROUP, DIRECT><<<grid, block, 0, stream>>>(                                                \
         static_cast<const u32x4*>(y), weights, static_cast<const u32x4*>(bias), recv_metadata, dst_slots,          \
