@@ -256,6 +256,29 @@ def test_both_layout_launch_plans(device, monkeypatch, launches, tokens, experts
     assert_layout(metadata, counts, oracle.layout(idx, experts, alignment), expand)
 
 
+@pytest.mark.parametrize("seed", range(24))
+def test_randomized_shapes(device, seed):
+    """Seeded random geometries: ragged token counts, hidden sizes that are not multiples of 512 or
+    even of 64 vectors, odd top-k, expert counts past one and two wavefronts of experts, odd
+    alignments -- every one checked bit for bit against the oracle through all walks."""
+    g = torch.Generator().manual_seed(1000 + seed)
+
+    def pick(options):
+        return options[int(torch.randint(len(options), (1,), generator=g))]
+
+    topk = pick([1, 2, 3, 4, 6, 7, 8, 11])
+    experts = max(topk, pick([1, 2, 5, 8, 31, 64, 65, 130, 300]))
+    tokens = pick([1, 2, 31, 33, 63, 100, 255, 256, 257, 511, 700])
+    hidden = 8 * pick([1, 3, 8, 31, 32, 33, 64, 65, 96, 128, 160, 257])
+    alignment = pick([1, 1, 2, 3, 8, 128])
+    kind = pick(["random", "dropout", "sparse", "biased"])
+    expand = pick([False, True, True])
+    zero_padding = expand and pick([False, True])
+    weighted = pick([False, True])
+    idx = cases.routing(kind, tokens, experts, topk, seed=seed)
+    run_dispatch_combine(device, idx, hidden, experts, alignment, expand, zero_padding, weighted, seed=seed)
+
+
 def test_empty_inputs(device):
     for expand in (False, True):
         idx = torch.empty((0, 4), dtype=torch.int64)
