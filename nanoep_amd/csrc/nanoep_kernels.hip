@@ -28,6 +28,7 @@
 //                          plain launch order, single-wavefront workgroups, nothing but the copy.
 //   combine_rows_kernel  : one wavefront per (source token, row chunk): gathers the token's rows in
 //                          ascending k, fp32 accumulate, one round-to-nearest-even bf16 store.
+//   combine_few_rows_kernel : the same for K <= 4 with the slot table, without the bookkeeping.
 //
 // Every byte moved is HBM-bound integer/byte work; there is no contraction, hence no MFMA.
 
@@ -1186,6 +1187,88 @@ __global__ void __launch_bounds__(kBlockThreads) copy_vectors_kernel(const u32x4
 // Launch helpers
 // ---------------------------------------------------------------------------------------------
 
+// Expanded layout with at most kTopk <= 4 rows per token and the slot table at hand: the same
+// gather-sum as combine_rows_kernel, carrying only what that case needs (the token's slots come as
+// scalars straight from the table).  With so few rows per token the kernel is short and close to a
+// copy, and the general kernel's bookkeeping showed (Mixtral-shaped batch: 19.3 us against 17.3 us
+// for the bare access pattern).
+template <int kTopk>
+__global__ void __launch_bounds__(1024) combine_few_rows_kernel(const u32x4* __restrict__ y,              // [C][vectors]
+                                                                const float* __restrict__ weights,       // [C] or null
+                                                                const u32x4* __restrict__ bias,          // [T][vectors] or null
+                                                                const int32_t* __restrict__ token_slots,  // [T][K]
+                                                                u32x4* __restrict__ out_x,               // [T][vectors]
+                                                                float* __restrict__ out_weights,         // [T][K] or null
+                                                                uint32_t tokens,
+                                                                uint32_t y_rows,
+                                                                uint32_t parts,
+                                                                uint32_t parts_magic,
+                                                                uint32_t parts_shift,
+                                                                uint32_t chunks_per_block,  // == blockDim.y
+                                                                uint32_t rows_per_block,    // == blockDim.z
+                                                                uint32_t vectors,
+                                                                uint32_t chunks,
+                                                                uint32_t topk,
+                                                                int multiple_reduction) {
+    NANOEP_FETCH_ARGS_4(y, token_slots, out_x, bias);
+    NANOEP_FETCH_ARGS_4(tokens, y_rows, parts, parts_magic);
+    NANOEP_FETCH_ARGS_4(parts_shift, chunks_per_block, rows_per_block, vectors);
+    NANOEP_FETCH_ARGS_4(chunks, topk, multiple_reduction, out_weights);
+    const uint32_t group = fast_divide(blockIdx.x, parts_magic, parts_shift);
+    const uint32_t part = blockIdx.x - group * parts;
+    const uint32_t token = group * rows_per_block + __builtin_amdgcn_readfirstlane(threadIdx.z);
+    const uint32_t chunk = part * chunks_per_block + __builtin_amdgcn_readfirstlane(threadIdx.y);
+    if (token >= tokens || chunk >= chunks)
+        return;
+    const uint32_t vector = chunk * kWave + threadIdx.x;
+    const bool in_row = vector < vectors;
+    const uint32_t load_vector = in_row ? vector : 0u;
+    const int32_t* slots = token_slots + static_cast<uint64_t>(token) * topk;
+    int32_t slot[kTopk];
+    bool valid[kTopk];
+#pragma unroll
+    for (int k = 0; k < kTopk; ++k) {
+        slot[k] = uniform_load(slots + (static_cast<uint32_t>(k) < topk ? k : 0));
+        valid[k] = static_cast<uint32_t>(k) < topk && slot[k] >= 0 && static_cast<uint32_t>(slot[k]) < y_rows;
+    }
+    u32x4 data[kTopk];
+#pragma unroll
+    for (int k = 0; k < kTopk; ++k)  // a masked k re-reads row 0 and drops it: the loads stay unconditional
+        data[k] = load_vec<true>(y + static_cast<uint64_t>(valid[k] ? slot[k] : 0) * vectors + load_vector);
+    u32x4 bias_data = {0u, 0u, 0u, 0u};
+    if (bias != nullptr)
+        bias_data = load_vec<true>(bias + static_cast<uint64_t>(token) * vectors + load_vector);
+    float acc[8] = {0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f};
+    int valid_count = 0;
+#pragma unroll
+    for (int k = 0; k < kTopk; ++k) {
+        if (valid[k]) {
+            accumulate(acc, data[k]);
+            ++valid_count;
+        }
+    }
+    if (multiple_reduction && valid_count >= 2) {
+#pragma unroll
+        for (int j = 0; j < 8; ++j)
+            acc[j] = 0.0f + __uint_as_float(bf16_round(acc[j]) << 16);
+    }
+    if (bias != nullptr)
+        accumulate(acc, bias_data);
+    if (in_row) {
+        u32x4 packed;
+        packed.x = bf16_round(acc[0]) | (bf16_round(acc[1]) << 16);
+        packed.y = bf16_round(acc[2]) | (bf16_round(acc[3]) << 16);
+        packed.z = bf16_round(acc[4]) | (bf16_round(acc[5]) << 16);
+        packed.w = bf16_round(acc[6]) | (bf16_round(acc[7]) << 16);
+        store_vec<true>(out_x + static_cast<uint64_t>(token) * vectors + vector, packed);
+    }
+    if (chunk == 0 && out_weights != nullptr && threadIdx.x < topk) {
+        const int32_t mine = slots[threadIdx.x];
+        const bool mine_valid = mine >= 0 && static_cast<uint32_t>(mine) < y_rows;
+        out_weights[static_cast<uint64_t>(token) * topk + threadIdx.x] = mine_valid ? weights[mine] : 0.0f;
+    }
+}
+
 // Compact layout: a token has one received row, so the combine is a row copy through fp32
 // (0.0f + x, which turns -0 into +0 and quiets NaNs, then the bias) with holes: tokens that were
 // not sent get 0 (+bias).  Plain launch order, nothing but the copy in the kernel.
@@ -1680,6 +1763,22 @@ int nanoep_combine(const void* y, const float* weights, const void* bias, const 
             static_cast<uint32_t>(recv_count), blocking.parts, parts_divisor.magic, parts_divisor.shift,
             blocking.chunks_per_block, blocking.rows_per_block, static_cast<uint32_t>(vectors), static_cast<uint32_t>(chunks),
             static_cast<uint32_t>(num_topk));
+        NANOEP_HIP_TRY(hipGetLastError());
+        return NANOEP_OK;
+    }
+    if (direct && num_topk >= 2 && num_topk <= 4) {
+#define NANOEP_LAUNCH_FEW(TOPK)                                                                                       \
+    combine_few_rows_kernel<TOPK><<<grid, block, 0, stream>>>(                                                       \
+        static_cast<const u32x4*>(y), weights, static_cast<const u32x4*>(bias), token_slots,                         \
+        static_cast<u32x4*>(out_x), out_weights, static_cast<uint32_t>(num_tokens), static_cast<uint32_t>(y_rows),   \
+        blocking.parts, parts_divisor.magic, parts_divisor.shift, blocking.chunks_per_block, blocking.rows_per_block, \
+        static_cast<uint32_t>(vectors), static_cast<uint32_t>(chunks), static_cast<uint32_t>(num_topk),              \
+        multiple_reduction ? 1 : 0)
+        if (num_topk == 2)
+            NANOEP_LAUNCH_FEW(2);
+        else
+            NANOEP_LAUNCH_FEW(4);
+#undef NANOEP_LAUNCH_FEW
         NANOEP_HIP_TRY(hipGetLastError());
         return NANOEP_OK;
     }
