@@ -393,37 +393,50 @@ DispatchResult dispatch(PeerRuntime& runtime,
         torch::Tensor recv_metadata, expert_counts, expert_offsets, dst_slots, send_counts, snapshot, prefix, token_slots, slot_order;
         // the slot-order list packs token * K + k into 32 bits
         const bool ordered = expand && tokens * topk < (int64_t{1} << 31);
-        allocate_for_consumer([&] {
-            recv_metadata = torch::empty({tokens, topk + 2}, int64_options.dtype(torch::kInt32));
-            expert_counts = torch::empty({local_experts}, int64_options);
-            expert_offsets = torch::empty({local_experts + 1}, int64_options);
-            dst_slots = torch::empty({tokens, 1}, int64_options);
-            send_counts = torch::empty({1}, int64_options);
-            snapshot = torch::empty_like(routing);
-            prefix = torch::empty({1}, int64_options);
-            if (expand)
-                token_slots = torch::empty({tokens, topk}, int64_options.dtype(torch::kInt32));
-            if (ordered)
-                slot_order = torch::empty({nanoep_slot_order_entries(tokens, static_cast<int>(topk), local_experts)}, int64_options);
-            return 0;
-        });
-        metadata = {recv_metadata, expert_counts, expert_offsets, dst_slots, send_counts, snapshot, prefix};
-        if (expand)
-            metadata.push_back(token_slots);  // private eighth entry: slot[t,k] in one lookup
-        if (ordered)
-            metadata.push_back(slot_order);  // private ninth entry: assignments in block-wise slot order
+        // The handle tensors of one call are views of two arenas (one per element type), and the
+        // views are made after the layout has been enqueued: on a path whose small-batch cost is
+        // host latency, the GPU starts three allocator round trips after the call instead of ten
+        // and works while the rest of the bookkeeping is done.
+        const int64_t order_entries = ordered ? nanoep_slot_order_entries(tokens, static_cast<int>(topk), local_experts) : 0;
+        const int64_t count64 = 2 * local_experts + 3 + tokens + tokens * topk + order_entries;
+        const int64_t count32 = tokens * (topk + 2) + (expand ? tokens * topk : 0);
         const size_t workspace_bytes = nanoep_layout_workspace_bytes(tokens, static_cast<int>(topk), local_experts);
         TORCH_CHECK(workspace_bytes > 0, "unsupported routing geometry for the layout kernels");
+        torch::Tensor arena64, arena32;
+        allocate_for_consumer([&] {
+            arena64 = torch::empty({count64}, int64_options);
+            arena32 = torch::empty({count32 > 0 ? count32 : 1}, int64_options.dtype(torch::kInt32));
+            return 0;
+        });
         auto workspace = torch::empty({static_cast<int64_t>(workspace_bytes)}, int64_options.dtype(torch::kUInt8));
+        // arena64: expert_counts [L] | expert_offsets [L+1] | send_counts [1] | recv_rank_prefix [1] |
+        //          dst_slots [T] | topk snapshot [T*K] | slot_order;   arena32: recv_metadata [T*(K+2)] | token_slots [T*K]
+        const int64_t at_offsets = local_experts, at_send = 2 * local_experts + 1, at_prefix = at_send + 1, at_dst = at_prefix + 1;
+        const int64_t at_snapshot = at_dst + tokens, at_order = at_snapshot + tokens * topk, at_table = tokens * (topk + 2);
+        int64_t* base64 = arena64.data_ptr<int64_t>();
+        int32_t* base32 = arena32.data_ptr<int32_t>();
         check_status(nanoep_layout(routing.data_ptr<int64_t>(), tokens, static_cast<int>(topk), local_experts, alignment, expand ? 1 : 0,
-                                   recv_metadata.data_ptr<int32_t>(), expert_counts.data_ptr<int64_t>(),
-                                   expert_offsets.data_ptr<int64_t>(), dst_slots.data_ptr<int64_t>(), send_counts.data_ptr<int64_t>(),
-                                   snapshot.data_ptr<int64_t>(), prefix.data_ptr<int64_t>(),
-                                   expand ? token_slots.data_ptr<int32_t>() : nullptr,
-                                   ordered && slot_order.numel() > 0 ? slot_order.data_ptr<int64_t>() : nullptr, workspace.data_ptr(),
-                                   workspace_bytes,
+                                   base32, base64, base64 + at_offsets, base64 + at_dst, base64 + at_send, base64 + at_snapshot,
+                                   base64 + at_prefix, expand ? base32 + at_table : nullptr,
+                                   order_entries > 0 ? base64 + at_order : nullptr, workspace.data_ptr(), workspace_bytes,
                                    host_counts, comm.stream()),
                      "layout");
+        expert_counts = arena64.narrow(0, 0, local_experts);
+        expert_offsets = arena64.narrow(0, at_offsets, local_experts + 1);
+        send_counts = arena64.narrow(0, at_send, 1);
+        prefix = arena64.narrow(0, at_prefix, 1);
+        dst_slots = arena64.narrow(0, at_dst, tokens).view({tokens, 1});
+        snapshot = arena64.narrow(0, at_snapshot, tokens * topk).view({tokens, topk});
+        recv_metadata = arena32.narrow(0, 0, tokens * (topk + 2)).view({tokens, topk + 2});
+        metadata = {recv_metadata, expert_counts, expert_offsets, dst_slots, send_counts, snapshot, prefix};
+        if (expand) {
+            token_slots = arena32.narrow(0, at_table, tokens * topk).view({tokens, topk});
+            metadata.push_back(token_slots);  // private eighth entry: slot[t,k] in one lookup
+        }
+        if (ordered) {
+            slot_order = arena64.narrow(0, at_order, order_entries);
+            metadata.push_back(slot_order);  // private ninth entry: assignments in block-wise slot order
+        }
 
         // The exact shapes (N, C) are only known once the layout kernels have run.  Waiting for
         // them before launching the permute would leave the GPU idle for a host round trip, so the
