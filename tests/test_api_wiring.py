@@ -283,3 +283,16 @@ def test_construction_checks_without_a_gpu():
         api.CudaBuffer(None, EPConfig(2, 2, 256, 4), allow_multiple_reduction="no")
     with pytest.raises(RuntimeError, match="no GPU"):
         api.CudaBuffer(None, EPConfig(2, 2, 256, 4))
+
+
+def test_reference_import_paths():
+    """`nano_ep`, `nano_ep.backends` and `nano_ep.backends.cuda` export these names (nano_ep/__init__.py,
+    nano_ep/backends/__init__.py); the same import paths exist here and name the same objects."""
+    import nanoep_amd
+    from nanoep_amd import backends
+    from nanoep_amd.backends import cuda
+
+    for name in ("CudaBuffer", "CudaEvent", "NativeCombineResult", "NativeDispatchResult", "NativeHandle", "NativeLayout"):
+        assert getattr(backends, name) is getattr(nanoep_amd, name) is getattr(cuda, name)
+    assert nanoep_amd.EPConfig is not None and nanoep_amd.__version__
+    assert callable(cuda.check_torch_deterministic)
