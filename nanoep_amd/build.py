@@ -25,6 +25,8 @@ KERNEL_LIBRARY = PACKAGE / "libnanoep_hip.so"
 EXTENSION_NAME = "_nanoep_torch"
 EXTENSION_LIBRARY = PACKAGE / f"{EXTENSION_NAME}.so"
 
+KERNEL_SOURCES = ["nanoep_layout.hip", "nanoep_dispatch.hip", "nanoep_combine.hip", "nanoep_abi.hip"]
+
 OFFLOAD_ARCH = "gfx950"
 # Packed fp32 instructions are disabled for every HIP translation unit of this project.
 HIPCC_FLAGS = [
@@ -59,7 +61,8 @@ def hipcc_path() -> str:
 
 
 def build_kernels(verbose: bool = False) -> Path:
-    command = [hipcc_path(), *HIPCC_FLAGS, f"-I{INCLUDE}", str(CSRC / "nanoep_kernels.hip"), "-o", str(KERNEL_LIBRARY)]
+    sources = [str(CSRC / name) for name in KERNEL_SOURCES]
+    command = [hipcc_path(), *HIPCC_FLAGS, f"-I{INCLUDE}", f"-I{CSRC}", *sources, "-o", str(KERNEL_LIBRARY)]
     _run(command, verbose)
     return KERNEL_LIBRARY
 

@@ -1,0 +1,207 @@
+// MI355X (gfx950, wave64) kernels for one rank's expert-parallel dispatch / combine, and the
+// C ABI declared in include/nanoep_hip.h: nanoep_layout.hip, nanoep_dispatch.hip,
+// nanoep_combine.hip, nanoep_abi.hip.  This header holds what they share.
+//
+// Data layout in HBM (all row-major, contiguous):
+//   x, recv_x, y, out_x, bias : bf16 rows of H elements, moved as 16-byte vectors (H/8 per row)
+//   topk_idx / snapshot       : int64 [T,K]
+//   recv_metadata             : int32 [N,K+2]   (src_rank, src_token, K values)
+//   weights                   : fp32 [T,K] at the source, [N,K] compact, [C] expanded
+//
+// Kernels
+//   layout_count_kernel  : one workgroup per block of tokens; LDS bit matrix (expert x token) built
+//                          with LDS atomics, popcount prefixes give the in-block stable rank of
+//                          every (token,k) and the block's per-expert histogram.
+//   layout_assign_kernel<fused scan> : (few blocks) every workgroup sums the block histograms into
+//                          LDS, scans the aligned expert totals and writes its tokens' part of the
+//                          handle and of the slot-order list; workgroup 0 publishes N, C to the host.
+//   layout_single_block_kernel : (one block) count and assignment passes in a single launch.
+//   layout_scan_kernel + layout_assign_kernel<no scan> : (many blocks) the same in two launches, one
+//                          workgroup doing the scans: slot = offset[e] + block_base[b][e] + rank.
+//   dispatch_ordered_kernel : expanded layouts with the layout's slot-order list: one wavefront per
+//                          (list entry, row chunk), token block by token block and expert-major
+//                          inside a block, so a block's source rows stay in one XCD's L2 and every
+//                          expert receives runs of consecutive rows; one 128-bit load and one
+//                          nontemporal 128-bit store per lane.
+//   dispatch_rows_kernel : the same work item walked in source-token order (small batches, handles
+//                          without the list); extra work items zero-fill the alignment gaps.
+//   dispatch_compact_kernel / combine_compact_kernel : compact layouts are row copies with holes;
+//                          plain launch order, single-wavefront workgroups, nothing but the copy.
+//   combine_rows_kernel  : one wavefront per (source token, row chunk): gathers the token's rows in
+//                          ascending k, fp32 accumulate, one round-to-nearest-even bf16 store.
+//   combine_few_rows_kernel : the same for K <= 4 with the slot table, without the bookkeeping.
+//
+// Every byte moved is HBM-bound integer/byte work; there is no contraction, hence no MFMA.
+#ifndef NANOEP_DEVICE_H_
+#define NANOEP_DEVICE_H_
+
+#include <hip/hip_runtime.h>
+
+#include <cstdint>
+#include <cstdio>
+#include <cstdlib>
+#include <cstring>
+#include <type_traits>
+
+#include "nanoep_hip.h"
+
+namespace nanoep {
+
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+
+constexpr int kWave = 64;
+constexpr int kWavesPerBlock = 4;
+constexpr int kBlockThreads = kWave * kWavesPerBlock;
+constexpr int kScanThreads = 1024;
+constexpr int kMaxTopk = 32;
+constexpr size_t kLayoutLdsBudget = 60 * 1024;
+
+// Last HIP failure seen on this thread (nanoep_last_hip_error reports it); defined in nanoep_abi.hip.
+extern thread_local hipError_t g_last_hip_error;
+
+#define NANOEP_HIP_TRY(expr)              \
+    do {                                  \
+        const hipError_t status_ = (expr); \
+        if (status_ != hipSuccess) {      \
+            ::nanoep::g_last_hip_error = status_;   \
+            return NANOEP_ERR_HIP;        \
+        }                                 \
+    } while (0)
+
+inline size_t align_up(size_t value, size_t alignment) { return (value + alignment - 1) / alignment * alignment; }
+
+inline int env_int(const char* name, int fallback) {
+    const char* text = std::getenv(name);
+    if (text == nullptr || *text == '\0')
+        return fallback;
+    return std::atoi(text);
+}
+
+// Calls f with the smallest compile-time bound in {4, 8, 16, 32} that covers num_topk.
+template <typename F>
+void with_topk_cap(int num_topk, F&& f) {
+    if (num_topk <= 4)
+        f(std::integral_constant<int, 4>{});
+    else if (num_topk <= 8)
+        f(std::integral_constant<int, 8>{});
+    else if (num_topk <= 16)
+        f(std::integral_constant<int, 16>{});
+    else
+        f(std::integral_constant<int, 32>{});
+}
+
+template <bool kNonTemporal>
+__device__ __forceinline__ u32x4 load_vec(const u32x4* p) {
+    if constexpr (kNonTemporal)
+        return __builtin_nontemporal_load(p);
+    else
+        return *p;
+}
+
+template <bool kNonTemporal>
+__device__ __forceinline__ void store_vec(u32x4* p, u32x4 v) {
+    if constexpr (kNonTemporal)
+        __builtin_nontemporal_store(v, p);
+    else
+        *p = v;
+}
+
+// Load through the scalar data path: the address must be wave-uniform and the memory read-only for
+// the duration of the kernel (true of all handle tensors here).  Keeps lookups out of the vector
+// memory pipeline and their results in SGPRs.
+template <class T>
+__device__ __forceinline__ T uniform_load(const T* p) {
+    return *(const __attribute__((address_space(4))) T*)(p);
+}
+
+// Workgroups are handed to the 8 XCDs round-robin by their linear id, and every XCD has its own L2.
+constexpr int kNumXcds = 8;
+
+// n / d for n < 2^31 as one 64-bit multiply and shift: magic = ceil(2^shift / d), shift = 31 + ceil(log2 d).
+struct FastDivisor {
+    uint32_t magic;
+    uint32_t shift;
+};
+
+inline FastDivisor make_fast_divisor(uint32_t divisor) {
+    uint32_t log2_ceil = 0;
+    while ((uint64_t{1} << log2_ceil) < divisor)
+        ++log2_ceil;
+    const uint32_t shift = 31 + log2_ceil;
+    const uint64_t power = uint64_t{1} << shift;
+    return {static_cast<uint32_t>((power + divisor - 1) / divisor), shift};
+}
+
+__device__ __forceinline__ uint32_t fast_divide(uint32_t n, uint32_t magic, uint32_t shift) {
+    return static_cast<uint32_t>((static_cast<uint64_t>(n) * magic) >> shift);
+}
+
+// Kernel arguments are fetched with scalar loads where they are first used, which strings several
+// dependent round trips along a short wavefront's life.  Naming them in an empty asm statement at
+// the top of the kernel makes the compiler fetch them all in one batch.
+#define NANOEP_FETCH_ARGS_2(a, b) asm volatile("" ::"s"(a), "s"(b))
+#define NANOEP_FETCH_ARGS_4(a, b, c, d) asm volatile("" ::"s"(a), "s"(b), "s"(c), "s"(d))
+
+constexpr int kMaxWavesPerBlock = 16;
+constexpr int kDefaultChunksPerBlock = 2;
+
+// Workgroup shape (64, chunks_per_block, rows_per_block) for rows of `chunks` 1 KiB chunks; a row
+// longer than chunks_per_block is covered by `parts` consecutive workgroups, and rows of a single
+// chunk are grouped so that a workgroup still has a few wavefronts.
+struct RowBlocking {
+    unsigned chunks_per_block;
+    unsigned rows_per_block;
+    unsigned parts;
+};
+
+enum WalkShape {
+    kTokenOrderWalk,  // two-wavefront workgroups: best or within noise of best for the expanded token-order walks
+    kSlotOrderWalk,   // the row split evenly over workgroups of up to 8 wavefronts
+    kRowCopyWalk,     // compact layouts (plain row copies): single-wavefront workgroups
+};
+
+inline RowBlocking pick_row_blocking(int chunks, WalkShape shape) {
+    RowBlocking blocking{};
+    int per_block = env_int("NANOEP_CHUNKS_PER_BLOCK", 0);
+    if (per_block < 1 || per_block > kMaxWavesPerBlock) {
+        per_block = kDefaultChunksPerBlock;
+        if (shape == kSlotOrderWalk) {
+            const int pieces = (chunks + 7) / 8;
+            per_block = (chunks + pieces - 1) / pieces;
+        } else if (shape == kRowCopyWalk) {
+            per_block = 1;
+        }
+    }
+    if (per_block > chunks)
+        per_block = chunks;
+    blocking.chunks_per_block = static_cast<unsigned>(per_block);
+    blocking.parts = static_cast<unsigned>((chunks + per_block - 1) / per_block);
+    int rows = 1;
+    if (blocking.parts == 1) {
+        rows = env_int("NANOEP_ROWS_PER_BLOCK", 0);
+        if (rows < 1 || rows * per_block > kMaxWavesPerBlock)
+            rows = per_block >= 4 ? 1 : 4 / per_block;
+    }
+    blocking.rows_per_block = static_cast<unsigned>(rows);
+    return blocking;
+}
+
+inline int validate_cu_budget(int num_cus) {
+    int device = 0;
+    NANOEP_HIP_TRY(hipGetDevice(&device));
+    static thread_local int cached_device = -1;
+    static thread_local int cached_cus = 0;
+    if (device != cached_device) {
+        int cus = 0;
+        NANOEP_HIP_TRY(hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, device));
+        cached_device = device;
+        cached_cus = cus;
+    }
+    return (num_cus < 0 || num_cus > cached_cus) ? NANOEP_ERR_INVALID_ARGUMENT : NANOEP_OK;
+}
+
+inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+
+}  // namespace nanoep
+
+#endif  // NANOEP_DEVICE_H_

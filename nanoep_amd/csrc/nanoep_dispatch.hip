@@ -1,0 +1,424 @@
+// Dispatch permute / expand: slot-order walk, token-order walks, compact row copy, zero fill.
+
+#include "nanoep_device.h"
+
+namespace nanoep {
+namespace {
+
+// One wavefront moves one 1 KiB chunk (64 lanes x 16 bytes) of one destination row with exactly
+// one 128-bit load and one nontemporal 128-bit store per lane: on this part a wavefront that issues
+// a single store and retires sustains more HBM write bandwidth than one that issues several.
+//
+// A workgroup is (64, chunks_per_block, rows_per_block): threadIdx.y is the chunk, threadIdx.z the
+// destination candidate, so no per-wave division by the chunk count is needed.  Candidates are
+// ordered (source token, k): the K destinations of a token are handled by consecutive workgroups
+// behind one XCD's L2, so only the first read of a source row goes to HBM, and every destination
+// row is written as one contiguous run by the wavefronts of one workgroup.  The source address
+// depends only on the block index, so its load is in flight while the wave-uniform lookups
+// (token_slots[t][k], or dst_slots[t] -> recv_metadata[row][2+k] for a handle without that table)
+// resolve the destination row.
+//
+// Zero-fill workgroups clear the alignment gaps: workgroup (e, g) owns gap candidates
+// j = g * waves .. of expert e, row offsets[e] + counts[e] + j while that is below offsets[e+1].
+// Every XCD takes one contiguous range of the copy work followed by one contiguous range of the
+// zero-fill work, so it gets its share of both.
+
+// How a token-order dispatch wavefront finds its destination row.
+enum DispatchLookup {
+    kLookupMetadata = 0,  // dst_slots -> recv_metadata row -> field k
+    kLookupTable = 1,     // token_slots[token][k]
+};
+
+// One zero-fill workgroup: each wavefront clears one whole gap row (and its weight).
+__device__ __forceinline__ void zero_fill_gap_rows(uint32_t block,
+                                                   uint32_t pad_per_expert,
+                                                   uint32_t pad_groups_per_expert,
+                                                   uint32_t chunks_per_block,
+                                                   uint32_t rows_per_block,
+                                                   const int64_t* __restrict__ expert_counts,
+                                                   const int64_t* __restrict__ expert_offsets,
+                                                   u32x4* __restrict__ recv_x,
+                                                   float* __restrict__ recv_weights,
+                                                   int64_t out_rows,
+                                                   int vectors) {
+    const uint32_t wave_y = __builtin_amdgcn_readfirstlane(threadIdx.y);
+    const uint32_t wave_z = __builtin_amdgcn_readfirstlane(threadIdx.z);
+    const uint32_t expert = block / pad_groups_per_expert;
+    const uint32_t group = block - expert * pad_groups_per_expert;
+    const uint32_t waves = chunks_per_block * rows_per_block;
+    const uint32_t j = group * waves + wave_z * chunks_per_block + wave_y;
+    if (j >= pad_per_expert)
+        return;
+    const int64_t out_row = uniform_load(expert_offsets + expert) + uniform_load(expert_counts + expert) + j;
+    if (out_row >= uniform_load(expert_offsets + expert + 1) || out_row >= out_rows)
+        return;
+    const u32x4 zero = {0u, 0u, 0u, 0u};
+    u32x4* dst = recv_x + out_row * vectors;
+    for (int vector = threadIdx.x; vector < vectors; vector += kWave)
+        store_vec<true>(dst + vector, zero);
+    if (threadIdx.x == 0 && recv_weights != nullptr)
+        recv_weights[out_row] = 0.0f;
+}
+
+template <int kLookup, bool kZeroFill>
+__global__ void __launch_bounds__(1024) dispatch_rows_kernel(const u32x4* __restrict__ x,                // [T][vectors]
+                                                             const float* __restrict__ weights,         // [T][K] or null
+                                                             const int32_t* __restrict__ recv_metadata,  // [N][K+2]
+                                                             const int64_t* __restrict__ dst_slots,     // [T]
+                                                             const int32_t* __restrict__ token_slots,   // [T][K] or null
+                                                             const int64_t* __restrict__ expert_counts,
+                                                             const int64_t* __restrict__ expert_offsets,
+                                                             u32x4* __restrict__ recv_x,                // [C or N][vectors]
+                                                             int64_t* __restrict__ recv_topk_idx,       // compact [N][K] or null
+                                                             float* __restrict__ recv_weights,          // [C] / [N][K] or null
+                                                             int64_t recv_count,
+                                                             int64_t out_rows,
+                                                             uint32_t copy_candidates,  // T*K expanded, T compact
+                                                             uint32_t copy_blocks,
+                                                             uint32_t copy_per_xcd,  // ceil(copy_blocks / 8)
+                                                             uint32_t pad_blocks,
+                                                             uint32_t pad_per_xcd,   // ceil(pad_blocks / 8)
+                                                             uint32_t parts,            // workgroups per candidate group (rows longer than 16 chunks)
+                                                             uint32_t parts_magic,      // fast divisor by parts
+                                                             uint32_t parts_shift,
+                                                             uint32_t chunks_per_block,  // == blockDim.y
+                                                             uint32_t rows_per_block,    // == blockDim.z
+                                                             uint32_t pad_per_expert,
+                                                             uint32_t pad_groups_per_expert,
+                                                             int vectors,
+                                                             int chunks,
+                                                             int num_topk,
+                                                             int topk_shift,  // log2(K) when K is a power of two, else -1
+                                                             int expand) {
+    NANOEP_FETCH_ARGS_4(x, weights, recv_x, recv_weights);
+    NANOEP_FETCH_ARGS_4(token_slots, copy_blocks, dst_slots, recv_metadata);
+    NANOEP_FETCH_ARGS_4(out_rows, recv_count, copy_candidates, copy_per_xcd);
+    NANOEP_FETCH_ARGS_4(parts_magic, parts_shift, vectors, chunks);
+    NANOEP_FETCH_ARGS_4(num_topk, topk_shift, expand, chunks_per_block);
+    // Workgroups are handed to the XCDs round-robin.  Each XCD takes one contiguous range of the
+    // copy work followed by one contiguous range of the zero-fill work, so neighbouring work items
+    // (which share their source rows) stay behind one L2 and every XCD gets its share of both.
+    // (kZeroFill is false when the launch has no zero-fill work: the copy path then carries none of
+    // its bookkeeping, which shows in a wavefront that lives about a microsecond)
+    const uint32_t xcd = blockIdx.x % kNumXcds;
+    const uint32_t index_in_xcd = blockIdx.x / kNumXcds;
+    const bool copy_work = !kZeroFill || index_in_xcd < copy_per_xcd;
+    uint32_t block = xcd * copy_per_xcd + index_in_xcd;
+    if (kZeroFill && !copy_work)
+        block = xcd * pad_per_xcd + (index_in_xcd - copy_per_xcd);
+    if (copy_work ? (index_in_xcd >= copy_per_xcd || block >= copy_blocks)
+                  : (index_in_xcd - copy_per_xcd >= pad_per_xcd || block >= pad_blocks))
+        return;
+    const int lane = threadIdx.x;
+    const uint32_t wave_y = __builtin_amdgcn_readfirstlane(threadIdx.y);
+    const uint32_t wave_z = __builtin_amdgcn_readfirstlane(threadIdx.z);
+
+    if (copy_work) {
+        const uint32_t group = fast_divide(block, parts_magic, parts_shift);
+        const uint32_t part = block - group * parts;
+        const uint32_t candidate = group * rows_per_block + wave_z;
+        const int chunk = static_cast<int>(part * chunks_per_block + wave_y);
+        if (candidate >= copy_candidates || chunk >= chunks)
+            return;
+        const int vector = chunk * kWave + lane;
+        const bool in_row = vector < vectors;
+        uint32_t token = candidate;
+        int k = 0;
+        int64_t out_row;
+        const int32_t* fields = nullptr;
+        if (expand) {
+            token = topk_shift >= 0 ? candidate >> topk_shift : candidate / static_cast<uint32_t>(num_topk);
+            k = static_cast<int>(candidate - token * num_topk);
+        }
+        token = __builtin_amdgcn_readfirstlane(token);
+        k = __builtin_amdgcn_readfirstlane(k);
+        // lanes past the end of a short row re-read vector 0 instead of branching around the load
+        const u32x4 data = x[static_cast<int64_t>(token) * vectors + (in_row ? vector : 0)];
+        if (kLookup == kLookupTable && expand) {
+            out_row = uniform_load(token_slots + static_cast<int64_t>(token) * num_topk + k);
+        } else {
+            const int64_t row = uniform_load(dst_slots + token);
+            if (row < 0 || row >= recv_count)
+                return;
+            fields = recv_metadata + row * (num_topk + 2);
+            out_row = expand ? static_cast<int64_t>(uniform_load(fields + 2 + k)) : row;
+        }
+        if (out_row < 0 || out_row >= out_rows)
+            return;
+        if (in_row)
+            store_vec<true>(recv_x + out_row * vectors + vector, data);
+        if (chunk != 0)
+            return;
+        if (expand) {
+            if (lane == 0 && recv_weights != nullptr)
+                recv_weights[out_row] = weights[static_cast<int64_t>(token) * num_topk + k];
+        } else if (lane < num_topk) {
+            if (recv_topk_idx != nullptr)
+                recv_topk_idx[out_row * num_topk + lane] = fields[2 + lane];
+            if (recv_weights != nullptr)
+                recv_weights[out_row * num_topk + lane] = weights[static_cast<int64_t>(token) * num_topk + lane];
+        }
+    } else {
+        zero_fill_gap_rows(block, pad_per_expert, pad_groups_per_expert, chunks_per_block, rows_per_block, expert_counts,
+                           expert_offsets, recv_x, recv_weights, out_rows, vectors);
+    }
+}
+
+// The slot-order walk, stripped to what its wavefronts need: a wavefront lives about a microsecond,
+// most of it waiting in a chain of scalar work -> list entry -> source load -> store, so every
+// scalar instruction and branch ahead of the source load is throughput.  Validity is folded into
+// one flag and the load is issued unconditionally (row 0 stands in).  kZeroFill is false when the
+// launch has no gap rows to clear: the copy path then carries none of that bookkeeping.
+template <bool kDeviceCount, bool kZeroFill>
+__global__ void __launch_bounds__(1024) dispatch_ordered_kernel(const u32x4* __restrict__ x,              // [T][vectors]
+                                                                const float* __restrict__ weights,       // [T][K] or null
+                                                                const int64_t* __restrict__ slot_order,  // [entries]
+                                                                const int64_t* __restrict__ live_count,  // device entry count (kDeviceCount)
+                                                                const int64_t* __restrict__ expert_counts,
+                                                                const int64_t* __restrict__ expert_offsets,
+                                                                u32x4* __restrict__ recv_x,        // [C][vectors]
+                                                                float* __restrict__ recv_weights,  // [C] or null
+                                                                uint32_t entries,
+                                                                uint32_t source_limit,  // T*K
+                                                                uint32_t out_rows,
+                                                                uint32_t copy_blocks,
+                                                                uint32_t copy_per_xcd,
+                                                                uint32_t pad_blocks,
+                                                                uint32_t pad_per_xcd,
+                                                                uint32_t pad_per_expert,
+                                                                uint32_t pad_groups_per_expert,
+                                                                uint32_t parts,
+                                                                uint32_t parts_magic,
+                                                                uint32_t parts_shift,
+                                                                uint32_t chunks_per_block,  // == blockDim.y
+                                                                uint32_t rows_per_block,    // == blockDim.z
+                                                                uint32_t vectors,
+                                                                uint32_t chunks,
+                                                                uint32_t topk_magic,  // fast divisor by K
+                                                                uint32_t topk_shift) {
+    NANOEP_FETCH_ARGS_4(x, weights, recv_x, recv_weights);
+    NANOEP_FETCH_ARGS_4(slot_order, entries, source_limit, out_rows);
+    NANOEP_FETCH_ARGS_4(copy_blocks, copy_per_xcd, parts, parts_magic);
+    NANOEP_FETCH_ARGS_4(parts_shift, chunks_per_block, rows_per_block, vectors);
+    NANOEP_FETCH_ARGS_4(chunks, topk_magic, topk_shift, live_count);
+    if (kDeviceCount) {
+        // The list length was not known when the grid was sized: shrink the walk to the entries in
+        // use, so that the per-XCD ranges split the real work and not its unused tail.
+        const int64_t live = uniform_load(live_count);
+        if (live >= 0 && live < static_cast<int64_t>(entries)) {
+            entries = static_cast<uint32_t>(live);
+            copy_blocks = (rows_per_block == 1 ? entries : (entries + rows_per_block - 1) / rows_per_block) * parts;
+            copy_per_xcd = (copy_blocks + kNumXcds - 1) / kNumXcds;
+        }
+    }
+    const uint32_t index_in_xcd = blockIdx.x / kNumXcds;
+    if (kZeroFill && index_in_xcd >= copy_per_xcd) {
+        const uint32_t pad_index = index_in_xcd - copy_per_xcd;
+        const uint32_t pad_block = (blockIdx.x % kNumXcds) * pad_per_xcd + pad_index;
+        if (pad_index < pad_per_xcd && pad_block < pad_blocks)
+            zero_fill_gap_rows(pad_block, pad_per_expert, pad_groups_per_expert, chunks_per_block, rows_per_block,
+                               expert_counts, expert_offsets, recv_x, recv_weights, out_rows, static_cast<int>(vectors));
+        return;
+    }
+    const uint32_t block = (blockIdx.x % kNumXcds) * copy_per_xcd + index_in_xcd;
+    if (index_in_xcd >= copy_per_xcd || block >= copy_blocks)
+        return;
+    const uint32_t group = fast_divide(block, parts_magic, parts_shift);
+    const uint32_t part = block - group * parts;
+    const uint32_t candidate = group * rows_per_block + __builtin_amdgcn_readfirstlane(threadIdx.z);
+    const uint32_t chunk = part * chunks_per_block + __builtin_amdgcn_readfirstlane(threadIdx.y);
+    if (candidate >= entries || chunk >= chunks)
+        return;
+    const int64_t entry = uniform_load(slot_order + candidate);
+    const uint32_t source = static_cast<uint32_t>(entry);
+    const uint32_t out_row = static_cast<uint32_t>(static_cast<uint64_t>(entry) >> 32);
+    const bool valid = entry >= 0 && source < source_limit && out_row < out_rows;
+    const uint32_t token = valid ? fast_divide(source, topk_magic, topk_shift) : 0u;
+    const uint32_t vector = chunk * kWave + threadIdx.x;
+    const bool in_row = vector < vectors;
+    const u32x4 data = x[static_cast<uint64_t>(token) * vectors + (in_row ? vector : 0u)];
+    if (!valid)
+        return;
+    if (in_row)
+        store_vec<true>(recv_x + static_cast<uint64_t>(out_row) * vectors + vector, data);
+    if (chunk == 0 && threadIdx.x == 0 && recv_weights != nullptr)
+        recv_weights[out_row] = weights[source];
+}
+
+// Compact layout: receive row r holds source token src_token(r), in token order, so the dispatch is
+// a row copy with holes.  Nothing is re-used, so workgroups walk the rows in plain launch order
+// (one linear stream over the whole device) and the kernel carries nothing but the copy.
+__global__ void __launch_bounds__(1024) dispatch_compact_kernel(const u32x4* __restrict__ x,                // [T][vectors]
+                                                                const float* __restrict__ weights,         // [T][K] or null
+                                                                const int32_t* __restrict__ recv_metadata,  // [N][K+2]
+                                                                const int64_t* __restrict__ dst_slots,     // [T]
+                                                                u32x4* __restrict__ recv_x,                // [N][vectors]
+                                                                int64_t* __restrict__ recv_topk_idx,       // [N][K] or null
+                                                                float* __restrict__ recv_weights,          // [N][K] or null
+                                                                uint32_t tokens,
+                                                                uint32_t recv_count,
+                                                                uint32_t parts,
+                                                                uint32_t parts_magic,
+                                                                uint32_t parts_shift,
+                                                                uint32_t chunks_per_block,  // == blockDim.y
+                                                                uint32_t rows_per_block,    // == blockDim.z
+                                                                uint32_t vectors,
+                                                                uint32_t chunks,
+                                                                uint32_t topk) {
+    NANOEP_FETCH_ARGS_4(x, dst_slots, recv_x, tokens);
+    NANOEP_FETCH_ARGS_4(recv_count, parts, parts_magic, parts_shift);
+    NANOEP_FETCH_ARGS_4(chunks_per_block, rows_per_block, vectors, chunks);
+    const uint32_t group = fast_divide(blockIdx.x, parts_magic, parts_shift);
+    const uint32_t part = blockIdx.x - group * parts;
+    const uint32_t token = group * rows_per_block + __builtin_amdgcn_readfirstlane(threadIdx.z);
+    const uint32_t chunk = part * chunks_per_block + __builtin_amdgcn_readfirstlane(threadIdx.y);
+    if (token >= tokens || chunk >= chunks)
+        return;
+    const uint32_t vector = chunk * kWave + threadIdx.x;
+    const bool in_row = vector < vectors;
+    // the source address depends on the block index alone: its load is in flight during the lookup
+    const u32x4 data = x[static_cast<uint64_t>(token) * vectors + (in_row ? vector : 0u)];
+    const int64_t row = uniform_load(dst_slots + token);
+    if (row < 0 || row >= static_cast<int64_t>(recv_count))
+        return;
+    if (in_row)
+        store_vec<true>(recv_x + static_cast<uint64_t>(row) * vectors + vector, data);
+    if (chunk == 0 && threadIdx.x < topk) {
+        const uint32_t lane = threadIdx.x;
+        if (recv_topk_idx != nullptr)
+            recv_topk_idx[row * topk + lane] = recv_metadata[row * (topk + 2) + 2 + lane];
+        if (recv_weights != nullptr)
+            recv_weights[row * topk + lane] = weights[static_cast<uint64_t>(token) * topk + lane];
+    }
+}
+
+
+}  // namespace
+}  // namespace nanoep
+
+using namespace nanoep;
+
+extern "C" {
+
+int nanoep_dispatch(const void* x, const float* weights, const int32_t* recv_metadata, const int64_t* dst_slots,
+                    const int32_t* token_slots, const int64_t* slot_order, int64_t slot_order_entries,
+                    const int64_t* expert_counts, const int64_t* expert_offsets,
+                    int64_t recv_count, int64_t expanded_capacity, int64_t num_tokens, int hidden, int num_topk,
+                    int64_t num_local_experts, int64_t alignment, int expand, int zero_padding, void* recv_x,
+                    int64_t* recv_topk_idx, float* recv_weights, int num_cus, void* stream_handle) {
+    if (hidden <= 0 || hidden % 8 != 0 || num_topk <= 0 || num_topk > kMaxTopk || num_local_experts <= 0 || alignment <= 0)
+        return NANOEP_ERR_INVALID_ARGUMENT;
+    if (recv_count < 0 || num_tokens < 0 || recv_count > num_tokens || num_tokens > INT32_MAX || expanded_capacity < 0 ||
+        expanded_capacity > INT32_MAX)
+        return NANOEP_ERR_INVALID_ARGUMENT;
+    if (expand && recv_topk_idx != nullptr)
+        return NANOEP_ERR_INVALID_ARGUMENT;
+    if (!aligned16(x) || !aligned16(recv_x))
+        return NANOEP_ERR_INVALID_ARGUMENT;
+    const int budget_status = validate_cu_budget(num_cus);
+    if (budget_status != NANOEP_OK)
+        return budget_status;
+    const int64_t out_rows = expand ? expanded_capacity : recv_count;
+    if (recv_count == 0 || out_rows == 0)
+        return NANOEP_OK;  // nothing was received: the outputs have no rows to write
+    if ((weights == nullptr) != (recv_weights == nullptr))
+        return NANOEP_ERR_INVALID_ARGUMENT;
+    if (x == nullptr || recv_metadata == nullptr || dst_slots == nullptr || recv_x == nullptr)
+        return NANOEP_ERR_INVALID_ARGUMENT;
+    const bool pad = expand && zero_padding && alignment > 1;
+    if (pad && (expert_counts == nullptr || expert_offsets == nullptr))
+        return NANOEP_ERR_INVALID_ARGUMENT;
+
+    // full list length without its trailing count word
+    const int64_t order_bound = nanoep_slot_order_entries(num_tokens, num_topk, num_local_experts) - 1;
+    // The walk pays off once every XCD has at least one whole token block of its own; below that
+    // the blocks' source rows would be fetched by several XCDs and the token-order walk is faster.
+    const int block_tokens = nanoep_layout_block_tokens(num_local_experts);
+    const int64_t token_blocks = block_tokens > 0 ? (num_tokens + block_tokens - 1) / block_tokens : 0;
+    const int order_switch = env_int("NANOEP_DISPATCH_ORDER", -1);  // 0 / 1 force the walk off / on
+    const bool ordered = expand && slot_order != nullptr && order_bound > 0 &&
+                         (order_switch < 0 ? token_blocks >= kNumXcds : order_switch != 0);
+    if (ordered && (slot_order_entries > order_bound || num_tokens * num_topk >= (int64_t{1} << 31)))
+        return NANOEP_ERR_INVALID_ARGUMENT;
+    // a negative entry count defers to the count word the layout stored behind the list
+    const int64_t* live_count = ordered && slot_order_entries < 0 ? slot_order + order_bound : nullptr;
+    if (live_count != nullptr)
+        slot_order_entries = order_bound;
+
+    const int vectors = hidden / 8;
+    const int chunks = (vectors + kWave - 1) / kWave;
+    const RowBlocking blocking = pick_row_blocking(chunks, ordered ? kSlotOrderWalk : expand ? kTokenOrderWalk : kRowCopyWalk);
+    const int64_t waves = static_cast<int64_t>(blocking.chunks_per_block) * blocking.rows_per_block;
+    const int64_t copy_candidates = ordered ? slot_order_entries : expand ? num_tokens * num_topk : num_tokens;
+    const int64_t copy_blocks = (copy_candidates + blocking.rows_per_block - 1) / blocking.rows_per_block * blocking.parts;
+    // No expert's gap exceeds alignment-1 rows, and all gaps together stay below C.
+    const int64_t pad_per_expert = !pad ? 0 : (alignment - 1 < expanded_capacity ? alignment - 1 : expanded_capacity);
+    const int64_t pad_groups_per_expert = (pad_per_expert + waves - 1) / waves;
+    const int64_t pad_blocks = num_local_experts * pad_groups_per_expert;
+    if (copy_candidates >= (int64_t{1} << 31) || copy_blocks + pad_blocks >= (int64_t{1} << 31) - 2 * kNumXcds)
+        return NANOEP_ERR_INVALID_ARGUMENT;
+    const uint32_t copy_per_xcd = static_cast<uint32_t>((copy_blocks + kNumXcds - 1) / kNumXcds);
+    const uint32_t pad_per_xcd = static_cast<uint32_t>((pad_blocks + kNumXcds - 1) / kNumXcds);
+    int topk_shift = -1;
+    if ((num_topk & (num_topk - 1)) == 0)
+        for (topk_shift = 0; (1 << topk_shift) < num_topk; ++topk_shift) {
+        }
+
+    const dim3 grid((copy_per_xcd + pad_per_xcd) * kNumXcds);
+    const dim3 block(kWave, blocking.chunks_per_block, blocking.rows_per_block);
+    const FastDivisor parts_divisor = make_fast_divisor(blocking.parts);
+    auto stream = static_cast<hipStream_t>(stream_handle);
+    if (ordered) {
+        const FastDivisor topk_divisor = make_fast_divisor(static_cast<uint32_t>(num_topk));
+#define NANOEP_LAUNCH_ORDERED(DEVICE_COUNT, ZERO_FILL)                                                                \
+    dispatch_ordered_kernel<DEVICE_COUNT, ZERO_FILL><<<grid, block, 0, stream>>>(                                    \
+        static_cast<const u32x4*>(x), weights, slot_order, live_count, expert_counts, expert_offsets,                \
+        static_cast<u32x4*>(recv_x), recv_weights, static_cast<uint32_t>(copy_candidates),                           \
+        static_cast<uint32_t>(num_tokens * num_topk), static_cast<uint32_t>(out_rows),                               \
+        static_cast<uint32_t>(copy_blocks), copy_per_xcd, static_cast<uint32_t>(pad_blocks), pad_per_xcd,            \
+        static_cast<uint32_t>(pad_per_expert),                                                                       \
+        static_cast<uint32_t>(pad_groups_per_expert > 0 ? pad_groups_per_expert : 1), blocking.parts,                \
+        parts_divisor.magic, parts_divisor.shift, blocking.chunks_per_block, blocking.rows_per_block,                \
+        static_cast<uint32_t>(vectors), static_cast<uint32_t>(chunks), topk_divisor.magic, topk_divisor.shift)
+        if (live_count != nullptr && pad_blocks > 0)
+            NANOEP_LAUNCH_ORDERED(true, true);
+        else if (live_count != nullptr)
+            NANOEP_LAUNCH_ORDERED(true, false);
+        else if (pad_blocks > 0)
+            NANOEP_LAUNCH_ORDERED(false, true);
+        else
+            NANOEP_LAUNCH_ORDERED(false, false);
+#undef NANOEP_LAUNCH_ORDERED
+    } else if (!expand) {
+        const int64_t blocks = (num_tokens + blocking.rows_per_block - 1) / blocking.rows_per_block * blocking.parts;
+        dispatch_compact_kernel<<<dim3(static_cast<unsigned>(blocks)), block, 0, stream>>>(
+            static_cast<const u32x4*>(x), weights, recv_metadata, dst_slots, static_cast<u32x4*>(recv_x), recv_topk_idx,
+            recv_weights, static_cast<uint32_t>(num_tokens), static_cast<uint32_t>(recv_count), blocking.parts,
+            parts_divisor.magic, parts_divisor.shift, blocking.chunks_per_block, blocking.rows_per_block,
+            static_cast<uint32_t>(vectors), static_cast<uint32_t>(chunks), static_cast<uint32_t>(num_topk));
+    } else {
+#define NANOEP_LAUNCH_ROWS(LOOKUP, ZERO_FILL)                                                                         \
+    dispatch_rows_kernel<LOOKUP, ZERO_FILL><<<grid, block, 0, stream>>>(                                             \
+        static_cast<const u32x4*>(x), weights, recv_metadata, dst_slots, token_slots, expert_counts, expert_offsets, \
+        static_cast<u32x4*>(recv_x), recv_topk_idx, recv_weights, recv_count, out_rows,                              \
+        static_cast<uint32_t>(copy_candidates), static_cast<uint32_t>(copy_blocks), copy_per_xcd,                    \
+        static_cast<uint32_t>(pad_blocks), pad_per_xcd, blocking.parts, parts_divisor.magic, parts_divisor.shift,    \
+        blocking.chunks_per_block, blocking.rows_per_block, static_cast<uint32_t>(pad_per_expert),                   \
+        static_cast<uint32_t>(pad_groups_per_expert > 0 ? pad_groups_per_expert : 1), vectors, chunks, num_topk,     \
+        topk_shift, expand ? 1 : 0)
+        const bool table = token_slots != nullptr && expand;
+        if (table && pad_blocks > 0)
+            NANOEP_LAUNCH_ROWS(kLookupTable, true);
+        else if (table)
+            NANOEP_LAUNCH_ROWS(kLookupTable, false);
+        else if (pad_blocks > 0)
+            NANOEP_LAUNCH_ROWS(kLookupMetadata, true);
+        else
+            NANOEP_LAUNCH_ROWS(kLookupMetadata, false);
+#undef NANOEP_LAUNCH_ROWS
+    }
+    NANOEP_HIP_TRY(hipGetLastError());
+    return NANOEP_OK;
+}
+
+}  // extern "C"

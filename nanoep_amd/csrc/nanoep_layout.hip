@@ -1,0 +1,759 @@
+// Routing layout: per-expert histograms, device-wide scan, stable token-order slots, slot-order list.
+
+#include <ctime>
+
+#include "nanoep_device.h"
+
+namespace nanoep {
+namespace {
+
+// Tokens handled by one layout workgroup: the LDS bit matrix has (L+1) rows of tokens/32 words
+// plus a 16-bit prefix per word, so the block shrinks as the expert count grows.
+int layout_tokens_per_block(int64_t local_experts) {
+    if (static_cast<size_t>(local_experts + 1) * 12 > kLayoutLdsBudget)  // three int32 arrays of the assignment kernel
+        return 0;
+    for (int tokens = 256; tokens >= 32; tokens /= 2) {
+        const size_t words = static_cast<size_t>(tokens / 32);
+        if (static_cast<size_t>(local_experts + 1) * (words * 6 + 4) <= kLayoutLdsBudget)
+            return tokens;
+    }
+    return 0;
+}
+
+struct LayoutWorkspace {
+    int32_t* block_counts;  // [NB][L+1]; column L counts tokens with any valid choice
+    int32_t* block_status;  // [NB]
+    int32_t* packed_rank;   // [T][K]  (expert << 8) | in-block rank, or -1
+    int32_t* local_row;     // [T]
+    int64_t* totals;        // [1] total assignments, handed from the scan kernel to the assignment kernel
+    size_t bytes;
+};
+
+LayoutWorkspace carve_layout_workspace(void* base, int64_t tokens, int topk, int64_t local_experts) {
+    const int per_block = layout_tokens_per_block(local_experts);
+    const int64_t blocks = per_block == 0 ? 0 : (tokens + per_block - 1) / per_block;
+    auto* cursor = static_cast<uint8_t*>(base);
+    size_t offset = 0;
+    LayoutWorkspace ws{};
+    ws.block_counts = reinterpret_cast<int32_t*>(cursor + offset);
+    offset = align_up(offset + static_cast<size_t>(blocks) * (local_experts + 1) * 4, 256);
+    ws.block_status = reinterpret_cast<int32_t*>(cursor + offset);
+    offset = align_up(offset + static_cast<size_t>(blocks) * 4, 256);
+    ws.packed_rank = reinterpret_cast<int32_t*>(cursor + offset);
+    offset = align_up(offset + static_cast<size_t>(tokens) * topk * 4, 256);
+    ws.local_row = reinterpret_cast<int32_t*>(cursor + offset);
+    offset = align_up(offset + static_cast<size_t>(tokens) * 4, 256);
+    ws.totals = reinterpret_cast<int64_t*>(cursor + offset);
+    offset = align_up(offset + 8, 256);
+    ws.bytes = offset + 256;
+    return ws;
+}
+
+// A (token, k) entry of the rank table packs (expert << kRankBits) | in-block rank; -1 marks a
+// masked choice.  A layout block never holds more than 256 tokens, so the rank fits 8 bits.
+constexpr int kRankBits = 8;
+constexpr int kRankMask = (1 << kRankBits) - 1;
+
+// One thread per token.  bits[e][w] has bit (token & 31) of word (token >> 5) set when the token
+// chose expert e; row L marks tokens with any valid choice.  Experts inside a token are distinct,
+// so the order of one expert's assignments is the token order and a popcount prefix is the rank.
+// The token's routing ids are fetched in one batch of independent loads (kCap >= K of them, the
+// surplus re-reads id 0) and stay in registers for both passes over the bit matrix.
+template <int kCap>
+__device__ __forceinline__ void layout_count_block(const int64_t* __restrict__ topk_idx,
+                                                   int64_t num_tokens,
+                                                   int num_topk,
+                                                   int local_experts,
+                                                   int words,
+                                                   int threads,
+                                                   int64_t* __restrict__ snapshot,
+                                                   int32_t* block_counts,
+                                                   int32_t* block_status,
+                                                   int32_t* packed_rank,
+                                                   int32_t* local_row) {
+    extern __shared__ uint32_t layout_lds[];
+    const int rows = local_experts + 1;
+    // bit rows are words + 1 apart: an odd stride spreads the experts a wavefront touches over the LDS banks
+    const int stride = words + 1;
+    uint32_t* bits = layout_lds;
+    auto* prefix = reinterpret_cast<uint16_t*>(bits + static_cast<size_t>(rows) * stride);
+    __shared__ int block_bad;
+
+    const int tokens_per_block = words * 32;
+    const int local_token = threadIdx.x;
+    const int64_t token = static_cast<int64_t>(blockIdx.x) * tokens_per_block + local_token;
+    const bool live = local_token < tokens_per_block && token < num_tokens;
+    const int word = local_token >> 5;
+    const uint32_t bit = 1u << (local_token & 31);
+
+    int64_t raw[kCap];
+    const int64_t* mine = topk_idx + (live ? token : 0) * num_topk;
+#pragma unroll
+    for (int k = 0; k < kCap; ++k)
+        raw[k] = mine[k < num_topk ? k : 0];
+
+    for (int i = threadIdx.x; i < rows * stride; i += threads)
+        bits[i] = 0;
+    if (threadIdx.x == 0)
+        block_bad = 0;
+    __syncthreads();
+
+    int ids[kCap];  // expert id, -1 masked, -2 out of range
+#pragma unroll
+    for (int k = 0; k < kCap; ++k) {
+        const int64_t expert = raw[k];
+        ids[k] = (expert >= 0 && expert < local_experts) ? static_cast<int>(expert) : (expert == -1 ? -1 : -2);
+        if (!live || k >= num_topk)
+            ids[k] = -1;
+        else
+            snapshot[token * num_topk + k] = expert;
+    }
+
+    int bad = 0;
+    bool any = false;
+#pragma unroll
+    for (int k = 0; k < kCap; ++k) {
+        const int id = ids[k];
+        if (id >= 0) {
+            const uint32_t old = atomicOr(&bits[static_cast<size_t>(id) * stride + word], bit);
+            if (old & bit)
+                bad |= NANOEP_ROUTING_DUPLICATE;
+            any = true;
+        } else if (id == -2) {
+            bad |= NANOEP_ROUTING_BAD_EXPERT;
+        }
+    }
+    if (any)
+        atomicOr(&bits[static_cast<size_t>(local_experts) * stride + word], bit);
+    if (bad)
+        atomicOr(&block_bad, bad);
+    __syncthreads();
+
+    for (int row = threadIdx.x; row < rows; row += threads) {
+        int running = 0;
+        for (int w = 0; w < words; ++w) {
+            prefix[static_cast<size_t>(row) * words + w] = static_cast<uint16_t>(running);
+            running += __popc(bits[static_cast<size_t>(row) * stride + w]);
+        }
+        block_counts[static_cast<int64_t>(blockIdx.x) * rows + row] = running;
+    }
+    if (threadIdx.x == 0)
+        block_status[blockIdx.x] = block_bad;
+    __syncthreads();
+
+    if (live) {
+        const uint32_t below = bit - 1;
+#pragma unroll
+        for (int k = 0; k < kCap; ++k) {
+            const int id = ids[k];
+            int32_t packed = -1;
+            if (id >= 0) {
+                const int rank = prefix[static_cast<size_t>(id) * words + word] +
+                                 __popc(bits[static_cast<size_t>(id) * stride + word] & below);
+                packed = (id << kRankBits) | rank;
+            }
+            if (k < num_topk)
+                packed_rank[token * num_topk + k] = packed;
+        }
+        const uint32_t received = bits[static_cast<size_t>(local_experts) * stride + word];
+        local_row[token] = (received & bit) ? prefix[static_cast<size_t>(local_experts) * words + word] + __popc(received & below) : -1;
+    }
+}
+
+template <int kCap>
+__global__ void __launch_bounds__(256) layout_count_kernel(const int64_t* __restrict__ topk_idx,
+                                                           int64_t num_tokens,
+                                                           int num_topk,
+                                                           int local_experts,
+                                                           int words,
+                                                           int threads,
+                                                           int64_t* __restrict__ snapshot,
+                                                           int32_t* __restrict__ block_counts,
+                                                           int32_t* __restrict__ block_status,
+                                                           int32_t* __restrict__ packed_rank,
+                                                           int32_t* __restrict__ local_row) {
+    layout_count_block<kCap>(topk_idx, num_tokens, num_topk, local_experts, words, threads, snapshot, block_counts,
+                             block_status, packed_rank, local_row);
+}
+
+__device__ __forceinline__ int64_t round_up_to(int64_t value, int64_t alignment) {
+    return alignment == 1 ? value : (value + alignment - 1) / alignment * alignment;
+}
+
+// Single workgroup.  Phase 1 turns every column of block_counts into its exclusive prefix over
+// blocks (threads are spread over columns x block segments so small expert counts still use the
+// whole workgroup).  Phase 2 scans the aligned expert totals.  The mailbox word 0 is stored last.
+__global__ void __launch_bounds__(kScanThreads) layout_scan_kernel(int32_t* __restrict__ block_counts,
+                                                                  const int32_t* __restrict__ block_status,
+                                                                  int num_blocks,
+                                                                  int local_experts,
+                                                                  int64_t alignment,
+                                                                  int64_t* __restrict__ expert_counts,
+                                                                  int64_t* __restrict__ expert_offsets,
+                                                                  int64_t* __restrict__ send_counts,
+                                                                  int64_t* __restrict__ recv_rank_prefix,
+                                                                  int64_t* __restrict__ totals,
+                                                                  int64_t* host_counts) {
+    extern __shared__ int32_t column_total[];  // [L+1]
+    __shared__ int32_t partial[kScanThreads];
+    __shared__ int64_t scan[kScanThreads];
+    __shared__ int64_t assignments[kScanThreads];
+    __shared__ int status_bits;
+
+    const int tid = threadIdx.x;
+    const int rows = local_experts + 1;
+    if (tid == 0)
+        status_bits = 0;
+
+    const int columns_per_pass = rows < kScanThreads ? rows : kScanThreads;
+    const int segments = kScanThreads / columns_per_pass;
+    const int blocks_per_segment = (num_blocks + segments - 1) / segments;
+    for (int column0 = 0; column0 < rows; column0 += columns_per_pass) {
+        const int column_local = tid % columns_per_pass;
+        const int segment = tid / columns_per_pass;
+        const int column = column0 + column_local;
+        const bool active = segment < segments && column < rows;
+        const int begin = segment * blocks_per_segment;
+        const int end = begin + blocks_per_segment < num_blocks ? begin + blocks_per_segment : num_blocks;
+        int sum = 0;
+        if (active)
+            for (int b = begin; b < end; ++b)
+                sum += block_counts[static_cast<int64_t>(b) * rows + column];
+        partial[tid] = active ? sum : 0;
+        __syncthreads();
+        if (active) {
+            int running = 0;
+            for (int s = 0; s < segment; ++s)
+                running += partial[s * columns_per_pass + column_local];
+            for (int b = begin; b < end; ++b) {
+                const int64_t at = static_cast<int64_t>(b) * rows + column;
+                const int count = block_counts[at];
+                block_counts[at] = running;
+                running += count;
+            }
+            if (segment == segments - 1)
+                column_total[column] = running;
+        }
+        __syncthreads();
+    }
+
+    int bad = 0;
+    for (int b = tid; b < num_blocks; b += kScanThreads)
+        bad |= block_status[b];
+    if (bad)
+        atomicOr(&status_bits, bad);
+
+    const int per_thread = (local_experts + kScanThreads - 1) / kScanThreads;
+    const int first = tid * per_thread;
+    const int last = first + per_thread < local_experts ? first + per_thread : local_experts;
+    int64_t padded_sum = 0, count_sum = 0;
+    for (int e = first; e < last; ++e) {
+        const int64_t count = column_total[e];
+        count_sum += count;
+        padded_sum += round_up_to(count, alignment);
+    }
+    scan[tid] = padded_sum;
+    assignments[tid] = count_sum;
+    __syncthreads();
+    for (int step = 1; step < kScanThreads; step *= 2) {
+        const int64_t add_scan = tid >= step ? scan[tid - step] : 0;
+        const int64_t add_assign = tid >= step ? assignments[tid - step] : 0;
+        __syncthreads();
+        scan[tid] += add_scan;
+        assignments[tid] += add_assign;
+        __syncthreads();
+    }
+    int64_t running = scan[tid] - padded_sum;
+    for (int e = first; e < last; ++e) {
+        const int64_t count = column_total[e];
+        expert_counts[e] = count;
+        expert_offsets[e] = running;
+        running += round_up_to(count, alignment);
+    }
+    if (tid == 0) {
+        const int64_t received = column_total[local_experts];
+        const int64_t capacity = scan[kScanThreads - 1];
+        expert_offsets[local_experts] = capacity;
+        send_counts[0] = received;
+        recv_rank_prefix[0] = received;
+        totals[0] = assignments[kScanThreads - 1];
+        host_counts[1] = capacity;
+        host_counts[2] = assignments[kScanThreads - 1];
+        host_counts[3] = status_bits;
+        __threadfence_system();
+        __hip_atomic_store(&host_counts[0], received, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_SYSTEM);
+    }
+}
+
+// Writes one token's part of the handle.  `slot_base[e]` is the first slot of this block's
+// assignments to expert e; `order_base[e]` is where expert e's run starts in the block's segment
+// of the slot-order list (`order` points at that segment, or is null).
+template <int kCap>
+__device__ __forceinline__ void assign_token_slots(int64_t token,
+                                                   int num_topk,
+                                                   int expand,
+                                                   int row_in_block,
+                                                   int64_t row_base,
+                                                   const int32_t* slot_base,
+                                                   const int32_t* order_base,
+                                                   const int32_t* __restrict__ packed_rank,
+                                                   int32_t* __restrict__ recv_metadata,
+                                                   int64_t* __restrict__ dst_slots,
+                                                   int32_t* __restrict__ token_slots,
+                                                   int64_t* __restrict__ order) {
+    int32_t packed[kCap];
+#pragma unroll
+    for (int k = 0; k < kCap; ++k)
+        packed[k] = packed_rank[token * num_topk + (k < num_topk ? k : 0)];
+    if (row_in_block < 0) {
+        dst_slots[token] = -1;
+        if (token_slots != nullptr)
+            for (int k = 0; k < num_topk; ++k)
+                token_slots[token * num_topk + k] = -1;
+        return;
+    }
+    const int64_t row = row_base + row_in_block;
+    dst_slots[token] = row;
+    int32_t* out = recv_metadata + row * (num_topk + 2);
+    out[0] = 0;
+    out[1] = static_cast<int32_t>(token);
+#pragma unroll
+    for (int k = 0; k < kCap; ++k) {
+        if (k >= num_topk)
+            break;
+        int32_t value = -1;
+        if (packed[k] >= 0) {
+            const int expert = packed[k] >> kRankBits;
+            const int rank = packed[k] & kRankMask;
+            value = expand ? slot_base[expert] + rank : expert;
+            if (order != nullptr) {
+                const uint32_t source = static_cast<uint32_t>(token * num_topk + k);
+                order[order_base[expert] + rank] = (static_cast<int64_t>(value) << 32) | source;
+            }
+        }
+        out[2 + k] = value;
+        if (token_slots != nullptr)
+            token_slots[token * num_topk + k] = value;
+    }
+}
+
+__device__ __forceinline__ int64_t wave_inclusive_scan(int64_t value) {
+    const int lane = threadIdx.x & (kWave - 1);
+#pragma unroll
+    for (int distance = 1; distance < kWave; distance *= 2) {
+        const int64_t other = __shfl_up(value, distance, kWave);
+        if (lane >= distance)
+            value += other;
+    }
+    return value;
+}
+
+// Slot assignment, one workgroup per block of tokens (the blocks of layout_count_kernel).
+//
+// kFusedScan: `block_counts` holds the raw block histograms and every workgroup sums them itself
+// (they sit in L2): per column the total over all blocks and the part from the blocks before its
+// own, then the aligned exclusive scan over experts, all in LDS; workgroup 0 also writes the
+// per-expert outputs and the host mailbox (word 0 last).  Otherwise layout_scan_kernel has done
+// that and `block_counts` holds each block's exclusive prefixes.
+//
+// Either way the workgroup also scans its own histogram over experts: that places every
+// assignment of the block in expert-major order inside the block's run of `slot_order`; the runs
+// of consecutive blocks follow each other without gaps and the unused tail of the list is -1.
+template <int kCap, bool kFusedScan>
+__device__ __forceinline__ void layout_assign_block(const int32_t* block_counts,
+                                                    const int32_t* block_status,
+                                                    int num_blocks,
+                                                    int64_t num_tokens,
+                                                    int num_topk,
+                                                    int local_experts,
+                                                    int tokens_per_block,
+                                                    int threads,
+                                                    int expand,
+                                                    int64_t alignment,
+                                                    const int32_t* packed_rank,
+                                                    const int32_t* local_row,
+                                                    int64_t* expert_counts,
+                                                    int64_t* expert_offsets,
+                                                    int64_t* send_counts,
+                                                    int64_t* __restrict__ recv_rank_prefix,
+                                                    const int64_t* totals,
+                                                    int64_t* host_counts,
+                                                    int32_t* __restrict__ recv_metadata,
+                                                    int64_t* __restrict__ dst_slots,
+                                                    int32_t* __restrict__ token_slots,
+                                                    int64_t* __restrict__ slot_order) {
+    extern __shared__ int32_t assign_lds[];
+    __shared__ int64_t wave_padded[kWavesPerBlock];
+    __shared__ int64_t wave_assigned[kWavesPerBlock];
+    __shared__ int32_t wave_own[kWavesPerBlock];
+    __shared__ int32_t wave_before[kWavesPerBlock];
+    __shared__ int status_bits;
+    const int rows = local_experts + 1;
+    int32_t* column_total = assign_lds;         // [L+1] totals over all blocks (fused scan only)
+    int32_t* slot_base = assign_lds + rows;     // [L+1] assignments before this block -> first slot per expert
+    int32_t* order_base = assign_lds + 2 * rows;  // [L+1] this block's histogram -> its exclusive scan
+
+    const int tid = threadIdx.x;
+    const int block = blockIdx.x;
+    const int64_t token = static_cast<int64_t>(block) * tokens_per_block + tid;
+    const bool live = tid < tokens_per_block && token < num_tokens;
+    const int row_in_block = live ? local_row[token] : -1;
+
+    if (kFusedScan) {
+        for (int i = tid; i < 2 * rows; i += threads)
+            assign_lds[i] = 0;
+        if (tid == 0)
+            status_bits = 0;
+        __syncthreads();
+
+        const int columns_per_pass = rows < threads ? rows : threads;
+        const int segments = threads / columns_per_pass;
+        const int blocks_per_segment = (num_blocks + segments - 1) / segments;
+        const int column_local = tid % columns_per_pass;
+        const int segment = tid / columns_per_pass;
+        const int begin = segment * blocks_per_segment;
+        const int end = begin + blocks_per_segment < num_blocks ? begin + blocks_per_segment : num_blocks;
+        for (int column0 = 0; column0 < rows; column0 += columns_per_pass) {
+            const int column = column0 + column_local;
+            if (segment < segments && column < rows) {
+                int total = 0, before = 0, own = 0;
+#pragma unroll 8
+                for (int b = begin; b < end; ++b) {
+                    const int count = block_counts[static_cast<int64_t>(b) * rows + column];
+                    total += count;
+                    before += b < block ? count : 0;
+                    own = b == block ? count : own;
+                }
+                if (segments == 1) {
+                    column_total[column] = total;
+                    slot_base[column] = before;
+                } else {
+                    atomicAdd(&column_total[column], total);
+                    atomicAdd(&slot_base[column], before);
+                }
+                if (block >= begin && block < end)
+                    order_base[column] = own;
+            }
+        }
+        if (block == 0) {
+            int bad = 0;
+            for (int b = tid; b < num_blocks; b += threads)
+                bad |= block_status[b];
+            if (bad)
+                atomicOr(&status_bits, bad);
+        }
+    } else {
+        const int32_t* mine = block_counts + static_cast<int64_t>(block) * rows;
+        const bool last_block = block + 1 >= num_blocks;
+        for (int column = tid; column < rows; column += threads) {
+            const int32_t before = mine[column];
+            int32_t next;
+            if (!last_block)
+                next = mine[rows + column];
+            else
+                next = static_cast<int32_t>(column < local_experts ? expert_counts[column] : send_counts[0]);
+            order_base[column] = next - before;
+            slot_base[column] = before;
+        }
+    }
+    __syncthreads();
+
+    const int per_thread = (local_experts + threads - 1) / threads;
+    const int first = tid * per_thread < local_experts ? tid * per_thread : local_experts;
+    const int last = first + per_thread < local_experts ? first + per_thread : local_experts;
+    int64_t padded_sum = 0, count_sum = 0;
+    int own_sum = 0, before_sum = 0;
+    for (int e = first; e < last; ++e) {
+        if (kFusedScan) {
+            const int64_t count = column_total[e];
+            count_sum += count;
+            padded_sum += round_up_to(count, alignment);
+        }
+        own_sum += order_base[e];
+        before_sum += slot_base[e];
+    }
+    const int64_t padded_scan = kFusedScan ? wave_inclusive_scan(padded_sum) : 0;
+    const int64_t assigned_scan = kFusedScan ? wave_inclusive_scan(count_sum) : 0;
+    const int own_scan = static_cast<int>(wave_inclusive_scan(own_sum));
+    const int before_scan = static_cast<int>(wave_inclusive_scan(before_sum));
+    const int wave = tid / kWave;
+    const int waves = threads / kWave;
+    if ((tid & (kWave - 1)) == kWave - 1) {
+        wave_padded[wave] = padded_scan;
+        wave_assigned[wave] = assigned_scan;
+        wave_own[wave] = own_scan;
+        wave_before[wave] = before_scan;
+    }
+    __syncthreads();
+    int64_t running = padded_scan - padded_sum;
+    int running_own = own_scan - own_sum;
+    int64_t capacity = 0, assigned = 0;
+    int own_total = 0, assigned_before = 0;  // this block's assignments, and those of the blocks before it
+    for (int w = 0; w < waves; ++w) {
+        running += w < wave ? wave_padded[w] : 0;
+        running_own += w < wave ? wave_own[w] : 0;
+        capacity += wave_padded[w];
+        assigned += wave_assigned[w];
+        own_total += wave_own[w];
+        assigned_before += wave_before[w];
+    }
+    if (!kFusedScan)
+        assigned = totals[0];
+    for (int e = first; e < last; ++e) {
+        if (kFusedScan) {
+            const int64_t count = column_total[e];
+            if (block == 0) {
+                expert_counts[e] = count;
+                expert_offsets[e] = running;
+            }
+            slot_base[e] += static_cast<int32_t>(running);
+            running += round_up_to(count, alignment);
+        } else {
+            slot_base[e] += static_cast<int32_t>(expert_offsets[e]);
+        }
+        const int own = order_base[e];
+        order_base[e] = running_own;
+        running_own += own;
+    }
+    if (kFusedScan && block == 0 && tid == 0) {
+        const int64_t received = column_total[local_experts];
+        expert_offsets[local_experts] = capacity;
+        send_counts[0] = received;
+        recv_rank_prefix[0] = received;
+        host_counts[1] = capacity;
+        host_counts[2] = assigned;
+        host_counts[3] = status_bits;
+        __threadfence_system();
+        __hip_atomic_store(&host_counts[0], received, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_SYSTEM);
+    }
+    __syncthreads();
+    // The list is dense: this block's run starts where the earlier blocks' assignments end.  Every
+    // block also clears as many entries of the unused tail [A, entries) as it has masked choices.
+    int64_t* order = nullptr;
+    if (slot_order != nullptr) {
+        order = slot_order + assigned_before;
+        const int64_t block_entries = static_cast<int64_t>(tokens_per_block) * num_topk;
+        int64_t* tail = slot_order + assigned + (block * block_entries - assigned_before);
+        const int holes = static_cast<int>(block_entries) - own_total;
+        for (int i = tid; i < holes; i += threads)
+            tail[i] = -1;
+        if (block == 0 && tid == 0)
+            slot_order[num_blocks * block_entries] = assigned;  // count word behind the list
+    }
+    if (live)
+        assign_token_slots<kCap>(token, num_topk, expand, row_in_block, slot_base[local_experts], slot_base, order_base,
+                                 packed_rank, recv_metadata, dst_slots, token_slots, order);
+}
+
+template <int kCap, bool kFusedScan>
+__global__ void __launch_bounds__(256) layout_assign_kernel(const int32_t* __restrict__ block_counts,
+                                                            const int32_t* __restrict__ block_status,
+                                                            int num_blocks,
+                                                            int64_t num_tokens,
+                                                            int num_topk,
+                                                            int local_experts,
+                                                            int tokens_per_block,
+                                                            int threads,
+                                                            int expand,
+                                                            int64_t alignment,
+                                                            const int32_t* __restrict__ packed_rank,
+                                                            const int32_t* __restrict__ local_row,
+                                                            int64_t* expert_counts,
+                                                            int64_t* expert_offsets,
+                                                            int64_t* send_counts,
+                                                            int64_t* recv_rank_prefix,
+                                                            const int64_t* __restrict__ totals,
+                                                            int64_t* host_counts,
+                                                            int32_t* recv_metadata,
+                                                            int64_t* dst_slots,
+                                                            int32_t* token_slots,
+                                                            int64_t* slot_order) {
+    layout_assign_block<kCap, kFusedScan>(block_counts, block_status, num_blocks, num_tokens, num_topk, local_experts,
+                                          tokens_per_block, threads, expand, alignment, packed_rank, local_row, expert_counts,
+                                          expert_offsets, send_counts, recv_rank_prefix, totals, host_counts, recv_metadata,
+                                          dst_slots, token_slots, slot_order);
+}
+
+// Whole layout in one launch when all tokens fit one block: the count pass, then (its results are
+// this workgroup's own global writes, made visible by the fence and the barrier) the assignment pass.
+template <int kCap>
+__global__ void __launch_bounds__(256) layout_single_block_kernel(const int64_t* topk_idx,
+                                                                  int64_t num_tokens,
+                                                                  int num_topk,
+                                                                  int local_experts,
+                                                                  int words,
+                                                                  int threads,
+                                                                  int expand,
+                                                                  int64_t alignment,
+                                                                  int64_t* snapshot,
+                                                                  int32_t* block_counts,
+                                                                  int32_t* block_status,
+                                                                  int32_t* packed_rank,
+                                                                  int32_t* local_row,
+                                                                  int64_t* expert_counts,
+                                                                  int64_t* expert_offsets,
+                                                                  int64_t* send_counts,
+                                                                  int64_t* recv_rank_prefix,
+                                                                  int64_t* host_counts,
+                                                                  int32_t* recv_metadata,
+                                                                  int64_t* dst_slots,
+                                                                  int32_t* token_slots,
+                                                                  int64_t* slot_order) {
+    layout_count_block<kCap>(topk_idx, num_tokens, num_topk, local_experts, words, threads, snapshot, block_counts,
+                             block_status, packed_rank, local_row);
+    __threadfence();
+    __syncthreads();
+    layout_assign_block<kCap, true>(block_counts, block_status, 1, num_tokens, num_topk, local_experts, words * 32, threads,
+                                    expand, alignment, packed_rank, local_row, expert_counts, expert_offsets, send_counts,
+                                    recv_rank_prefix, nullptr, host_counts, recv_metadata, dst_slots, token_slots, slot_order);
+}
+
+
+}  // namespace
+}  // namespace nanoep
+
+using namespace nanoep;
+
+extern "C" {
+
+size_t nanoep_layout_workspace_bytes(int64_t num_tokens, int num_topk, int64_t num_local_experts) {
+    if (num_tokens < 0 || num_topk <= 0 || num_local_experts <= 0)
+        return 0;
+    return carve_layout_workspace(nullptr, num_tokens, num_topk, num_local_experts).bytes;
+}
+
+int nanoep_layout_block_tokens(int64_t num_local_experts) {
+    return num_local_experts <= 0 ? 0 : layout_tokens_per_block(num_local_experts);
+}
+
+int64_t nanoep_slot_order_entries(int64_t num_tokens, int num_topk, int64_t num_local_experts) {
+    if (num_tokens < 0 || num_topk <= 0 || num_local_experts <= 0)
+        return 0;
+    const int per_block = layout_tokens_per_block(num_local_experts);
+    if (per_block == 0 || num_tokens == 0)
+        return 0;
+    return (num_tokens + per_block - 1) / per_block * per_block * num_topk + 1;
+}
+
+int nanoep_layout(const int64_t* topk_idx, int64_t num_tokens, int num_topk, int64_t num_local_experts,
+                  int64_t alignment, int expand, int32_t* recv_metadata, int64_t* expert_counts,
+                  int64_t* expert_offsets, int64_t* dst_slots, int64_t* send_counts, int64_t* topk_snapshot,
+                  int64_t* recv_rank_prefix, int32_t* token_slots, int64_t* slot_order, void* workspace,
+                  size_t workspace_bytes, int64_t* host_counts, void* stream_handle) {
+    if (num_tokens < 0 || num_tokens > INT32_MAX || num_topk <= 0 || num_topk > kMaxTopk || num_local_experts <= 0 ||
+        num_local_experts >= (int64_t{1} << (31 - kRankBits)) || alignment <= 0 || alignment > (int64_t{1} << 31))
+        return NANOEP_ERR_INVALID_ARGUMENT;
+    if (expert_counts == nullptr || expert_offsets == nullptr || send_counts == nullptr || recv_rank_prefix == nullptr ||
+        host_counts == nullptr || workspace == nullptr)
+        return NANOEP_ERR_INVALID_ARGUMENT;
+    if (num_tokens > 0 && (topk_idx == nullptr || recv_metadata == nullptr || dst_slots == nullptr || topk_snapshot == nullptr))
+        return NANOEP_ERR_INVALID_ARGUMENT;
+    // the slot-order list packs token * K + k into 32 bits and only exists for the expanded layout
+    if (slot_order != nullptr && (!expand || num_tokens * num_topk >= (int64_t{1} << 31)))
+        return NANOEP_ERR_INVALID_ARGUMENT;
+    const int tokens_per_block = layout_tokens_per_block(num_local_experts);
+    if (tokens_per_block == 0)
+        return NANOEP_ERR_INVALID_ARGUMENT;
+    const LayoutWorkspace ws = carve_layout_workspace(workspace, num_tokens, num_topk, num_local_experts);
+    if (ws.bytes > workspace_bytes)
+        return NANOEP_ERR_WORKSPACE;
+    const int64_t blocks64 = (num_tokens + tokens_per_block - 1) / tokens_per_block;
+    const int blocks = static_cast<int>(blocks64);
+    const int experts = static_cast<int>(num_local_experts);
+    const int words = tokens_per_block / 32;
+    auto stream = static_cast<hipStream_t>(stream_handle);
+
+    __atomic_store_n(&host_counts[0], int64_t{-1}, __ATOMIC_RELEASE);
+    const int count_threads = tokens_per_block < kWave ? kWave : tokens_per_block;
+    // Two launches when every block can afford to sum the block histograms itself
+    // (blocks x (L+1) loads spread over the workgroup), three with a single-workgroup scan otherwise.
+    bool fused_scan = blocks > 0 && static_cast<int64_t>(blocks) * (experts + 1) <= int64_t{32} * count_threads;
+    const int forced_launches = env_int("NANOEP_LAYOUT_LAUNCHES", 0);
+    if (forced_launches == 3)
+        fused_scan = false;
+    else if (forced_launches == 2 && blocks > 0)
+        fused_scan = true;
+    hipError_t launch_status = hipSuccess;
+    with_topk_cap(num_topk, [&](auto cap) {
+        constexpr int kCap = decltype(cap)::value;
+        if (blocks == 1 && forced_launches == 0) {
+            const size_t count_lds = static_cast<size_t>(experts + 1) * (words * 6 + 4);
+            const size_t assign_lds = static_cast<size_t>(experts + 1) * 12;
+            layout_single_block_kernel<kCap><<<1, count_threads, count_lds > assign_lds ? count_lds : assign_lds, stream>>>(
+                topk_idx, num_tokens, num_topk, experts, words, count_threads, expand, alignment, topk_snapshot,
+                ws.block_counts, ws.block_status, ws.packed_rank, ws.local_row, expert_counts, expert_offsets, send_counts,
+                recv_rank_prefix, host_counts, recv_metadata, dst_slots, token_slots, slot_order);
+            launch_status = hipGetLastError();
+            return;
+        }
+        if (blocks > 0) {
+            const size_t lds = static_cast<size_t>(experts + 1) * (words * 6 + 4);
+            layout_count_kernel<kCap><<<blocks, count_threads, lds, stream>>>(
+                topk_idx, num_tokens, num_topk, experts, words, count_threads, topk_snapshot, ws.block_counts,
+                ws.block_status, ws.packed_rank, ws.local_row);
+            if ((launch_status = hipGetLastError()) != hipSuccess)
+                return;
+        }
+        const size_t assign_lds = static_cast<size_t>(experts + 1) * 12;
+        if (fused_scan) {
+            layout_assign_kernel<kCap, true><<<blocks, count_threads, assign_lds, stream>>>(
+                ws.block_counts, ws.block_status, blocks, num_tokens, num_topk, experts, tokens_per_block, count_threads,
+                expand, alignment, ws.packed_rank, ws.local_row, expert_counts, expert_offsets, send_counts,
+                recv_rank_prefix, ws.totals, host_counts, recv_metadata, dst_slots, token_slots, slot_order);
+            launch_status = hipGetLastError();
+            return;
+        }
+        layout_scan_kernel<<<1, kScanThreads, static_cast<size_t>(experts + 1) * 4, stream>>>(
+            ws.block_counts, ws.block_status, blocks, experts, alignment, expert_counts, expert_offsets, send_counts,
+            recv_rank_prefix, ws.totals, host_counts);
+        if ((launch_status = hipGetLastError()) != hipSuccess)
+            return;
+        if (blocks > 0) {
+            layout_assign_kernel<kCap, false><<<blocks, count_threads, assign_lds, stream>>>(
+                ws.block_counts, ws.block_status, blocks, num_tokens, num_topk, experts, tokens_per_block, count_threads,
+                expand, alignment, ws.packed_rank, ws.local_row, expert_counts, expert_offsets, send_counts,
+                recv_rank_prefix, ws.totals, host_counts, recv_metadata, dst_slots, token_slots, slot_order);
+            launch_status = hipGetLastError();
+        }
+    });
+    NANOEP_HIP_TRY(launch_status);
+    return NANOEP_OK;
+}
+
+int nanoep_wait_counts(int64_t* host_counts, void* stream_handle, double timeout_seconds,
+                       int64_t out[NANOEP_HOST_COUNT_WORDS]) {
+    if (host_counts == nullptr || out == nullptr)
+        return NANOEP_ERR_INVALID_ARGUMENT;
+    auto stream = static_cast<hipStream_t>(stream_handle);
+    timespec start{};
+    clock_gettime(CLOCK_MONOTONIC, &start);
+    uint64_t spins = 0;
+    while (true) {
+        const int64_t received = __atomic_load_n(&host_counts[0], __ATOMIC_ACQUIRE);
+        if (received >= 0)
+            break;
+        if ((++spins & 0x3ff) == 0) {
+            // A finished (or failed) stream with no published count means the layout never ran.
+            const hipError_t state = hipStreamQuery(stream);
+            if (state != hipErrorNotReady) {
+                if (state != hipSuccess) {
+                    g_last_hip_error = state;
+                    return NANOEP_ERR_HIP;
+                }
+                if (__atomic_load_n(&host_counts[0], __ATOMIC_ACQUIRE) >= 0)
+                    break;
+                return NANOEP_ERR_TIMEOUT;
+            }
+            timespec now{};
+            clock_gettime(CLOCK_MONOTONIC, &now);
+            const double elapsed = (now.tv_sec - start.tv_sec) + 1e-9 * (now.tv_nsec - start.tv_nsec);
+            if (elapsed > timeout_seconds)
+                return NANOEP_ERR_TIMEOUT;
+        }
+    }
+    for (int i = 0; i < NANOEP_HOST_COUNT_WORDS; ++i)
+        out[i] = __atomic_load_n(&host_counts[i], __ATOMIC_RELAXED);
+    return out[3] != 0 ? NANOEP_ERR_ROUTING : NANOEP_OK;
+}
+
+}  // extern "C"
