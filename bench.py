@@ -272,7 +272,8 @@ def main():
     value = (d_bytes + c_bytes) / (ms_per_step * 1e-3) / 1e9
     result.update(
         {
-            "metric": "dispatch+combine achieved HBM bandwidth (algorithmic bytes / wall time), 4096x7168 bf16, 256 experts top-8",
+            "metric": "dispatch+combine achieved HBM bandwidth (algorithmic bytes / wall time), "
+                      f"{workload.tokens}x{workload.hidden} bf16, {workload.experts} experts top-{workload.topk}",
             "value": round(value, 1),
             "unit": "GB/s",
             "n_gpus": 1,
