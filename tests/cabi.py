@@ -132,9 +132,8 @@ def dispatch(x, weights, metadata, counts, num_local_experts, alignment, expand,
              use_table=True, use_order=True, order_count="exact", walk="forced"):
     """Returns (recv_x, recv_topk_idx | None, recv_weights | None) through nanoep_dispatch.
 
-    The library picks the slot-order walk by itself only for batches of at least eight token
-    blocks; walk="forced" makes it walk whatever list it is given, so that small cases cover that
-    kernel too, walk="auto" leaves the choice to the library.
+    walk="forced" sets the library's switch for the slot-order walk explicitly, walk="auto" leaves
+    the environment alone (the library then walks the list whenever it is given one).
     """
     recv_metadata, expert_counts, expert_offsets, dst_slots = metadata[0], metadata[1], metadata[2], metadata[3]
     received, capacity = counts[0], counts[1]

@@ -94,12 +94,12 @@ def test_readme_round_trip(device):
         pytest.param(True, True, False, "skew", 256, 4, id="expanded-skew"),
     ],
 )
-@pytest.mark.parametrize("walk", ["auto", "slot-order"])
+@pytest.mark.parametrize("walk", ["slot-order", "token-order"])
 def test_fresh_and_cached_replay(device, monkeypatch, walk, expand, zero_padding, weighted, kind, hidden, alignment):
-    # small batches take the token-order walk by themselves; forcing the slot-order walk covers
-    # that kernel (fresh: device-side entry count, replay: exact count) through the public API
-    if walk == "slot-order":
-        monkeypatch.setenv("NANOEP_DISPATCH_ORDER", "1")
+    # the library walks the slot-order list of its own handles (fresh: device-side entry count,
+    # replay: exact count); the switch covers the token-order walk with the slot table as well
+    if walk == "token-order":
+        monkeypatch.setenv("NANOEP_DISPATCH_ORDER", "0")
     tokens, experts, topk = 19, 3, 3
     idx = cases.routing(kind, tokens, experts, topk, seed=2)
     x = cases.payload(tokens, hidden)
