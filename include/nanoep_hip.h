@@ -60,9 +60,10 @@ int nanoep_window_layout(int ranks, int64_t max_tokens, int hidden, int topk, in
 /* Device scratch needed by nanoep_layout for (T, K, L). */
 size_t nanoep_layout_workspace_bytes(int64_t num_tokens, int num_topk, int64_t num_local_experts);
 
-/* Tokens per block of the routing layout for L local experts (0: L is not supported).  The
+/* Tokens per block of the routing layout for T tokens and L local experts (0: L is not
+ * supported): 256, fewer for very many experts or for batches of fewer than 2048 tokens.  The
  * slot-order list is ordered block of consecutive tokens by block. */
-int nanoep_layout_block_tokens(int64_t num_local_experts);
+int nanoep_layout_block_tokens(int64_t num_tokens, int64_t num_local_experts);
 
 /* Number of int64 words nanoep_layout writes to the slot-order list for (T, K, L): the block
  * count times block_tokens * K entries (an upper bound of the A that carry assignments), then one

@@ -9,15 +9,23 @@ namespace {
 
 // Tokens handled by one layout workgroup: the LDS bit matrix has (L+1) rows of tokens/32 words
 // plus a 16-bit prefix per word, so the block shrinks as the expert count grows.
-int layout_tokens_per_block(int64_t local_experts) {
+int layout_tokens_per_block(int64_t tokens_total, int64_t local_experts) {
     if (static_cast<size_t>(local_experts + 1) * 12 > kLayoutLdsBudget)  // three int32 arrays of the assignment kernel
         return 0;
+    int chosen = 0;
     for (int tokens = 256; tokens >= 32; tokens /= 2) {
         const size_t words = static_cast<size_t>(tokens / 32);
-        if (static_cast<size_t>(local_experts + 1) * (words * 6 + 4) <= kLayoutLdsBudget)
-            return tokens;
+        if (static_cast<size_t>(local_experts + 1) * (words * 6 + 4) <= kLayoutLdsBudget) {
+            chosen = tokens;
+            break;
+        }
     }
-    return 0;
+    // The dispatch hands every XCD whole token blocks when there are at least eight of them: small
+    // batches take smaller blocks (down to 64 tokens) to get there.  A batch that fits one block
+    // keeps it: its whole layout is then a single launch.
+    while (tokens_total > chosen && chosen > 64 && (tokens_total + chosen - 1) / chosen < 8)
+        chosen /= 2;
+    return chosen;
 }
 
 struct LayoutWorkspace {
@@ -30,7 +38,7 @@ struct LayoutWorkspace {
 };
 
 LayoutWorkspace carve_layout_workspace(void* base, int64_t tokens, int topk, int64_t local_experts) {
-    const int per_block = layout_tokens_per_block(local_experts);
+    const int per_block = layout_tokens_per_block(tokens, local_experts);
     const int64_t blocks = per_block == 0 ? 0 : (tokens + per_block - 1) / per_block;
     auto* cursor = static_cast<uint8_t*>(base);
     size_t offset = 0;
@@ -622,14 +630,14 @@ size_t nanoep_layout_workspace_bytes(int64_t num_tokens, int num_topk, int64_t n
     return carve_layout_workspace(nullptr, num_tokens, num_topk, num_local_experts).bytes;
 }
 
-int nanoep_layout_block_tokens(int64_t num_local_experts) {
-    return num_local_experts <= 0 ? 0 : layout_tokens_per_block(num_local_experts);
+int nanoep_layout_block_tokens(int64_t num_tokens, int64_t num_local_experts) {
+    return num_local_experts <= 0 || num_tokens < 0 ? 0 : layout_tokens_per_block(num_tokens, num_local_experts);
 }
 
 int64_t nanoep_slot_order_entries(int64_t num_tokens, int num_topk, int64_t num_local_experts) {
     if (num_tokens < 0 || num_topk <= 0 || num_local_experts <= 0)
         return 0;
-    const int per_block = layout_tokens_per_block(num_local_experts);
+    const int per_block = layout_tokens_per_block(num_tokens, num_local_experts);
     if (per_block == 0 || num_tokens == 0)
         return 0;
     return (num_tokens + per_block - 1) / per_block * per_block * num_topk + 1;
@@ -651,7 +659,7 @@ int nanoep_layout(const int64_t* topk_idx, int64_t num_tokens, int num_topk, int
     // the slot-order list packs token * K + k into 32 bits and only exists for the expanded layout
     if (slot_order != nullptr && (!expand || num_tokens * num_topk >= (int64_t{1} << 31)))
         return NANOEP_ERR_INVALID_ARGUMENT;
-    const int tokens_per_block = layout_tokens_per_block(num_local_experts);
+    const int tokens_per_block = layout_tokens_per_block(num_tokens, num_local_experts);
     if (tokens_per_block == 0)
         return NANOEP_ERR_INVALID_ARGUMENT;
     const LayoutWorkspace ws = carve_layout_workspace(workspace, num_tokens, num_topk, num_local_experts);

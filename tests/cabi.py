@@ -42,7 +42,7 @@ def lib() -> ctypes.CDLL:
         handle.nanoep_layout_workspace_bytes.restype = sz
         handle.nanoep_layout_workspace_bytes.argtypes = [i64, i, i64]
         handle.nanoep_layout_block_tokens.restype = i
-        handle.nanoep_layout_block_tokens.argtypes = [i64]
+        handle.nanoep_layout_block_tokens.argtypes = [i64, i64]
         handle.nanoep_slot_order_entries.restype = i64
         handle.nanoep_slot_order_entries.argtypes = [i64, i, i64]
         handle.nanoep_layout.argtypes = [p, i64, i, i64, i64, i, p, p, p, p, p, p, p, p, p, p, sz, p, p]

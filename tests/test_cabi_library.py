@@ -68,9 +68,10 @@ def test_argument_checks_come_before_any_device_work():
     assert library.nanoep_layout(null, 4, 2, 4, 0, 0, null, null, null, null, null, null, null, null, null, null, 0, null, null) == 1
     # a slot-order list only exists for the expanded layout
     assert library.nanoep_layout(null, 4, 2, 4, 1, 0, null, 8, 8, null, 8, null, 8, null, 8, 8, 0, 8, null) == 1
-    assert library.nanoep_slot_order_entries(4096, 8, 256) == 4096 * 8 + 1 and library.nanoep_layout_block_tokens(256) == 256
+    assert library.nanoep_slot_order_entries(4096, 8, 256) == 4096 * 8 + 1 and library.nanoep_layout_block_tokens(4096, 256) == 256
     assert library.nanoep_slot_order_entries(100, 3, 8) == 256 * 3 + 1 and library.nanoep_slot_order_entries(0, 3, 8) == 0
-    assert library.nanoep_layout_block_tokens(6000) == 0 and library.nanoep_layout_block_tokens(0) == 0
+    assert library.nanoep_layout_block_tokens(4096, 6000) == 0 and library.nanoep_layout_block_tokens(4096, 0) == 0
+    assert [library.nanoep_layout_block_tokens(t, 256) for t in (1, 256, 257, 512, 1024, 1536, 1792, 1793, 2048, 100000)] == [256, 256, 64, 64, 128, 128, 128, 256, 256, 256]
     out = (ctypes.c_int64 * 4)()
     assert library.nanoep_wait_counts(null, null, 0.0, out) == 1
 

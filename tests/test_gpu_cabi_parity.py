@@ -47,7 +47,7 @@ def assert_layout(metadata, counts, expected: oracle.Layout, expand):
         # private slot-order list: block of consecutive tokens by block, the valid assignments as
         # (slot << 32) | (t * K + k) in ascending slot order, without gaps; -1 from entry A on
         tokens, topk = expected.topk_idx.shape
-        block_tokens = cabi.lib().nanoep_layout_block_tokens(expected.expert_counts.numel())
+        block_tokens = cabi.lib().nanoep_layout_block_tokens(tokens, expected.expert_counts.numel())
         flat = table.flatten().to(torch.int64)
         packed = (flat << 32) | torch.arange(flat.numel(), dtype=torch.int64)
         want = []
