@@ -233,6 +233,92 @@ def test_baseline_shapes(device, name, tokens, hidden, experts, topk, kind, expa
     run_dispatch_combine(device, idx, hidden, experts, alignment, expand, zero_padding, True, seed=6)
 
 
+def closed_form_slots(idx, experts, alignment):
+    """slot[t,k] from the definition, evaluated with torch on the device of idx: experts ascending,
+    inside an expert the tokens ascending, every expert's range padded to the alignment."""
+    flat = idx.flatten()
+    valid = flat >= 0
+    counts = torch.bincount(flat[valid], minlength=experts)
+    padded = (counts + alignment - 1) // alignment * alignment
+    offsets = torch.cumsum(padded, 0) - padded
+    keys = torch.where(valid, flat, torch.full_like(flat, experts))
+    order = torch.sort(keys, stable=True).indices  # (t, k) pairs expert by expert, tokens ascending
+    sorted_keys = keys[order]
+    first_of_expert = torch.cumsum(counts, 0) - counts
+    live = sorted_keys < experts
+    position = torch.arange(flat.numel(), device=idx.device)
+    slot_sorted = torch.where(
+        live, offsets[sorted_keys.clamp(max=experts - 1)] + position - first_of_expert[sorted_keys.clamp(max=experts - 1)],
+        torch.full_like(position, -1),
+    )
+    slots = torch.empty_like(flat)
+    slots[order] = slot_sorted
+    return slots.view_as(idx), counts, int(padded.sum())
+
+
+@pytest.mark.parametrize(
+    "tokens,hidden,experts,topk,expand,alignment",
+    [
+        pytest.param(40960, 7168, 256, 8, True, 1, id="expanded-4.7GB"),
+        pytest.param(40960, 7168, 64, 8, True, 128, id="expanded-align128-4.5GB"),
+        pytest.param(303104, 7168, 8, 2, False, 1, id="compact-4.3GB"),
+    ],
+)
+def test_rows_beyond_four_gib(device, tokens, hidden, experts, topk, expand, alignment):
+    """Receive buffers larger than 2^32 bytes: row addresses must be formed in 64 bits.  At this size
+    the check is by properties that fix the result without the CPU oracle: the slots against their
+    closed form, every received row against its source row bit for bit, padding rows zero, and
+    combine over identity experts equal to multiplicity * x, exact for small-integer payloads."""
+    small = cases.routing("dropout", 700, 40, 6, seed=3)  # the closed form itself, against the oracle
+    want = oracle.layout(small, 40, 8)
+    small_slots, small_counts, small_capacity = closed_form_slots(small, 40, 8)
+    assert torch.equal(small_slots[want.src_tokens], want.expanded_slots) and small_capacity == want.expanded_capacity
+    assert torch.equal(small_counts, want.expert_counts)
+
+    g = torch.Generator(device=device).manual_seed(99)
+    idx = torch.rand(tokens, experts, device=device, generator=g).topk(topk, dim=1).indices.to(torch.int64)
+    idx = torch.where(torch.rand(tokens, topk, device=device, generator=g) < 0.05, torch.full_like(idx, -1), idx)
+    idx = idx.contiguous()
+    x = torch.randint(-4, 5, (tokens, hidden), device=device, generator=g).to(torch.bfloat16)
+    w = torch.rand(tokens, topk, device=device, generator=g)
+
+    metadata, counts = cabi.layout(idx, experts, alignment, expand)
+    slots, expert_counts, capacity = closed_form_slots(idx, experts, alignment)
+    sent = (idx >= 0).any(dim=1)
+    assert counts[0] == int(sent.sum()) and counts[1] == capacity and counts[2] == int((idx >= 0).sum()) and counts[3] == 0
+    assert torch.equal(metadata[1], expert_counts)
+    rows = capacity if expand else counts[0]
+    assert rows * hidden * 2 > 2**32
+    row_of_token = torch.where(sent, torch.cumsum(sent, 0) - 1, torch.full((tokens,), -1, device=device))
+    assert torch.equal(metadata[3].flatten(), row_of_token)
+    if expand:
+        assert torch.equal(metadata[0][:, 2:].to(torch.int64), slots[sent])
+        assert torch.equal(metadata[7].to(torch.int64), slots)
+
+    recv_x, recv_idx, recv_w = cabi.dispatch(x, w, metadata, counts, experts, alignment, expand, expand, poison=POISON)
+    torch.cuda.synchronize()
+    assert recv_x.shape == (rows, hidden)
+    if expand:
+        written = torch.zeros(rows, dtype=torch.bool, device=device)
+        for k in range(topk):
+            live = slots[:, k] >= 0
+            assert torch.equal(bits(recv_x[slots[live, k]]), bits(x[live])), f"payload of choice {k}"
+            assert torch.equal(recv_w[slots[live, k]], w[live, k])
+            written[slots[live, k]] = True
+        assert int(written.sum()) == counts[2]
+        assert not recv_x[~written].view(torch.int16).any() and not recv_w[~written].view(torch.int32).any()
+    else:
+        assert torch.equal(bits(recv_x), bits(x[sent]))
+        assert torch.equal(recv_w, w[sent])
+        assert torch.equal(recv_idx, idx[sent])
+
+    out, out_w = cabi.combine(recv_x, recv_w, None, metadata, counts, expand, poison=POISON)
+    torch.cuda.synchronize()
+    multiplicity = (idx >= 0).sum(dim=1, keepdim=True) if expand else sent[:, None].to(torch.int64)
+    assert torch.equal(out.float(), x.float() * multiplicity)  # |sum| <= 32: exact in bf16
+    assert torch.equal(out_w, torch.where(idx >= 0, w, torch.zeros_like(w)))
+
+
 @pytest.mark.parametrize("topk,experts,hidden", [(1, 4, 256), (5, 16, 1024), (12, 40, 512), (32, 64, 256), (32, 32, 2048)])
 @pytest.mark.parametrize("expand", [False, True], ids=["compact", "expanded"])
 def test_topk_range(device, topk, experts, hidden, expand):
