@@ -50,7 +50,7 @@ __device__ __forceinline__ void zero_fill_gap_rows(uint32_t block,
     if (j >= pad_per_expert)
         return;
     const int64_t out_row = uniform_load(expert_offsets + expert) + uniform_load(expert_counts + expert) + j;
-    if (out_row >= uniform_load(expert_offsets + expert + 1) || out_row >= out_rows)
+    if (out_row < 0 || out_row >= uniform_load(expert_offsets + expert + 1) || out_row >= out_rows)
         return;
     const u32x4 zero = {0u, 0u, 0u, 0u};
     u32x4* dst = recv_x + out_row * vectors;

@@ -293,7 +293,8 @@ __global__ void __launch_bounds__(kScanThreads) layout_scan_kernel(int32_t* __re
     }
 }
 
-// Writes one token's part of the handle.  `slot_base[e]` is the first slot of this block's
+// Writes one token's part of the handle.  `packed` holds the token's entries of the rank table,
+// `slot_base[e]` is the first slot of this block's
 // assignments to expert e; `order_base[e]` is where expert e's run starts in the block's segment
 // of the slot-order list (`order` points at that segment, or is null).
 template <int kCap>
@@ -304,15 +305,11 @@ __device__ __forceinline__ void assign_token_slots(int64_t token,
                                                    int64_t row_base,
                                                    const int32_t* slot_base,
                                                    const int32_t* order_base,
-                                                   const int32_t* __restrict__ packed_rank,
+                                                   const int32_t (&packed)[kCap],
                                                    int32_t* __restrict__ recv_metadata,
                                                    int64_t* __restrict__ dst_slots,
                                                    int32_t* __restrict__ token_slots,
                                                    int64_t* __restrict__ order) {
-    int32_t packed[kCap];
-#pragma unroll
-    for (int k = 0; k < kCap; ++k)
-        packed[k] = packed_rank[token * num_topk + (k < num_topk ? k : 0)];
     if (row_in_block < 0) {
         dst_slots[token] = -1;
         if (token_slots != nullptr)
@@ -406,6 +403,11 @@ __device__ __forceinline__ void layout_assign_block(const int32_t* block_counts,
     const int64_t token = static_cast<int64_t>(block) * tokens_per_block + tid;
     const bool live = tid < tokens_per_block && token < num_tokens;
     const int row_in_block = live ? local_row[token] : -1;
+    // fetched here, ahead of the scans, so that the round trip overlaps them
+    int32_t packed[kCap];
+#pragma unroll
+    for (int k = 0; k < kCap; ++k)
+        packed[k] = live ? packed_rank[token * num_topk + (k < num_topk ? k : 0)] : -1;
 
     if (kFusedScan) {
         for (int i = tid; i < 2 * rows; i += threads)
@@ -421,26 +423,40 @@ __device__ __forceinline__ void layout_assign_block(const int32_t* block_counts,
         const int segment = tid / columns_per_pass;
         const int begin = segment * blocks_per_segment;
         const int end = begin + blocks_per_segment < num_blocks ? begin + blocks_per_segment : num_blocks;
-        for (int column0 = 0; column0 < rows; column0 += columns_per_pass) {
+        // two columns a pass: with one more column than threads (L a multiple of the workgroup
+        // size, plus the received-token column) the loads of both are in flight together
+        for (int column0 = 0; column0 < rows; column0 += 2 * columns_per_pass) {
             const int column = column0 + column_local;
-            if (segment < segments && column < rows) {
-                int total = 0, before = 0, own = 0;
+            const int second = column + columns_per_pass;
+            const bool active = segment < segments && column < rows;
+            const bool active_second = segment < segments && second < rows;
+            int total[2] = {0, 0}, before[2] = {0, 0}, own[2] = {0, 0};
+            if (active) {
 #pragma unroll 8
                 for (int b = begin; b < end; ++b) {
                     const int count = block_counts[static_cast<int64_t>(b) * rows + column];
-                    total += count;
-                    before += b < block ? count : 0;
-                    own = b == block ? count : own;
+                    const int count_second = active_second ? block_counts[static_cast<int64_t>(b) * rows + second] : 0;
+                    total[0] += count;
+                    total[1] += count_second;
+                    before[0] += b < block ? count : 0;
+                    before[1] += b < block ? count_second : 0;
+                    own[0] = b == block ? count : own[0];
+                    own[1] = b == block ? count_second : own[1];
                 }
+            }
+            for (int i = 0; i < 2; ++i) {
+                const int at = i == 0 ? column : second;
+                if (!(i == 0 ? active : active_second))
+                    continue;
                 if (segments == 1) {
-                    column_total[column] = total;
-                    slot_base[column] = before;
+                    column_total[at] = total[i];
+                    slot_base[at] = before[i];
                 } else {
-                    atomicAdd(&column_total[column], total);
-                    atomicAdd(&slot_base[column], before);
+                    atomicAdd(&column_total[at], total[i]);
+                    atomicAdd(&slot_base[at], before[i]);
                 }
                 if (block >= begin && block < end)
-                    order_base[column] = own;
+                    order_base[at] = own[i];
             }
         }
         if (block == 0) {
@@ -550,7 +566,7 @@ __device__ __forceinline__ void layout_assign_block(const int32_t* block_counts,
     }
     if (live)
         assign_token_slots<kCap>(token, num_topk, expand, row_in_block, slot_base[local_experts], slot_base, order_base,
-                                 packed_rank, recv_metadata, dst_slots, token_slots, order);
+                                 packed, recv_metadata, dst_slots, token_slots, order);
 }
 
 template <int kCap, bool kFusedScan>
