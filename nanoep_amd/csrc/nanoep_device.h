@@ -142,6 +142,9 @@ __device__ __forceinline__ uint32_t fast_divide(uint32_t n, uint32_t magic, uint
 #define NANOEP_FETCH_ARGS_2(a, b) asm volatile("" ::"s"(a), "s"(b))
 #define NANOEP_FETCH_ARGS_4(a, b, c, d) asm volatile("" ::"s"(a), "s"(b), "s"(c), "s"(d))
 
+// Last-level (memory-side) cache of the MI355X: 256 MiB.
+constexpr int64_t kLastLevelCacheBytes = int64_t{256} << 20;
+
 constexpr int kMaxWavesPerBlock = 16;
 constexpr int kDefaultChunksPerBlock = 2;
 

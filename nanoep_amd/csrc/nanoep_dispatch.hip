@@ -169,7 +169,10 @@ __global__ void __launch_bounds__(1024) dispatch_rows_kernel(const u32x4* __rest
 // scalar instruction and branch ahead of the source load is throughput.  Validity is folded into
 // one flag and the load is issued unconditionally (row 0 stands in).  kZeroFill is false when the
 // launch has no gap rows to clear: the copy path then carries none of that bookkeeping.
-template <bool kDeviceCount, bool kZeroFill>
+// kSpan is the number of consecutive 1 KiB chunks a wavefront moves (loads issued back to back,
+// then the stores).  One is best while the source fits the last-level cache; beyond that size the
+// single-chunk walk loses a quarter of its rate and two chunks a wavefront win it back.
+template <bool kDeviceCount, bool kZeroFill, int kSpan>
 __global__ void __launch_bounds__(1024) dispatch_ordered_kernel(const u32x4* __restrict__ x,              // [T][vectors]
                                                                 const float* __restrict__ weights,       // [T][K] or null
                                                                 const int64_t* __restrict__ slot_order,  // [entries]
@@ -193,7 +196,7 @@ __global__ void __launch_bounds__(1024) dispatch_ordered_kernel(const u32x4* __r
                                                                 uint32_t chunks_per_block,  // == blockDim.y
                                                                 uint32_t rows_per_block,    // == blockDim.z
                                                                 uint32_t vectors,
-                                                                uint32_t chunks,
+                                                                uint32_t chunks,      // pieces of kSpan chunks in a row
                                                                 uint32_t topk_magic,  // fast divisor by K
                                                                 uint32_t topk_shift) {
     NANOEP_FETCH_ARGS_4(x, weights, recv_x, recv_weights);
@@ -234,13 +237,21 @@ __global__ void __launch_bounds__(1024) dispatch_ordered_kernel(const u32x4* __r
     const uint32_t out_row = static_cast<uint32_t>(static_cast<uint64_t>(entry) >> 32);
     const bool valid = entry >= 0 && source < source_limit && out_row < out_rows;
     const uint32_t token = valid ? fast_divide(source, topk_magic, topk_shift) : 0u;
-    const uint32_t vector = chunk * kWave + threadIdx.x;
-    const bool in_row = vector < vectors;
-    const u32x4 data = x[static_cast<uint64_t>(token) * vectors + (in_row ? vector : 0u)];
+    const uint32_t vector = chunk * (kSpan * kWave) + threadIdx.x;
+    u32x4 data[kSpan];
+#pragma unroll
+    for (int s = 0; s < kSpan; ++s) {
+        const uint32_t at = vector + s * kWave;
+        data[s] = x[static_cast<uint64_t>(token) * vectors + (at < vectors ? at : 0u)];
+    }
     if (!valid)
         return;
-    if (in_row)
-        store_vec<true>(recv_x + static_cast<uint64_t>(out_row) * vectors + vector, data);
+#pragma unroll
+    for (int s = 0; s < kSpan; ++s) {
+        const uint32_t at = vector + s * kWave;
+        if (at < vectors)
+            store_vec<true>(recv_x + static_cast<uint64_t>(out_row) * vectors + at, data[s]);
+    }
     if (chunk == 0 && threadIdx.x == 0 && recv_weights != nullptr)
         recv_weights[out_row] = weights[source];
 }
@@ -344,7 +355,17 @@ int nanoep_dispatch(const void* x, const float* weights, const int32_t* recv_met
         slot_order_entries = order_bound;
 
     const int vectors = hidden / 8;
-    const int chunks = (vectors + kWave - 1) / kWave;
+    int chunks = (vectors + kWave - 1) / kWave;
+    // Chunks per wavefront of the slot-order walk: two once the source outgrows the last-level cache
+    // (NANOEP_DISPATCH_SPAN=1|2 overrides).  `chunks` then counts pieces of that many chunks.
+    int span = 1;
+    if (ordered) {
+        span = static_cast<int64_t>(num_tokens) * hidden * 2 > kLastLevelCacheBytes ? 2 : 1;
+        const int forced_span = env_int("NANOEP_DISPATCH_SPAN", 0);
+        if (forced_span == 1 || forced_span == 2)
+            span = forced_span;
+        chunks = (chunks + span - 1) / span;
+    }
     const RowBlocking blocking = pick_row_blocking(chunks, ordered ? kSlotOrderWalk : expand ? kTokenOrderWalk : kRowCopyWalk);
     const int64_t waves = static_cast<int64_t>(blocking.chunks_per_block) * blocking.rows_per_block;
     const int64_t copy_candidates = ordered ? slot_order_entries : expand ? num_tokens * num_topk : num_tokens;
@@ -368,8 +389,8 @@ int nanoep_dispatch(const void* x, const float* weights, const int32_t* recv_met
     auto stream = static_cast<hipStream_t>(stream_handle);
     if (ordered) {
         const FastDivisor topk_divisor = make_fast_divisor(static_cast<uint32_t>(num_topk));
-#define NANOEP_LAUNCH_ORDERED(DEVICE_COUNT, ZERO_FILL)                                                                \
-    dispatch_ordered_kernel<DEVICE_COUNT, ZERO_FILL><<<grid, block, 0, stream>>>(                                    \
+#define NANOEP_LAUNCH_ORDERED_SPAN(DEVICE_COUNT, ZERO_FILL, SPAN)                                                     \
+    dispatch_ordered_kernel<DEVICE_COUNT, ZERO_FILL, SPAN><<<grid, block, 0, stream>>>(                              \
         static_cast<const u32x4*>(x), weights, slot_order, live_count, expert_counts, expert_offsets,                \
         static_cast<u32x4*>(recv_x), recv_weights, static_cast<uint32_t>(copy_candidates),                           \
         static_cast<uint32_t>(num_tokens * num_topk), static_cast<uint32_t>(out_rows),                               \
@@ -378,6 +399,13 @@ int nanoep_dispatch(const void* x, const float* weights, const int32_t* recv_met
         static_cast<uint32_t>(pad_groups_per_expert > 0 ? pad_groups_per_expert : 1), blocking.parts,                \
         parts_divisor.magic, parts_divisor.shift, blocking.chunks_per_block, blocking.rows_per_block,                \
         static_cast<uint32_t>(vectors), static_cast<uint32_t>(chunks), topk_divisor.magic, topk_divisor.shift)
+#define NANOEP_LAUNCH_ORDERED(DEVICE_COUNT, ZERO_FILL)             \
+    do {                                                           \
+        if (span == 2)                                             \
+            NANOEP_LAUNCH_ORDERED_SPAN(DEVICE_COUNT, ZERO_FILL, 2); \
+        else                                                       \
+            NANOEP_LAUNCH_ORDERED_SPAN(DEVICE_COUNT, ZERO_FILL, 1); \
+    } while (0)
         if (live_count != nullptr && pad_blocks > 0)
             NANOEP_LAUNCH_ORDERED(true, true);
         else if (live_count != nullptr)
@@ -387,6 +415,7 @@ int nanoep_dispatch(const void* x, const float* weights, const int32_t* recv_met
         else
             NANOEP_LAUNCH_ORDERED(false, false);
 #undef NANOEP_LAUNCH_ORDERED
+#undef NANOEP_LAUNCH_ORDERED_SPAN
     } else if (!expand) {
         const int64_t blocks = (num_tokens + blocking.rows_per_block - 1) / blocking.rows_per_block * blocking.parts;
         dispatch_compact_kernel<<<dim3(static_cast<unsigned>(blocks)), block, 0, stream>>>(

@@ -129,11 +129,12 @@ def slot_order_of(metadata, use_order=True):
 
 
 def dispatch(x, weights, metadata, counts, num_local_experts, alignment, expand, zero_padding, *, num_cus=0, poison=None,
-             use_table=True, use_order=True, order_count="exact", walk="forced"):
+             use_table=True, use_order=True, order_count="exact", walk="forced", span=None):
     """Returns (recv_x, recv_topk_idx | None, recv_weights | None) through nanoep_dispatch.
 
     walk="forced" sets the library's switch for the slot-order walk explicitly, walk="auto" leaves
-    the environment alone (the library then walks the list whenever it is given one).
+    the environment alone (the library then walks the list whenever it is given one).  span=1|2
+    forces the number of chunks a wavefront of that walk moves (the library picks it by source size).
     """
     recv_metadata, expert_counts, expert_offsets, dst_slots = metadata[0], metadata[1], metadata[2], metadata[3]
     received, capacity = counts[0], counts[1]
@@ -155,8 +156,11 @@ def dispatch(x, weights, metadata, counts, num_local_experts, alignment, expand,
     # exact count A, or -1: the kernel reads A from the word behind the list
     order_entries = 0 if order is None else (counts[2] if order_count == "exact" else -1)
     previous = os.environ.pop("NANOEP_DISPATCH_ORDER", None)
+    previous_span = os.environ.pop("NANOEP_DISPATCH_SPAN", None)
     if walk == "forced":
         os.environ["NANOEP_DISPATCH_ORDER"] = "1"
+    if span is not None:
+        os.environ["NANOEP_DISPATCH_SPAN"] = str(span)
     try:
         status = lib().nanoep_dispatch(
             ptr(x), ptr(weights), ptr(recv_metadata), ptr(dst_slots), ptr(token_slots_of(metadata, use_table)),
@@ -166,8 +170,11 @@ def dispatch(x, weights, metadata, counts, num_local_experts, alignment, expand,
         )
     finally:
         os.environ.pop("NANOEP_DISPATCH_ORDER", None)
+        os.environ.pop("NANOEP_DISPATCH_SPAN", None)
         if previous is not None:
             os.environ["NANOEP_DISPATCH_ORDER"] = previous
+        if previous_span is not None:
+            os.environ["NANOEP_DISPATCH_SPAN"] = previous_span
     check(status)
     return recv_x, recv_idx, recv_w
 

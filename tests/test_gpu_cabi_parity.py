@@ -90,6 +90,15 @@ def run_dispatch_combine(device, idx, hidden, experts, alignment, expand, zero_p
         )
         assert torch.equal(device_x.view(torch.int16), got_x.view(torch.int16))
         assert device_w is None or torch.equal(device_w.view(torch.int32), got_w.view(torch.int32))
+        # ... so must the walk that moves two chunks a wavefront (the library's choice for sources
+        # beyond the last-level cache), with either entry count
+        for order_count in ("exact", "device"):
+            wide_x, _, wide_w = cabi.dispatch(
+                x.to(device), None if w is None else w.to(device), metadata, counts, experts, alignment, expand, zero_padding,
+                num_cus=num_cus, poison=POISON, order_count=order_count, span=2,
+            )
+            assert torch.equal(wide_x.view(torch.int16), got_x.view(torch.int16))
+            assert wide_w is None or torch.equal(wide_w.view(torch.int32), got_w.view(torch.int32))
         # ... so must the same call with the library's switches left alone
         auto_x, _, auto_w = cabi.dispatch(
             x.to(device), None if w is None else w.to(device), metadata, counts, experts, alignment, expand, zero_padding,
