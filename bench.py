@@ -275,7 +275,7 @@ def main():
     if not workload.expand:
         combine_kernel = "combine_compact_kernel"
     else:
-        combine_kernel = "combine_few_rows_kernel" if 2 <= workload.topk <= 4 else "combine_rows_kernel"
+        combine_kernel = "combine_few_rows_kernel" if workload.topk <= 4 else "combine_rows_kernel"
     result.update(
         {
             "metric": "dispatch+combine achieved HBM bandwidth (algorithmic bytes / wall time), "

@@ -315,7 +315,8 @@ int nanoep_combine(const void* y, const float* weights, const void* bias, const 
 
     const int vectors = hidden / 8;
     const int chunks = (vectors + kWave - 1) / kWave;
-    const RowBlocking blocking = pick_row_blocking(chunks, expand ? kTokenOrderWalk : kRowCopyWalk);
+    // top-1 expanded combines are row copies like the compact ones
+    const RowBlocking blocking = pick_row_blocking(chunks, expand && num_topk > 1 ? kTokenOrderWalk : kRowCopyWalk);
     const int64_t blocks = (num_tokens + blocking.rows_per_block - 1) / blocking.rows_per_block * blocking.parts;
     if (blocks >= (int64_t{1} << 31))
         return NANOEP_ERR_INVALID_ARGUMENT;
@@ -337,7 +338,7 @@ int nanoep_combine(const void* y, const float* weights, const void* bias, const 
         NANOEP_HIP_TRY(hipGetLastError());
         return NANOEP_OK;
     }
-    if (direct && num_topk >= 2 && num_topk <= 4) {
+    if (direct && num_topk <= 4) {
 #define NANOEP_LAUNCH_FEW(TOPK)                                                                                       \
     combine_few_rows_kernel<TOPK><<<grid, block, 0, stream>>>(                                                       \
         static_cast<const u32x4*>(y), weights, static_cast<const u32x4*>(bias), token_slots,                         \
@@ -345,7 +346,9 @@ int nanoep_combine(const void* y, const float* weights, const void* bias, const 
         blocking.parts, parts_divisor.magic, parts_divisor.shift, blocking.chunks_per_block, blocking.rows_per_block, \
         static_cast<uint32_t>(vectors), static_cast<uint32_t>(chunks), static_cast<uint32_t>(num_topk),              \
         multiple_reduction ? 1 : 0)
-        if (num_topk == 2)
+        if (num_topk == 1)
+            NANOEP_LAUNCH_FEW(1);
+        else if (num_topk == 2)
             NANOEP_LAUNCH_FEW(2);
         else
             NANOEP_LAUNCH_FEW(4);
