@@ -188,10 +188,17 @@ def main():
     device = torch.device("cuda", 0)
     torch.cuda.set_device(device)
 
-    rotation = 8  # 8 x 58.7 MB of sources: more than the 256 MB last-level cache
-    batches = [workloads.make_inputs(workload, seed=seed) for seed in range(rotation)]
-    x_cpu, idx_cpu, w_cpu = batches[0]
-    xs = [batch[0].to(device) for batch in batches]
+    # Rotating source copies: at least 8, and at least three times the 256 MiB last-level cache in
+    # total, so that no launch finds its source cache resident (8 x 58.7 MB at the headline batch,
+    # 24 copies of a 33.5 MB source).  Copy 0 is the batch that is checked against the oracle.
+    x_cpu, idx_cpu, w_cpu = workloads.make_inputs(workload, seed=0)
+    source_bytes = max(1, x_cpu.numel() * x_cpu.element_size())
+    rotation = min(32, max(8, -(-3 * (256 << 20) // source_bytes)))
+    generator = torch.Generator(device=device).manual_seed(1)
+    xs = [x_cpu.to(device)] + [
+        torch.randn(x_cpu.shape, device=device, generator=generator, dtype=torch.float32).to(torch.bfloat16)
+        for _ in range(rotation - 1)
+    ]
     idx = idx_cpu.to(device)
     weights = w_cpu.to(device)
 
@@ -306,6 +313,7 @@ def main():
                 "assignments": assignments,
                 "expanded_capacity": capacity,
                 "step": "cached-handle dispatch + combine through Buffer.dispatch / Buffer.combine",
+                "rotating_source_copies": rotation,
             },
             "frac_of_hbm_peak": round(value / HBM_PEAK_GBS, 4),
             "gpu_us_per_step": round(gpu_step_seconds / args.steps * 1e6, 2),
