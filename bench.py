@@ -64,7 +64,7 @@ def layout_gpu_us(workload, idx, iterations=50):
     library.nanoep_layout_workspace_bytes.argtypes = [i64, ctypes.c_int, i64]
     library.nanoep_slot_order_entries.restype = i64
     library.nanoep_slot_order_entries.argtypes = [i64, ctypes.c_int, i64]
-    library.nanoep_layout.argtypes = [p, i64, ctypes.c_int, i64, i64, ctypes.c_int, p, p, p, p, p, p, p, p, p, p, ctypes.c_size_t, p, p]
+    library.nanoep_layout.argtypes = [p, i64, ctypes.c_int, i64, i64, ctypes.c_int, ctypes.c_int, p, p, p, p, p, p, p, p, p, p, ctypes.c_size_t, p, p]
     tokens, topk, experts = workload.tokens, workload.topk, workload.experts
     device = idx.device
     nbytes = library.nanoep_layout_workspace_bytes(tokens, topk, experts)
@@ -83,7 +83,7 @@ def layout_gpu_us(workload, idx, iterations=50):
 
     def launch():
         status = library.nanoep_layout(idx.data_ptr(), tokens, topk, experts, workload.alignment, int(workload.expand),
-                                       metadata.data_ptr(), counts.data_ptr(), offsets.data_ptr(), dst_slots.data_ptr(),
+                                       workload.hidden, metadata.data_ptr(), counts.data_ptr(), offsets.data_ptr(), dst_slots.data_ptr(),
                                        sent.data_ptr(), snapshot.data_ptr(), prefix.data_ptr(),
                                        table.data_ptr() if workload.expand else None,
                                        order.data_ptr() if workload.expand else None, workspace.data_ptr(), nbytes,

@@ -24,7 +24,7 @@ using namespace nanoep;
 
 extern "C" {
 
-int nanoep_abi_version(void) { return 2; }
+int nanoep_abi_version(void) { return 3; }
 
 const char* nanoep_status_string(int status) {
     switch (status) {

@@ -207,9 +207,11 @@ __global__ void __launch_bounds__(1024) dispatch_ordered_kernel(const u32x4* __r
     if (kDeviceCount) {
         // The list length was not known when the grid was sized: shrink the walk to the entries in
         // use, so that the per-XCD ranges split the real work and not its unused tail.
+        // A word that cannot be a count (the layout did not run) walks nothing: the buffer's tail
+        // behind the layout's blocks is never written.
         const int64_t live = uniform_load(live_count);
-        if (live >= 0 && live < static_cast<int64_t>(entries)) {
-            entries = static_cast<uint32_t>(live);
+        if (live != static_cast<int64_t>(entries)) {
+            entries = live >= 0 && live < static_cast<int64_t>(entries) ? static_cast<uint32_t>(live) : 0u;
             copy_blocks = (rows_per_block == 1 ? entries : (entries + rows_per_block - 1) / rows_per_block) * parts;
             copy_per_xcd = (copy_blocks + kNumXcds - 1) / kNumXcds;
         }

@@ -7,25 +7,47 @@
 namespace nanoep {
 namespace {
 
-// Tokens handled by one layout workgroup: the LDS bit matrix has (L+1) rows of tokens/32 words
-// plus a 16-bit prefix per word, so the block shrinks as the expert count grows.
-int layout_tokens_per_block(int64_t tokens_total, int64_t local_experts) {
+// Largest block of tokens a layout workgroup handles (one thread per token).
+constexpr int kMaxBlockTokens = 512;
+// An XCD's L2: the rows of one token block should fit it, since the dispatch walks the slot-order
+// list block by block and wants every re-use of a source row to hit that cache.
+constexpr int64_t kXcdL2Bytes = int64_t{4} << 20;
+
+// Tokens handled by one layout workgroup = tokens of one block of the slot-order list.
+//  * `hidden` (bf16 elements of a payload row, 0 = not known) sizes the block so that its rows fit an
+//    XCD's L2: 512 tokens up to 4096 elements, 256 up to 8192 (and when it is not known), 128, 64.
+//  * The LDS bit matrix has (L+1) rows of tokens/32 words plus a 16-bit prefix per word, so the block
+//    shrinks as the expert count grows.
+//  * The dispatch hands every XCD whole token blocks when there are at least eight of them: batches
+//    of more than 256 tokens take smaller blocks (down to 64 tokens) to get there.  A batch of up to
+//    256 tokens is one block: its whole layout is then a single launch.
+int layout_tokens_per_block(int64_t tokens_total, int64_t local_experts, int hidden) {
     if (static_cast<size_t>(local_experts + 1) * 12 > kLayoutLdsBudget)  // three int32 arrays of the assignment kernel
         return 0;
+    int largest = 256;
+    if (hidden > 0)
+        for (largest = kMaxBlockTokens; largest > 64 && static_cast<int64_t>(largest) * hidden * 2 > kXcdL2Bytes; largest /= 2) {
+        }
+    if (tokens_total <= 256 && largest > 256)
+        largest = 256;
     int chosen = 0;
-    for (int tokens = 256; tokens >= 32; tokens /= 2) {
+    for (int tokens = largest; tokens >= 32; tokens /= 2) {
         const size_t words = static_cast<size_t>(tokens / 32);
         if (static_cast<size_t>(local_experts + 1) * (words * 6 + 4) <= kLayoutLdsBudget) {
             chosen = tokens;
             break;
         }
     }
-    // The dispatch hands every XCD whole token blocks when there are at least eight of them: small
-    // batches take smaller blocks (down to 64 tokens) to get there.  A batch that fits one block
-    // keeps it: its whole layout is then a single launch.
-    while (tokens_total > chosen && chosen > 64 && (tokens_total + chosen - 1) / chosen < 8)
+    while (tokens_total > 256 && chosen > 64 && (tokens_total + chosen - 1) / chosen < 8)
         chosen /= 2;
     return chosen;
+}
+
+// Smallest block any `hidden` can lead to for this batch: what the workspace is sized for.
+int layout_smallest_block(int64_t tokens_total, int64_t local_experts) {
+    const int narrow = layout_tokens_per_block(tokens_total, local_experts, 1 << 20);
+    const int wide = layout_tokens_per_block(tokens_total, local_experts, 8);
+    return narrow < wide ? narrow : wide;
 }
 
 struct LayoutWorkspace {
@@ -38,7 +60,7 @@ struct LayoutWorkspace {
 };
 
 LayoutWorkspace carve_layout_workspace(void* base, int64_t tokens, int topk, int64_t local_experts) {
-    const int per_block = layout_tokens_per_block(tokens, local_experts);
+    const int per_block = layout_smallest_block(tokens, local_experts);
     const int64_t blocks = per_block == 0 ? 0 : (tokens + per_block - 1) / per_block;
     auto* cursor = static_cast<uint8_t*>(base);
     size_t offset = 0;
@@ -58,8 +80,9 @@ LayoutWorkspace carve_layout_workspace(void* base, int64_t tokens, int topk, int
 }
 
 // A (token, k) entry of the rank table packs (expert << kRankBits) | in-block rank; -1 marks a
-// masked choice.  A layout block never holds more than 256 tokens, so the rank fits 8 bits.
-constexpr int kRankBits = 8;
+// masked choice.  A layout block never holds more than 512 tokens, so the rank fits 9 bits.
+constexpr int kRankBits = 9;
+static_assert(kMaxBlockTokens <= (1 << kRankBits), "in-block ranks must fit the packed entry");
 constexpr int kRankMask = (1 << kRankBits) - 1;
 
 // One thread per token.  bits[e][w] has bit (token & 31) of word (token >> 5) set when the token
@@ -169,7 +192,7 @@ __device__ __forceinline__ void layout_count_block(const int64_t* __restrict__ t
 }
 
 template <int kCap>
-__global__ void __launch_bounds__(256) layout_count_kernel(const int64_t* __restrict__ topk_idx,
+__global__ void __launch_bounds__(kMaxBlockTokens) layout_count_kernel(const int64_t* __restrict__ topk_idx,
                                                            int64_t num_tokens,
                                                            int num_topk,
                                                            int local_experts,
@@ -388,10 +411,10 @@ __device__ __forceinline__ void layout_assign_block(const int32_t* block_counts,
                                                     int32_t* __restrict__ token_slots,
                                                     int64_t* __restrict__ slot_order) {
     extern __shared__ int32_t assign_lds[];
-    __shared__ int64_t wave_padded[kWavesPerBlock];
-    __shared__ int64_t wave_assigned[kWavesPerBlock];
-    __shared__ int32_t wave_own[kWavesPerBlock];
-    __shared__ int32_t wave_before[kWavesPerBlock];
+    __shared__ int64_t wave_padded[kMaxBlockTokens / kWave];
+    __shared__ int64_t wave_assigned[kMaxBlockTokens / kWave];
+    __shared__ int32_t wave_own[kMaxBlockTokens / kWave];
+    __shared__ int32_t wave_before[kMaxBlockTokens / kWave];
     __shared__ int status_bits;
     const int rows = local_experts + 1;
     int32_t* column_total = assign_lds;         // [L+1] totals over all blocks (fused scan only)
@@ -562,7 +585,8 @@ __device__ __forceinline__ void layout_assign_block(const int32_t* block_counts,
         for (int i = tid; i < holes; i += threads)
             tail[i] = -1;
         if (block == 0 && tid == 0)
-            slot_order[num_blocks * block_entries] = assigned;  // count word behind the list
+            // count word: last word of the buffer, whose size does not depend on the block size
+            slot_order[(num_tokens + kMaxBlockTokens - 1) / kMaxBlockTokens * kMaxBlockTokens * num_topk] = assigned;
     }
     if (live)
         assign_token_slots<kCap>(token, num_topk, expand, row_in_block, slot_base[local_experts], slot_base, order_base,
@@ -570,7 +594,7 @@ __device__ __forceinline__ void layout_assign_block(const int32_t* block_counts,
 }
 
 template <int kCap, bool kFusedScan>
-__global__ void __launch_bounds__(256) layout_assign_kernel(const int32_t* __restrict__ block_counts,
+__global__ void __launch_bounds__(kMaxBlockTokens) layout_assign_kernel(const int32_t* __restrict__ block_counts,
                                                             const int32_t* __restrict__ block_status,
                                                             int num_blocks,
                                                             int64_t num_tokens,
@@ -601,7 +625,7 @@ __global__ void __launch_bounds__(256) layout_assign_kernel(const int32_t* __res
 // Whole layout in one launch when all tokens fit one block: the count pass, then (its results are
 // this workgroup's own global writes, made visible by the fence and the barrier) the assignment pass.
 template <int kCap>
-__global__ void __launch_bounds__(256) layout_single_block_kernel(const int64_t* topk_idx,
+__global__ void __launch_bounds__(kMaxBlockTokens) layout_single_block_kernel(const int64_t* topk_idx,
                                                                   int64_t num_tokens,
                                                                   int num_topk,
                                                                   int local_experts,
@@ -646,26 +670,26 @@ size_t nanoep_layout_workspace_bytes(int64_t num_tokens, int num_topk, int64_t n
     return carve_layout_workspace(nullptr, num_tokens, num_topk, num_local_experts).bytes;
 }
 
-int nanoep_layout_block_tokens(int64_t num_tokens, int64_t num_local_experts) {
-    return num_local_experts <= 0 || num_tokens < 0 ? 0 : layout_tokens_per_block(num_tokens, num_local_experts);
+int nanoep_layout_block_tokens(int64_t num_tokens, int64_t num_local_experts, int hidden) {
+    return num_local_experts <= 0 || num_tokens < 0 || hidden < 0 ? 0 : layout_tokens_per_block(num_tokens, num_local_experts, hidden);
 }
 
 int64_t nanoep_slot_order_entries(int64_t num_tokens, int num_topk, int64_t num_local_experts) {
     if (num_tokens < 0 || num_topk <= 0 || num_local_experts <= 0)
         return 0;
-    const int per_block = layout_tokens_per_block(num_tokens, num_local_experts);
-    if (per_block == 0 || num_tokens == 0)
+    if (layout_smallest_block(num_tokens, num_local_experts) == 0 || num_tokens == 0)
         return 0;
-    return (num_tokens + per_block - 1) / per_block * per_block * num_topk + 1;
+    // whole blocks of any size the layout may take, then the count word
+    return (num_tokens + kMaxBlockTokens - 1) / kMaxBlockTokens * kMaxBlockTokens * num_topk + 1;
 }
 
 int nanoep_layout(const int64_t* topk_idx, int64_t num_tokens, int num_topk, int64_t num_local_experts,
-                  int64_t alignment, int expand, int32_t* recv_metadata, int64_t* expert_counts,
+                  int64_t alignment, int expand, int hidden, int32_t* recv_metadata, int64_t* expert_counts,
                   int64_t* expert_offsets, int64_t* dst_slots, int64_t* send_counts, int64_t* topk_snapshot,
                   int64_t* recv_rank_prefix, int32_t* token_slots, int64_t* slot_order, void* workspace,
                   size_t workspace_bytes, int64_t* host_counts, void* stream_handle) {
     if (num_tokens < 0 || num_tokens > INT32_MAX || num_topk <= 0 || num_topk > kMaxTopk || num_local_experts <= 0 ||
-        num_local_experts >= (int64_t{1} << (31 - kRankBits)) || alignment <= 0 || alignment > (int64_t{1} << 31))
+        num_local_experts >= (int64_t{1} << (31 - kRankBits)) || alignment <= 0 || alignment > (int64_t{1} << 31) || hidden < 0)
         return NANOEP_ERR_INVALID_ARGUMENT;
     if (expert_counts == nullptr || expert_offsets == nullptr || send_counts == nullptr || recv_rank_prefix == nullptr ||
         host_counts == nullptr || workspace == nullptr)
@@ -675,7 +699,7 @@ int nanoep_layout(const int64_t* topk_idx, int64_t num_tokens, int num_topk, int
     // the slot-order list packs token * K + k into 32 bits and only exists for the expanded layout
     if (slot_order != nullptr && (!expand || num_tokens * num_topk >= (int64_t{1} << 31)))
         return NANOEP_ERR_INVALID_ARGUMENT;
-    const int tokens_per_block = layout_tokens_per_block(num_tokens, num_local_experts);
+    const int tokens_per_block = layout_tokens_per_block(num_tokens, num_local_experts, hidden);
     if (tokens_per_block == 0)
         return NANOEP_ERR_INVALID_ARGUMENT;
     const LayoutWorkspace ws = carve_layout_workspace(workspace, num_tokens, num_topk, num_local_experts);

@@ -416,7 +416,7 @@ DispatchResult dispatch(PeerRuntime& runtime,
         int64_t* base64 = arena64.data_ptr<int64_t>();
         int32_t* base32 = arena32.data_ptr<int32_t>();
         check_status(nanoep_layout(routing.data_ptr<int64_t>(), tokens, static_cast<int>(topk), local_experts, alignment, expand ? 1 : 0,
-                                   base32, base64, base64 + at_offsets, base64 + at_dst, base64 + at_send, base64 + at_snapshot,
+                                   static_cast<int>(hidden), base32, base64, base64 + at_offsets, base64 + at_dst, base64 + at_send, base64 + at_snapshot,
                                    base64 + at_prefix, expand ? base32 + at_table : nullptr,
                                    order_entries > 0 ? base64 + at_order : nullptr, workspace.data_ptr(), workspace_bytes,
                                    host_counts, comm.stream()),

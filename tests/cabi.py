@@ -42,10 +42,10 @@ def lib() -> ctypes.CDLL:
         handle.nanoep_layout_workspace_bytes.restype = sz
         handle.nanoep_layout_workspace_bytes.argtypes = [i64, i, i64]
         handle.nanoep_layout_block_tokens.restype = i
-        handle.nanoep_layout_block_tokens.argtypes = [i64, i64]
+        handle.nanoep_layout_block_tokens.argtypes = [i64, i64, i]
         handle.nanoep_slot_order_entries.restype = i64
         handle.nanoep_slot_order_entries.argtypes = [i64, i, i64]
-        handle.nanoep_layout.argtypes = [p, i64, i, i64, i64, i, p, p, p, p, p, p, p, p, p, p, sz, p, p]
+        handle.nanoep_layout.argtypes = [p, i64, i, i64, i64, i, i, p, p, p, p, p, p, p, p, p, p, sz, p, p]
         handle.nanoep_wait_counts.argtypes = [p, p, dbl, ctypes.POINTER(i64)]
         handle.nanoep_dispatch.argtypes = [p, p, p, p, p, p, i64, p, p, i64, i64, i64, i, i, i64, i64, i, i, p, p, p, i, p]
         handle.nanoep_combine.argtypes = [p, p, p, p, p, p, i64, i64, i64, i, i, i, i, p, p, i, p]
@@ -80,8 +80,9 @@ def window_layout(ranks, tokens, hidden, topk, experts, multi=False) -> list[int
     return list(out)
 
 
-def layout(topk_idx: torch.Tensor, num_local_experts: int, alignment: int, expand: bool, *, raise_on_routing=True):
-    """Runs the layout kernels and returns (metadata list of 7, or 9 when expanded, (N, C, A, status))."""
+def layout(topk_idx: torch.Tensor, num_local_experts: int, alignment: int, expand: bool, *, raise_on_routing=True, hidden=0):
+    """Runs the layout kernels and returns (metadata list of 7, or 9 when expanded, (N, C, A, status)).
+    hidden is the row width the handle will be used with (0: not known); it sizes the token blocks."""
     device = topk_idx.device
     tokens, topk = topk_idx.shape
     i64 = dict(dtype=torch.int64, device=device)
@@ -102,7 +103,7 @@ def layout(topk_idx: torch.Tensor, num_local_experts: int, alignment: int, expan
     mailbox = torch.empty(HOST_COUNT_WORDS, dtype=torch.int64, pin_memory=True)
     check(
         lib().nanoep_layout(
-            ptr(topk_idx), tokens, topk, num_local_experts, alignment, int(expand), ptr(recv_metadata),
+            ptr(topk_idx), tokens, topk, num_local_experts, alignment, int(expand), hidden, ptr(recv_metadata),
             ptr(expert_counts), ptr(expert_offsets), ptr(dst_slots), ptr(send_counts), ptr(snapshot), ptr(prefix),
             ptr(token_slots), ptr(slot_order), ptr(workspace), ws_bytes, mailbox.data_ptr(), stream_handle(),
         )

@@ -12,7 +12,7 @@ int main(void) {
            (long long)window[1], (long long)window[2], (long long)window[3], (long long)window[4]);
     printf("invalid %d '%s'\n", nanoep_dispatch(NULL, NULL, NULL, NULL, NULL, NULL, 0, NULL, NULL, 0, 0, 0, 7, 2, 4, 1, 0, 0, NULL, NULL, NULL, 0, NULL),
            nanoep_status_string(NANOEP_ERR_INVALID_ARGUMENT));
-    printf("sizes %lld %d %lu\n", (long long)nanoep_slot_order_entries(4096, 8, 256), nanoep_layout_block_tokens(4096, 256),
+    printf("sizes %lld %d %lu\n", (long long)nanoep_slot_order_entries(4096, 8, 256), nanoep_layout_block_tokens(4096, 256, 7168),
            (unsigned long)(nanoep_layout_workspace_bytes(4096, 8, 256) > 0));
     return 0;
 }

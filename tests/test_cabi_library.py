@@ -23,7 +23,7 @@ def test_every_declared_symbol_is_exported():
 
 def test_version_and_status_strings():
     library = cabi.lib()
-    assert library.nanoep_abi_version() == 2
+    assert library.nanoep_abi_version() == 3
     texts = [library.nanoep_status_string(code).decode() for code in range(0, 7)]
     assert texts[0] == "ok" and len(set(texts[:6])) == 6 and texts[6] == "unknown status"
     assert library.nanoep_last_hip_error().decode() == ""
@@ -64,14 +64,21 @@ def test_argument_checks_come_before_any_device_work():
     assert library.nanoep_combine(null, null, null, null, null, null, 0, 0, 0, 250, 2, 1, 0, null, null, 0, null) == 1
     assert library.nanoep_combine(null, null, null, null, null, null, 3, 0, 2, 256, 2, 1, 0, null, null, 0, null) == 1
     assert library.nanoep_copy_bytes(null, null, 24, null) == 1
-    assert library.nanoep_layout(null, -1, 2, 4, 1, 0, null, null, null, null, null, null, null, null, null, null, 0, null, null) == 1
-    assert library.nanoep_layout(null, 4, 2, 4, 0, 0, null, null, null, null, null, null, null, null, null, null, 0, null, null) == 1
+    assert library.nanoep_layout(null, -1, 2, 4, 1, 0, 0, null, null, null, null, null, null, null, null, null, null, 0, null, null) == 1
+    assert library.nanoep_layout(null, 4, 2, 4, 0, 0, 0, null, null, null, null, null, null, null, null, null, null, 0, null, null) == 1
     # a slot-order list only exists for the expanded layout
-    assert library.nanoep_layout(null, 4, 2, 4, 1, 0, null, 8, 8, null, 8, null, 8, null, 8, 8, 0, 8, null) == 1
-    assert library.nanoep_slot_order_entries(4096, 8, 256) == 4096 * 8 + 1 and library.nanoep_layout_block_tokens(4096, 256) == 256
-    assert library.nanoep_slot_order_entries(100, 3, 8) == 256 * 3 + 1 and library.nanoep_slot_order_entries(0, 3, 8) == 0
-    assert library.nanoep_layout_block_tokens(4096, 6000) == 0 and library.nanoep_layout_block_tokens(4096, 0) == 0
-    assert [library.nanoep_layout_block_tokens(t, 256) for t in (1, 256, 257, 512, 1024, 1536, 1792, 1793, 2048, 100000)] == [256, 256, 64, 64, 128, 128, 128, 256, 256, 256]
+    assert library.nanoep_layout(null, 4, 2, 4, 1, 0, 0, null, 8, 8, null, 8, null, 8, null, 8, 8, 0, 8, null) == 1
+    assert library.nanoep_slot_order_entries(4096, 8, 256) == 4096 * 8 + 1 and library.nanoep_layout_block_tokens(4096, 256, 0) == 256
+    assert library.nanoep_slot_order_entries(100, 3, 8) == 512 * 3 + 1 and library.nanoep_slot_order_entries(0, 3, 8) == 0
+    assert library.nanoep_layout_block_tokens(4096, 6000, 0) == 0 and library.nanoep_layout_block_tokens(4096, 0, 0) == 0
+    sizes = (1, 256, 257, 512, 1024, 1536, 1792, 1793, 2048, 4095, 4096, 100000)
+    assert [library.nanoep_layout_block_tokens(t, 256, 0) for t in sizes] == [256, 256, 64, 64, 128, 128, 128, 256, 256, 256, 256, 256]
+    assert [library.nanoep_layout_block_tokens(t, 256, 7168) for t in sizes] == [256, 256, 64, 64, 128, 128, 128, 256, 256, 256, 256, 256]
+    # rows of up to 4096 elements: 512-token blocks fit an XCD's L2, once there are eight of them
+    assert [library.nanoep_layout_block_tokens(t, 256, 4096) for t in sizes] == [256, 256, 64, 64, 128, 128, 128, 256, 256, 512, 512, 512]
+    assert [library.nanoep_layout_block_tokens(100000, 256, h) for h in (8, 2048, 4104, 8192, 8200, 16384, 16392, 1 << 20)] == [512, 512, 256, 256, 128, 128, 64, 64]
+    assert library.nanoep_layout_block_tokens(100000, 700, 2048) == 256  # 512-token blocks of 701 LDS rows do not fit
+    assert library.nanoep_layout_block_tokens(4096, 256, -1) == 0
     out = (ctypes.c_int64 * 4)()
     assert library.nanoep_wait_counts(null, null, 0.0, out) == 1
 
@@ -88,6 +95,6 @@ def test_plain_c_client_compiles_links_and_runs(tmp_path):
         check=True, capture_output=True, text=True,
     )
     out = subprocess.run([str(binary)], check=True, capture_output=True, text=True, timeout=60).stdout.splitlines()
-    assert out[0] == "abi 2 status 0 window 0 96 160 160 9888"
+    assert out[0] == "abi 3 status 0 window 0 96 160 160 9888"
     assert out[1].startswith("invalid 1 '") and "invalid" in out[1].lower()
     assert out[2] == "sizes 32769 256 1"

@@ -28,7 +28,7 @@ def assert_bits_equal(actual, expected, what):
     assert torch.equal(bits(actual.cpu()), bits(expected)), f"{what}: bit mismatch"
 
 
-def assert_layout(metadata, counts, expected: oracle.Layout, expand):
+def assert_layout(metadata, counts, expected: oracle.Layout, expand, hidden=0):
     assert counts[0] == expected.recv_count and counts[1] == expected.expanded_capacity
     assert counts[2] == int(expected.expert_counts.sum()) and counts[3] == 0
     for actual, want, name in zip(
@@ -47,7 +47,7 @@ def assert_layout(metadata, counts, expected: oracle.Layout, expand):
         # private slot-order list: block of consecutive tokens by block, the valid assignments as
         # (slot << 32) | (t * K + k) in ascending slot order, without gaps; -1 from entry A on
         tokens, topk = expected.topk_idx.shape
-        block_tokens = cabi.lib().nanoep_layout_block_tokens(tokens, expected.expert_counts.numel())
+        block_tokens = cabi.lib().nanoep_layout_block_tokens(tokens, expected.expert_counts.numel(), hidden)
         flat = table.flatten().to(torch.int64)
         packed = (flat << 32) | torch.arange(flat.numel(), dtype=torch.int64)
         want = []
@@ -55,11 +55,15 @@ def assert_layout(metadata, counts, expected: oracle.Layout, expand):
             part = packed[first * topk : (first + block_tokens) * topk]
             want.append(part[flat[first * topk : (first + block_tokens) * topk] >= 0].sort().values)
         entries = cabi.lib().nanoep_slot_order_entries(tokens, topk, expected.expert_counts.numel())
+        got = metadata[8].cpu()
+        assert got.numel() == entries == ((tokens + 511) // 512 * 512 * topk + 1 if tokens else 0)
         if entries:
-            want.append(torch.full((entries - 1 - counts[2],), -1, dtype=torch.int64))
-            want.append(torch.tensor([counts[2]], dtype=torch.int64))  # count word behind the list
-        want = torch.cat(want) if want else torch.empty(0, dtype=torch.int64)
-        assert torch.equal(metadata[8].cpu(), want), "slot_order"
+            blocks = (tokens + block_tokens - 1) // block_tokens
+            want.append(torch.full((blocks * block_tokens * topk - counts[2],), -1, dtype=torch.int64))
+            want = torch.cat(want)
+            assert torch.equal(got[: want.numel()], want), "slot_order"
+            assert (got[want.numel() : -1] == -7).all(), "the buffer behind the last block is not written"
+            assert int(got[-1]) == counts[2], "count word at the end of the buffer"
 
 
 def run_dispatch_combine(device, idx, hidden, experts, alignment, expand, zero_padding, weighted, *, seed=0, num_cus=0):
@@ -67,8 +71,8 @@ def run_dispatch_combine(device, idx, hidden, experts, alignment, expand, zero_p
     x = cases.payload(tokens, hidden, seed=123 + seed)
     w = cases.gate_weights(tokens, topk, seed=7 + seed) if weighted else None
     expected_layout = oracle.layout(idx, experts, alignment)
-    metadata, counts = cabi.layout(idx.to(device), experts, alignment, expand)
-    assert_layout(metadata, counts, expected_layout, expand)
+    metadata, counts = cabi.layout(idx.to(device), experts, alignment, expand, hidden=hidden)
+    assert_layout(metadata, counts, expected_layout, expand, hidden)
     want_x, want_idx, want_w, _ = oracle.dispatch(x, idx, experts, w, do_expand=expand, alignment=alignment, lay=expected_layout)
     got_x, got_idx, got_w = cabi.dispatch(
         x.to(device), None if w is None else w.to(device), metadata, counts, experts, alignment, expand, zero_padding,
@@ -291,7 +295,7 @@ def test_rows_beyond_four_gib(device, tokens, hidden, experts, topk, expand, ali
     x = torch.randint(-4, 5, (tokens, hidden), device=device, generator=g).to(torch.bfloat16)
     w = torch.rand(tokens, topk, device=device, generator=g)
 
-    metadata, counts = cabi.layout(idx, experts, alignment, expand)
+    metadata, counts = cabi.layout(idx, experts, alignment, expand, hidden=hidden)
     slots, expert_counts, capacity = closed_form_slots(idx, experts, alignment)
     sent = (idx >= 0).any(dim=1)
     assert counts[0] == int(sent.sum()) and counts[1] == capacity and counts[2] == int((idx >= 0).sum()) and counts[3] == 0
@@ -342,13 +346,14 @@ def test_topk_range(device, topk, experts, hidden, expand):
     [(1000, 16, 4, "mixed", 8), (4096, 256, 8, "dropout", 1), (700, 1500, 9, "sparse", 3), (2049, 8, 2, "skew", 128), (5000, 40, 17, "random", 1)],
 )
 @pytest.mark.parametrize("expand", [False, True], ids=["compact", "expanded"])
-def test_both_layout_launch_plans(device, monkeypatch, launches, tokens, experts, topk, kind, alignment, expand):
+@pytest.mark.parametrize("hidden", [0, 2048, 16384], ids=["blocks-256", "blocks-512", "blocks-128"])
+def test_both_layout_launch_plans(device, monkeypatch, hidden, launches, tokens, experts, topk, kind, alignment, expand):
     """The layout runs as two launches (every block scans the block histograms itself) or three
     (single-workgroup scan), chosen by size; both plans must give the oracle's handle."""
     monkeypatch.setenv("NANOEP_LAYOUT_LAUNCHES", launches)
     idx = cases.routing(kind, tokens, experts, topk, seed=5)
-    metadata, counts = cabi.layout(idx.to(device), experts, alignment, expand)
-    assert_layout(metadata, counts, oracle.layout(idx, experts, alignment), expand)
+    metadata, counts = cabi.layout(idx.to(device), experts, alignment, expand, hidden=hidden)
+    assert_layout(metadata, counts, oracle.layout(idx, experts, alignment), expand, hidden)
 
 
 @pytest.mark.parametrize("seed", range(24))
