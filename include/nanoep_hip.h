@@ -63,11 +63,11 @@ size_t nanoep_layout_workspace_bytes(int64_t num_tokens, int num_topk, int64_t n
 /* Tokens per block of the routing layout for T tokens, L local experts and payload rows of
  * `hidden` bf16 elements (0: not known; the answer is 0 when L is not supported).  The slot-order
  * list is ordered block of consecutive tokens by block, and a block's rows should fit one XCD's 4 MiB
- * L2: 512 tokens up to hidden 4096, 256 up to 8192 (and when hidden is not known), then 128 and 64;
- * fewer for very many experts, and for batches of 257..4095 tokens so that there are eight blocks. */
+ * L2: 256 tokens up to hidden 8192 (and when hidden is not known), then 128 and 64; fewer for very
+ * many experts, and for batches of 257..2047 tokens so that there are eight blocks. */
 int nanoep_layout_block_tokens(int64_t num_tokens, int64_t num_local_experts, int hidden);
 
-/* Number of int64 words of the slot-order buffer for (T, K, L): T rounded up to 512, times K
+/* Number of int64 words of the slot-order buffer for (T, K, L): T rounded up to 256, times K
  * entries (an upper bound of the A that carry assignments), then one word holding A.  0 when T == 0. */
 int64_t nanoep_slot_order_entries(int64_t num_tokens, int num_topk, int64_t num_local_experts);
 

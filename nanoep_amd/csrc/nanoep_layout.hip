@@ -8,14 +8,16 @@ namespace nanoep {
 namespace {
 
 // Largest block of tokens a layout workgroup handles (one thread per token).
-constexpr int kMaxBlockTokens = 512;
+constexpr int kMaxBlockTokens = 256;
 // An XCD's L2: the rows of one token block should fit it, since the dispatch walks the slot-order
 // list block by block and wants every re-use of a source row to hit that cache.
 constexpr int64_t kXcdL2Bytes = int64_t{4} << 20;
 
 // Tokens handled by one layout workgroup = tokens of one block of the slot-order list.
 //  * `hidden` (bf16 elements of a payload row, 0 = not known) sizes the block so that its rows fit an
-//    XCD's L2: 512 tokens up to 4096 elements, 256 up to 8192 (and when it is not known), 128, 64.
+//    XCD's L2: 256 tokens up to 8192 elements (and when it is not known), then 128 and 64.  (Blocks
+//    of 512 tokens for rows of up to 4096 elements make the dispatch 1-4 % faster and the layout
+//    itself 5 us slower: half as many workgroups, each with a longer chain.)
 //  * The LDS bit matrix has (L+1) rows of tokens/32 words plus a 16-bit prefix per word, so the block
 //    shrinks as the expert count grows.
 //  * The dispatch hands every XCD whole token blocks when there are at least eight of them: batches
@@ -28,8 +30,6 @@ int layout_tokens_per_block(int64_t tokens_total, int64_t local_experts, int hid
     if (hidden > 0)
         for (largest = kMaxBlockTokens; largest > 64 && static_cast<int64_t>(largest) * hidden * 2 > kXcdL2Bytes; largest /= 2) {
         }
-    if (tokens_total <= 256 && largest > 256)
-        largest = 256;
     int chosen = 0;
     for (int tokens = largest; tokens >= 32; tokens /= 2) {
         const size_t words = static_cast<size_t>(tokens / 32);
@@ -80,8 +80,8 @@ LayoutWorkspace carve_layout_workspace(void* base, int64_t tokens, int topk, int
 }
 
 // A (token, k) entry of the rank table packs (expert << kRankBits) | in-block rank; -1 marks a
-// masked choice.  A layout block never holds more than 512 tokens, so the rank fits 9 bits.
-constexpr int kRankBits = 9;
+// masked choice.  A layout block never holds more than 256 tokens, so the rank fits 8 bits.
+constexpr int kRankBits = 8;
 static_assert(kMaxBlockTokens <= (1 << kRankBits), "in-block ranks must fit the packed entry");
 constexpr int kRankMask = (1 << kRankBits) - 1;
 
