@@ -1,7 +1,7 @@
 """Seeded synthetic routing / payload generators shared by the CPU and GPU tests.
 
 Kinds follow the reference's make_case vocabulary (nano_ep/testing/cases.py:29-55: random, masked,
-skew, mixed) plus the BASELINE configurations (dropout mask, Zipf popularity, biased logits)."""
+skew, mixed) plus the benchmark workloads' routing (dropout mask, Zipf popularity, biased logits)."""
 
 from __future__ import annotations
 

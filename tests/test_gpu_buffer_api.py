@@ -3,7 +3,7 @@
 The cases restate what the reference checks at world_size == 1: the README round trip
 (README.md:44-70), fresh + cached replay with pointer-stable metadata and untouched earlier results
 (tests/native/test_native_dispatch.py:93-208), async_op / previous_event stream handling and the
-exact multiplicity round trip (tests/distributed/worker.py:180-343), plus the five BASELINE shapes.
+exact multiplicity round trip (tests/distributed/worker.py:180-343), plus the five benchmark shapes of nanoep_amd/workloads.py.
 """
 
 import pytest
@@ -68,7 +68,7 @@ def assert_dispatch_result(result, x, idx, weights, experts, expand, alignment, 
 
 
 def test_readme_round_trip(device):
-    """BASELINE config 1: identity experts weighted once, combine reproduces x."""
+    """The README toy shape (16 x 256, two experts, top-2): identity experts weighted once, combine reproduces x."""
     config = EPConfig(num_experts=2, num_topk=2, hidden=256, num_max_tokens_per_rank=16)
     x = cases.payload(16, 256, seed=0).to(device)
     indices = torch.tensor([[0, 1]], dtype=torch.int64).repeat(16, 1).to(device)
