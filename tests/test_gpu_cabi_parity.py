@@ -379,6 +379,29 @@ def test_randomized_shapes(device, seed):
     run_dispatch_combine(device, idx, hidden, experts, alignment, expand, zero_padding, weighted, seed=seed)
 
 
+@pytest.mark.parametrize("seed", range(10))
+def test_randomized_multi_block_shapes(device, seed):
+    """Seeded batches of a thousand to nine thousand tokens (many layout blocks, token counts that
+    are no multiple of a block, both layout plans by size, rows of 512 bytes to 18 KiB), checked bit
+    for bit against the oracle through all walks."""
+    g = torch.Generator().manual_seed(7000 + seed)
+
+    def pick(options):
+        return options[int(torch.randint(len(options), (1,), generator=g))]
+
+    topk = pick([1, 2, 4, 6, 8, 9, 16])
+    experts = max(topk, pick([8, 32, 64, 160, 256, 384, 1000]))
+    tokens = pick([1000, 2047, 2048, 3000, 4097, 6000, 8192, 9001])
+    hidden = pick([256, 512, 1024, 2048, 2816, 4096, 7168, 8192, 9216])
+    alignment = pick([1, 1, 8, 128])
+    kind = pick(["random", "dropout", "sparse", "biased"])
+    expand = pick([True, True, False])
+    zero_padding = expand and pick([False, True])
+    weighted = pick([False, True])
+    idx = cases.routing(kind, tokens, experts, topk, seed=100 + seed)
+    run_dispatch_combine(device, idx, hidden, experts, alignment, expand, zero_padding, weighted, seed=seed)
+
+
 def test_empty_inputs(device):
     for expand in (False, True):
         idx = torch.empty((0, 4), dtype=torch.int64)
