@@ -6,6 +6,8 @@ The cases restate what the reference checks at world_size == 1: the README round
 exact multiplicity round trip (tests/distributed/worker.py:180-343), plus the five benchmark shapes of nanoep_amd/workloads.py.
 """
 
+import dataclasses
+
 import pytest
 import torch
 from torch.utils import deterministic
@@ -147,6 +149,48 @@ def test_fresh_and_cached_replay(device, monkeypatch, walk, expand, zero_padding
         want, want_w = oracle.combine(y, lay.recv_metadata(expand), lay.dst_slots, do_expand=expand, weights=yw, bias=bias)
         assert_same_bits(result.x, want, "combined x")
         assert_same_bits(result.topk_weights, want_w, "combined weights")
+    finally:
+        buffer.close()
+
+
+@pytest.mark.parametrize(
+    "tokens,hidden,switch",
+    [
+        pytest.param(2048, 4096, None, id="16MiB-rebuilds-by-itself"),
+        pytest.param(37, 512, "1", id="small-forced-rebuild"),
+        pytest.param(2048, 4096, "0", id="16MiB-token-order-forced"),
+    ],
+)
+def test_replay_with_only_the_reference_handle_tensors(device, monkeypatch, tokens, hidden, switch):
+    """A handle that carries just the reference's seven tensors (as one that went through the
+    reference's own Python class would) replays to the same bytes: the extension makes the private
+    slot-order list again on the device for large payloads, or walks in token order."""
+    if switch is not None:
+        monkeypatch.setenv("NANOEP_REBUILD_ORDER", switch)
+    experts, topk, alignment = 16, 4, 8
+    idx = cases.routing("dropout", tokens, experts, topk, seed=9)
+    x, w = cases.payload(tokens, hidden, seed=4), cases.gate_weights(tokens, topk)
+    buffer = Buffer(None, EPConfig(experts, topk, hidden, tokens))
+    try:
+        fresh = buffer.dispatch(x.to(device), topk_idx=idx.to(device), weights=w.to(device), do_expand=True,
+                                alignment=alignment, zero_padding=True)
+        bare = dataclasses.replace(fresh.handle, token_slots=None, slot_order=None)
+        for step in (1, 2):
+            new_x, new_w = x * step + 1, w - step
+            replay = buffer.dispatch(new_x.to(device), weights=new_w.to(device), handle=bare, zero_padding=True)
+            assert replay.handle is bare
+            assert_dispatch_result(replay, new_x, idx, new_w, experts, True, alignment, True)
+            full = buffer.dispatch(new_x.to(device), weights=new_w.to(device), handle=fresh.handle, zero_padding=True)
+            assert torch.equal(replay.x.view(torch.int16), full.x.view(torch.int16))
+            assert torch.equal(replay.topk_weights.view(torch.int32), full.topk_weights.view(torch.int32))
+        # a fresh dispatch after such replays still reads its own counts
+        again = buffer.dispatch(x.to(device), topk_idx=idx.flip(0).contiguous().to(device), do_expand=True, alignment=alignment)
+        lay = oracle.layout(idx.flip(0).contiguous(), experts, alignment)
+        assert again.handle.layout.recv_count == lay.recv_count and again.handle.layout.expanded_capacity == lay.expanded_capacity
+        combined = buffer.combine(full.x, bare)
+        want, _ = oracle.combine(full.x.cpu(), oracle.layout(idx, experts, alignment).recv_metadata(True),
+                                 oracle.layout(idx, experts, alignment).dst_slots, do_expand=True)
+        assert_same_bits(combined.x, want, "combine through the bare handle")
     finally:
         buffer.close()
 
