@@ -1,183 +1,140 @@
-"""Python surface of the dispatch / combine buffer for one rank on one MI355X.
+"""The buffer object: `CudaBuffer.dispatch` / `.combine` / `.close` for one rank on one MI355X.
 
-Keeps the reference's public API (nano_ep/backends/cuda.py:23-444): the result and handle
-dataclasses, `CudaBuffer(group, config, *, allow_multiple_reduction)`, `dispatch`, `combine`,
-`close`, and `CudaEvent.current_stream_wait()`, with the same keyword arguments, validation order
-and exception types, so code written against `nano_ep` runs on PyTorch-ROCm with world_size == 1.
-Everything below the `self._backend.dispatch / combine` calls is the native extension.
+The call surface is the reference's (`CudaBuffer` in nano_ep/backends/cuda.py:90-444): the same
+keyword arguments, the same order of argument checks, `ValueError` for misuse of arguments and
+handles, `RuntimeError` for a closed buffer and for the deterministic-fill conflict, `TypeError`
+for a non-bool `allow_multiple_reduction`.  What differs is underneath: there is no peer window,
+no collective bootstrap and no JIT; every call ends in one native call of `_nanoep_torch`.
 """
 
 from __future__ import annotations
-
-from dataclasses import dataclass
 
 import torch
 from torch.utils import deterministic
 
 from ._native import load_extension
 from .config import EPConfig
+from .handles import CudaEvent, NativeCombineResult, NativeDispatchResult, NativeHandle, NativeLayout
+
+__all__ = [
+    "Buffer",
+    "CudaBuffer",
+    "CudaEvent",
+    "NativeCombineResult",
+    "NativeDispatchResult",
+    "NativeHandle",
+    "NativeLayout",
+    "check_torch_deterministic",
+]
+
+# The reference's row-width contract (nano_ep/backends/cuda.py:104-105); the kernels need H % 8.
+HIDDEN_MULTIPLE = 256
 
 
 def check_torch_deterministic():
-    """Same refusal as the reference (nano_ep/backends/cuda.py:16-20)."""
-    if torch.are_deterministic_algorithms_enabled() and deterministic.fill_uninitialized_memory:
+    """Deterministic mode fills every new tensor; the outputs here are allocated uninitialised and
+    written exactly once by the kernels, so the combination is refused as the reference refuses it
+    (nano_ep/backends/cuda.py:16-20)."""
+    filling = torch.are_deterministic_algorithms_enabled() and deterministic.fill_uninitialized_memory
+    if filling:
         raise RuntimeError(
             "NanoEP does not support deterministic algorithms with fill_uninitialized_memory enabled; "
             "disable one of these PyTorch settings"
         )
 
 
-@dataclass
-class NativeLayout:
-    recv_metadata: torch.Tensor  # int32 [N, K+2]: src_rank, src_token, K x (local expert id | expanded slot | -1)
-    expert_counts: torch.Tensor  # int64 [L]
-    expert_offsets: torch.Tensor  # int64 [L+1], padded exclusive offsets ending at C
-    recv_rank_prefix: torch.Tensor  # int64 [R]
-    recv_count: int  # N
-    expanded_capacity: int  # C
+def _plain_int(value) -> bool:
+    return isinstance(value, int) and not isinstance(value, bool)
 
 
-@dataclass
-class NativeHandle:
-    config: EPConfig
-    rank: int
-    world_size: int
-    do_expand: bool
-    alignment: int
-    topk_idx: torch.Tensor  # int64 [T, K] routing snapshot
-    layout: NativeLayout
-    dst_slots: torch.Tensor  # int64 [T, R]
-    send_counts: torch.Tensor  # int64 [R]
-    owner: object
-    x_dtype: torch.dtype
-    num_sms: int | None = None
-    # int32 [T, K] slot of every (token, k), -1 when masked: the same mapping as dst_slots +
-    # recv_metadata in one lookup.  Only expanded handles made by this package carry it.
-    token_slots: torch.Tensor | None = None
-    # int64 list of every valid assignment as (slot << 32) | (t * K + k), one segment per block of
-    # consecutive tokens, ascending slot inside a segment, -1 in unused entries: the order in which
-    # a replayed dispatch walks its work.  Only expanded handles made by this package carry it.
-    slot_order: torch.Tensor | None = None
-
-
-@dataclass
-class NativeDispatchResult:
-    x: torch.Tensor
-    topk_idx: torch.Tensor | None
-    topk_weights: torch.Tensor | None
-    handle: NativeHandle
-    event: "CudaEvent | None"
-
-
-@dataclass
-class NativeCombineResult:
-    x: torch.Tensor
-    topk_weights: torch.Tensor | None
-    event: "CudaEvent | None"
-
-
-class CudaEvent:
-    def __init__(self, event, keepalive: tuple = ()):
-        self.event = event
-        self.keepalive = keepalive
-
-    def current_stream_wait(self):
-        """Wait on the consumer stream and protect tensors used on that stream."""
-        self.event.current_stream_wait()
+def _raw_event(previous_event) -> int:
+    """Raw event handle for the native call, -1 for none."""
+    return previous_event.cuda_event if previous_event is not None else -1
 
 
 def _handle_metadata(handle: NativeHandle) -> list[torch.Tensor]:
-    layout = handle.layout
-    metadata = [
-        layout.recv_metadata,
-        layout.expert_counts,
-        layout.expert_offsets,
-        handle.dst_slots,
-        handle.send_counts,
-        handle.topk_idx,
-        layout.recv_rank_prefix,
-    ]
-    if getattr(handle, "token_slots", None) is not None:
-        metadata.append(handle.token_slots)
-        if getattr(handle, "slot_order", None) is not None:
-            metadata.append(handle.slot_order)
-    return metadata
+    return NativeHandle.tensors(handle)
 
 
 class CudaBuffer:
+    """One rank's dispatch / combine endpoint.  `Buffer` is the same class."""
+
     def __init__(self, group, config: EPConfig, *, allow_multiple_reduction: bool = False):
-        """Create the buffer and its communication stream.
-
-        `group` is None or a torch.distributed Gloo group of size 1: this build runs one rank on
-        one GPU, so the reference's collective bootstrap (nano_ep/backends/cuda.py:90-231) reduces
-        to local checks.
-        """
-        self._group = group
-        self._config = config
+        """`group` is None or a torch.distributed Gloo group with a single member: with one rank
+        the reference's collective bootstrap (nano_ep/backends/cuda.py:90-231) comes down to the
+        local checks below."""
+        self._closed = True  # until everything below has succeeded
+        self._runtime = self._comm_stream = None
+        self._group, self._config = group, config
         self._allow_multiple_reduction = allow_multiple_reduction
-        self._world_size = 1
-        self._rank = 0
-        self._runtime = None
-        self._comm_stream = None
-        self._closed = True
-        if group is not None:
-            import torch.distributed as dist
+        self._rank, self._world_size = self._inspect_group(group)
 
-            if dist.get_backend(group) != "gloo":
-                raise ValueError("CudaBuffer requires a Gloo control group")
-            if dist.get_world_size(group=group) != 1:
-                raise ValueError("this build runs one rank on one GPU: the control group must have world_size == 1")
-            self._rank = dist.get_rank(group=group)
         if not isinstance(allow_multiple_reduction, bool):
             raise TypeError("allow_multiple_reduction must be bool")
         if not torch.cuda.is_available():
             raise RuntimeError("CudaBuffer environment check failed: no GPU is visible to PyTorch-ROCm")
-        if config.num_experts % self._world_size != 0:
+        if config.num_experts % self._world_size:
             raise ValueError("num_experts must be divisible by world_size")
-        if config.hidden % 256 != 0:
-            raise ValueError("CUDA EP hidden must be a positive multiple of 256")
+        if config.hidden % HIDDEN_MULTIPLE:
+            raise ValueError(f"CUDA EP hidden must be a positive multiple of {HIDDEN_MULTIPLE}")
 
         self._device = torch.cuda.current_device()
-        properties = torch.cuda.get_device_properties(self._device)
-        self._device_sms = properties.multi_processor_count
-        self._gpu_uuids = (str(getattr(properties, "uuid", self._device)),)
+        card = torch.cuda.get_device_properties(self._device)
+        self._device_sms = card.multi_processor_count
+        self._gpu_uuids = (str(getattr(card, "uuid", self._device)),)
         self._auto_num_sms = None
 
         self._backend = load_extension()
-        (
-            self._signal_offset,
-            self._count_offset,
-            self._payload_offset,
-            self._return_offset,
-            self._num_bytes,
-        ) = self._backend.window_layout(
-            self._world_size,
-            config.num_max_tokens_per_rank,
-            config.hidden,
-            config.num_topk,
-            config.num_experts,
+        # The window geometry is computed for callers that ask for it; no window is allocated,
+        # since with one rank rows go straight from the source tensor to the exact-shaped outputs.
+        offsets = self._backend.window_layout(
+            self._world_size, config.num_max_tokens_per_rank, config.hidden, config.num_topk, config.num_experts,
             allow_multiple_reduction,
         )
-        # No peer window is allocated: with one rank, rows go straight from the source tensor to
-        # the exact-shaped outputs.  The runtime owns the device id and the host count mailbox.
+        self._signal_offset, self._count_offset, self._payload_offset, self._return_offset, self._num_bytes = offsets
+        # The runtime owns the device id and the pinned mailbox the layout kernels report N and C in.
         self._runtime = self._backend.PeerRuntime(self._rank, self._world_size, self._num_bytes)
         self._handle = self._runtime.export_local_handle()
         self._runtime.import_peer_handles([self._handle])
         self._comm_stream = torch.cuda.Stream(device=self._device)
         self._closed = False
 
-    def _resolve_num_sms(self, num_sms: int | None, handle: NativeHandle | None) -> int:
+    @staticmethod
+    def _inspect_group(group) -> tuple[int, int]:
+        """(rank, world_size) of the control group; only a single-member Gloo group is accepted."""
+        if group is None:
+            return 0, 1
+        import torch.distributed as dist
+
+        if dist.get_backend(group) != "gloo":
+            raise ValueError("CudaBuffer requires a Gloo control group")
+        if dist.get_world_size(group=group) != 1:
+            raise ValueError("this build runs one rank on one GPU: the control group must have world_size == 1")
+        return dist.get_rank(group=group), 1
+
+    # ------------------------------------------------------------------ shared argument handling
+
+    def _require_open(self) -> None:
+        if self._closed:
+            raise RuntimeError("CudaBuffer is closed")
+
+    def _resolve_num_sms(self, num_sms, handle) -> int:
+        """The compute-unit budget of a call: an explicit number, else the handle's, else the whole
+        device.  0 asks for the automatic choice, which without peers is the whole device as well
+        (nano_ep/backends/_sms.py:50-51)."""
+        whole = self._device_sms
         if num_sms is None:
-            return self._device_sms if handle is None or handle.num_sms is None else handle.num_sms
-        if isinstance(num_sms, bool) or not isinstance(num_sms, int) or not 0 <= num_sms <= self._device_sms:
-            raise ValueError(f"num_sms must be an integer between 0 and {self._device_sms}")
-        if num_sms > 0:
+            inherited = None if handle is None else handle.num_sms
+            return whole if inherited is None else inherited
+        if not _plain_int(num_sms) or num_sms < 0 or num_sms > whole:
+            raise ValueError(f"num_sms must be an integer between 0 and {whole}")
+        if num_sms:
             return num_sms
         if self._auto_num_sms is None:
-            # The reference's link-bandwidth model returns the whole device when there are no peers
-            # (nano_ep/backends/_sms.py:50-51).
-            self._auto_num_sms = self._device_sms
+            self._auto_num_sms = whole
         return self._auto_num_sms
+
+    # ------------------------------------------------------------------ dispatch
 
     def dispatch(
         self,
@@ -193,99 +150,99 @@ class CudaBuffer:
         async_op: bool = False,
         num_sms: int | None = None,
     ) -> NativeDispatchResult:
-        "Dispatch payloads using fresh or cached routing; return exact receive layouts."
+        """Send token rows to their experts' receive layout.
+
+        Fresh: pass `topk_idx` (int64 [T, K], ids or -1); the result carries a handle.  Cached:
+        pass that `handle` instead; its routing snapshot, layout and alignment are reused and only
+        the payload (and weights) are new.  `do_expand=True` gives one row per (token, choice) in
+        expert-major slots padded to `alignment`, otherwise one row per received token.
+        """
         check_torch_deterministic()
-        if self._closed:
-            raise RuntimeError("CudaBuffer is closed")
-        if handle is not None:
-            if handle.owner is not self:
-                raise ValueError("cached handle belongs to another CudaBuffer")
-            if topk_idx is not None:
-                raise ValueError("cached dispatch uses the handle snapshot; omit topk_idx")
-            if alignment is not None and alignment != handle.alignment:
-                raise ValueError("cached dispatch must retain the handle alignment")
-            if do_expand is not None and do_expand != handle.do_expand:
-                raise ValueError("cached dispatch must retain the handle layout")
+        self._require_open()
+        replay = handle is not None
+        if replay:
+            self._check_replay_arguments(handle, topk_idx, alignment, do_expand)
         elif topk_idx is None:
             raise ValueError("fresh dispatch requires topk_idx")
-        if alignment is not None and (isinstance(alignment, bool) or not isinstance(alignment, int) or alignment <= 0):
+        if alignment is not None and not (_plain_int(alignment) and alignment > 0):
             raise ValueError("alignment must be a positive integer")
-        if do_expand is not None and not isinstance(do_expand, bool):
+        if not (do_expand is None or isinstance(do_expand, bool)):
             raise ValueError("do_expand must be bool or None")
 
-        routing = handle.topk_idx if handle is not None else topk_idx
-        if x.shape[1] != self._config.hidden:
+        geometry = self._config
+        routing = handle.topk_idx if replay else topk_idx
+        if x.shape[1] != geometry.hidden:
             raise ValueError("x hidden dimension does not match the buffer configuration")
-        if routing.shape != (x.shape[0], self._config.num_topk):
+        if tuple(routing.shape) != (x.shape[0], geometry.num_topk):
             raise ValueError("routing snapshot/topk_idx shape must match the buffer configuration")
 
-        if handle is None:
-            expand = False if do_expand is None else do_expand
-            expert_alignment = 1 if alignment is None else alignment
-            cached_metadata = []
-            cached_expanded_capacity = 0
+        if replay:
+            expand, slot_alignment = handle.do_expand, handle.alignment
+            known_tensors, known_capacity = _handle_metadata(handle), handle.layout.expanded_capacity
         else:
-            expand = handle.do_expand
-            expert_alignment = handle.alignment
-            cached_expanded_capacity = handle.layout.expanded_capacity
-            cached_metadata = _handle_metadata(handle)
+            expand, slot_alignment = bool(do_expand), (alignment or 1)
+            known_tensors, known_capacity = [], 0
 
-        main_sms = self._resolve_num_sms(num_sms, handle)
-        outputs, metadata, counts, completed = self._backend.dispatch(
-            self._runtime,
-            x,
-            routing,
-            weights,
-            self._config.num_experts,
-            self._config.num_max_tokens_per_rank,
-            expert_alignment,
-            cached_metadata,
-            cached_expanded_capacity,
-            self._allow_multiple_reduction,
-            expand,
-            zero_padding,
-            main_sms,
-            self._comm_stream.cuda_stream,
-            -1 if previous_event is None else previous_event.cuda_event,
-            async_op,
+        budget = self._resolve_num_sms(num_sms, handle)
+        outputs, metadata, (received, capacity), completed = self._backend.dispatch(
+            self._runtime, x, routing, weights,
+            geometry.num_experts, geometry.num_max_tokens_per_rank, slot_alignment,
+            known_tensors, known_capacity,
+            self._allow_multiple_reduction, expand, zero_padding, budget,
+            self._comm_stream.cuda_stream, _raw_event(previous_event), async_op,
         )
-        recv_count, expanded_capacity = counts
+        if not replay:
+            handle = self._new_handle(metadata, received, capacity, expand, slot_alignment, x.dtype, budget)
 
-        if handle is None:
-            layout = NativeLayout(
-                recv_metadata=metadata[0],
-                expert_counts=metadata[1],
-                expert_offsets=metadata[2],
-                recv_rank_prefix=metadata[6],
-                recv_count=recv_count,
-                expanded_capacity=expanded_capacity,
-            )
-            handle = NativeHandle(
-                config=self._config,
-                rank=self._rank,
-                world_size=self._world_size,
-                do_expand=expand,
-                alignment=expert_alignment,
-                topk_idx=metadata[5],
-                layout=layout,
-                dst_slots=metadata[3],
-                send_counts=metadata[4],
-                owner=self,
-                x_dtype=x.dtype,
-                num_sms=main_sms,
-                token_slots=metadata[7] if len(metadata) > 7 else None,
-                slot_order=metadata[8] if len(metadata) > 8 else None,
-            )
-
-        event = CudaEvent(completed, keepalive=(self, x, routing, weights, handle)) if async_op else None
-
+        payload, local_ids, gate = outputs
         return NativeDispatchResult(
-            x=outputs[0],
-            topk_idx=None if expand else outputs[1],
-            topk_weights=outputs[2] if weights is not None else None,
+            x=payload,
+            topk_idx=None if expand else local_ids,
+            topk_weights=None if weights is None else gate,
             handle=handle,
-            event=event,
+            event=CudaEvent(completed, keepalive=(self, x, routing, weights, handle)) if async_op else None,
         )
+
+    def _check_replay_arguments(self, handle, topk_idx, alignment, do_expand) -> None:
+        if handle.owner is not self:
+            raise ValueError("cached handle belongs to another CudaBuffer")
+        if topk_idx is not None:
+            raise ValueError("cached dispatch uses the handle snapshot; omit topk_idx")
+        if alignment is not None and alignment != handle.alignment:
+            raise ValueError("cached dispatch must retain the handle alignment")
+        if do_expand is not None and do_expand != handle.do_expand:
+            raise ValueError("cached dispatch must retain the handle layout")
+
+    def _new_handle(self, metadata, received, capacity, expand, slot_alignment, dtype, budget) -> NativeHandle:
+        """Wrap what a fresh native dispatch returned: seven tensors in the reference's order
+        (nano_ep/backends/cuda.py:328-345), then the private slot table and slot-order list."""
+        recv_metadata, counts, offsets, dst_slots, send_counts, snapshot, prefix = metadata[:7]
+        private = list(metadata[7:9]) + [None, None]
+        return NativeHandle(
+            config=self._config,
+            rank=self._rank,
+            world_size=self._world_size,
+            do_expand=expand,
+            alignment=slot_alignment,
+            topk_idx=snapshot,
+            layout=NativeLayout(
+                recv_metadata=recv_metadata,
+                expert_counts=counts,
+                expert_offsets=offsets,
+                recv_rank_prefix=prefix,
+                recv_count=received,
+                expanded_capacity=capacity,
+            ),
+            dst_slots=dst_slots,
+            send_counts=send_counts,
+            owner=self,
+            x_dtype=dtype,
+            num_sms=budget,
+            token_slots=private[0],
+            slot_order=private[1],
+        )
+
+    # ------------------------------------------------------------------ combine
 
     def combine(
         self,
@@ -298,61 +255,52 @@ class CudaBuffer:
         async_op: bool = False,
         num_sms: int | None = None,
     ) -> NativeCombineResult:
-        "Return expert outputs to their source and reduce in FP32, without gate weighting."
+        """Bring expert outputs back to their source tokens: per token the fp32 sum of its valid
+        rows in ascending choice order (plus `bias`), rounded to bf16 once.  Gate weights are not
+        applied; when given they are returned at their original (token, choice) positions."""
         check_torch_deterministic()
-        if self._closed:
-            raise RuntimeError("CudaBuffer is closed")
+        self._require_open()
         if handle.owner is not self:
             raise ValueError("combine handle belongs to another CudaBuffer")
         if handle.config != self._config:
             raise ValueError("combine handle configuration does not match this CudaBuffer")
 
-        device = torch.device("cuda", self._device)
-        layout = handle.layout
-        rows = layout.expanded_capacity if handle.do_expand else layout.recv_count
-        hidden = self._config.hidden
-        if x.device != device or x.dtype != torch.bfloat16 or x.shape != (rows, hidden) or not x.is_contiguous():
+        here = torch.device("cuda", self._device)
+        hidden, topk = self._config.hidden, self._config.num_topk
+        expand = handle.do_expand
+        rows = handle.layout.expanded_capacity if expand else handle.layout.recv_count
+
+        def fits(tensor, dtype, shape) -> bool:
+            return tensor.device == here and tensor.dtype == dtype and tuple(tensor.shape) == shape and tensor.is_contiguous()
+
+        if not fits(x, torch.bfloat16, (rows, hidden)):
             raise ValueError("combine x must be contiguous CUDA bfloat16 with the handle's exact receive shape")
-        weight_shape = (rows,) if handle.do_expand else (rows, self._config.num_topk)
-        if weights is not None and (
-            weights.device != device or weights.dtype != torch.float32 or weights.shape != weight_shape or not weights.is_contiguous()
-        ):
+        if weights is not None and not fits(weights, torch.float32, (rows,) if expand else (rows, topk)):
             raise ValueError("combine weights must be contiguous CUDA float32 with the handle's receive layout")
-        source_tokens = handle.topk_idx.shape[0]
-        if bias is not None and (
-            bias.device != device or bias.dtype != x.dtype or bias.shape != (source_tokens, hidden) or not bias.is_contiguous()
-        ):
+        if bias is not None and not fits(bias, x.dtype, (handle.topk_idx.shape[0], hidden)):
             raise ValueError("combine bias must be contiguous source [T,H], with the x dtype on this buffer's device")
 
         metadata = _handle_metadata(handle)
-        main_sms = self._resolve_num_sms(num_sms, handle)
+        budget = self._resolve_num_sms(num_sms, handle)
         with torch.cuda.device(self._device):
-            outputs, completed = self._backend.combine(
-                self._runtime,
-                x,
-                metadata,
-                weights,
-                bias,
-                self._config.num_max_tokens_per_rank,
-                handle.do_expand,
-                self._allow_multiple_reduction,
-                main_sms,
-                self._comm_stream.cuda_stream,
-                -1 if previous_event is None else previous_event.cuda_event,
-                async_op,
+            (combined, restored), completed = self._backend.combine(
+                self._runtime, x, metadata, weights, bias,
+                self._config.num_max_tokens_per_rank, expand, self._allow_multiple_reduction, budget,
+                self._comm_stream.cuda_stream, _raw_event(previous_event), async_op,
             )
-
             event = CudaEvent(completed, keepalive=(self, x, handle, weights, bias)) if async_op else None
+        return NativeCombineResult(x=combined, topk_weights=None if weights is None else restored, event=event)
 
-        return NativeCombineResult(x=outputs[0], topk_weights=outputs[1] if weights is not None else None, event=event)
+    # ------------------------------------------------------------------ lifetime
 
     @property
     def comm_stream(self) -> torch.cuda.Stream:
-        """The stream dispatch and combine kernels are launched on."""
+        """The stream asynchronous dispatch and combine kernels are launched on."""
         return self._comm_stream
 
     def close(self):
-        """Drain the GPU and release the runtime.  Idempotent; dispatch/combine fail afterwards."""
+        """Drain the GPU and release the runtime.  A second call does nothing; dispatch and combine
+        raise afterwards."""
         if self._closed:
             return
         torch.cuda.synchronize(self._device)
