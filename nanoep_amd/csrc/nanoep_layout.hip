@@ -82,6 +82,8 @@ LayoutWorkspace carve_layout_workspace(void* base, int64_t tokens, int topk, int
 // A (token, k) entry of the rank table packs (expert << kRankBits) | in-block rank; -1 marks a
 // masked choice.  A layout block never holds more than 256 tokens, so the rank fits 8 bits.
 constexpr int kRankBits = 8;
+// Most blocks for which every assignment workgroup scans the block histograms itself.
+constexpr int kFusedScanMaxBlocks = 1024;
 static_assert(kMaxBlockTokens <= (1 << kRankBits), "in-block ranks must fit the packed entry");
 constexpr int kRankMask = (1 << kRankBits) - 1;
 
@@ -713,9 +715,12 @@ int nanoep_layout(const int64_t* topk_idx, int64_t num_tokens, int num_topk, int
 
     __atomic_store_n(&host_counts[0], int64_t{-1}, __ATOMIC_RELEASE);
     const int count_threads = tokens_per_block < kWave ? kWave : tokens_per_block;
-    // Two launches when every block can afford to sum the block histograms itself
-    // (blocks x (L+1) loads spread over the workgroup), three with a single-workgroup scan otherwise.
-    bool fused_scan = blocks > 0 && static_cast<int64_t>(blocks) * (experts + 1) <= int64_t{32} * count_threads;
+    // Two launches while every block can afford to sum the block histograms itself (blocks x (L+1)
+    // loads from L2, spread over the workgroup): measured faster than the single-workgroup scan up to
+    // 1024 blocks whatever the expert count (8192 tokens, 256 experts: 21 against 27 us; 262144
+    // tokens: 159 against 198 us).  Beyond, the blocks^2 loads lose (2^20 tokens, 8 experts: 124
+    // against 67 us) and a third launch does the scan once.
+    bool fused_scan = blocks > 0 && blocks <= kFusedScanMaxBlocks;
     const int forced_launches = env_int("NANOEP_LAYOUT_LAUNCHES", 0);
     if (forced_launches == 3)
         fused_scan = false;
