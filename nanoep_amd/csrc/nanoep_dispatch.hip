@@ -260,7 +260,11 @@ __global__ void __launch_bounds__(1024) dispatch_ordered_kernel(const u32x4* __r
 
 // Compact layout: receive row r holds source token src_token(r), in token order, so the dispatch is
 // a row copy with holes.  Nothing is re-used, so workgroups walk the rows in plain launch order
-// (one linear stream over the whole device) and the kernel carries nothing but the copy.
+// (one linear stream over the whole device) and the payload wavefronts carry nothing but the copy.
+// The rows' ids and weights are moved by `side_blocks` workgroups of their own at the front of the
+// grid, one lane per (token, k): hung onto the first payload wavefront of every row they cost 11 us
+// of a 95 us kernel at 32768 x 4096, top-8 (two more dependent round trips in one wavefront in
+// eight); on their own, with full wavefronts and coalesced rows, next to nothing.
 __global__ void __launch_bounds__(1024) dispatch_compact_kernel(const u32x4* __restrict__ x,                // [T][vectors]
                                                                 const float* __restrict__ weights,         // [T][K] or null
                                                                 const int32_t* __restrict__ recv_metadata,  // [N][K+2]
@@ -277,12 +281,32 @@ __global__ void __launch_bounds__(1024) dispatch_compact_kernel(const u32x4* __r
                                                                 uint32_t rows_per_block,    // == blockDim.z
                                                                 uint32_t vectors,
                                                                 uint32_t chunks,
-                                                                uint32_t topk) {
+                                                                uint32_t topk,
+                                                                uint32_t topk_magic,  // fast divisor by K
+                                                                uint32_t topk_shift,
+                                                                uint32_t side_blocks) {
     NANOEP_FETCH_ARGS_4(x, dst_slots, recv_x, tokens);
     NANOEP_FETCH_ARGS_4(recv_count, parts, parts_magic, parts_shift);
     NANOEP_FETCH_ARGS_4(chunks_per_block, rows_per_block, vectors, chunks);
-    const uint32_t group = fast_divide(blockIdx.x, parts_magic, parts_shift);
-    const uint32_t part = blockIdx.x - group * parts;
+    if (blockIdx.x < side_blocks) {
+        const uint32_t wave = threadIdx.z * chunks_per_block + threadIdx.y;
+        const uint32_t flat = (blockIdx.x * (chunks_per_block * rows_per_block) + wave) * kWave + threadIdx.x;
+        const uint32_t token = fast_divide(flat, topk_magic, topk_shift);
+        if (token >= tokens)
+            return;
+        const uint32_t k = flat - token * topk;
+        const int64_t row = dst_slots[token];
+        if (row < 0 || row >= static_cast<int64_t>(recv_count))
+            return;
+        if (recv_topk_idx != nullptr)
+            recv_topk_idx[row * topk + k] = recv_metadata[row * (topk + 2) + 2 + k];
+        if (recv_weights != nullptr)
+            recv_weights[row * topk + k] = weights[flat];
+        return;
+    }
+    const uint32_t payload_block = blockIdx.x - side_blocks;
+    const uint32_t group = fast_divide(payload_block, parts_magic, parts_shift);
+    const uint32_t part = payload_block - group * parts;
     const uint32_t token = group * rows_per_block + __builtin_amdgcn_readfirstlane(threadIdx.z);
     const uint32_t chunk = part * chunks_per_block + __builtin_amdgcn_readfirstlane(threadIdx.y);
     if (token >= tokens || chunk >= chunks)
@@ -296,13 +320,6 @@ __global__ void __launch_bounds__(1024) dispatch_compact_kernel(const u32x4* __r
         return;
     if (in_row)
         store_vec<true>(recv_x + static_cast<uint64_t>(row) * vectors + vector, data);
-    if (chunk == 0 && threadIdx.x < topk) {
-        const uint32_t lane = threadIdx.x;
-        if (recv_topk_idx != nullptr)
-            recv_topk_idx[row * topk + lane] = recv_metadata[row * (topk + 2) + 2 + lane];
-        if (recv_weights != nullptr)
-            recv_weights[row * topk + lane] = weights[static_cast<uint64_t>(token) * topk + lane];
-    }
 }
 
 
@@ -420,11 +437,18 @@ int nanoep_dispatch(const void* x, const float* weights, const int32_t* recv_met
 #undef NANOEP_LAUNCH_ORDERED_SPAN
     } else if (!expand) {
         const int64_t blocks = (num_tokens + blocking.rows_per_block - 1) / blocking.rows_per_block * blocking.parts;
-        dispatch_compact_kernel<<<dim3(static_cast<unsigned>(blocks)), block, 0, stream>>>(
+        // one lane per (token, k) for the ids and weights, when the caller wants either
+        const int64_t side_lanes = recv_topk_idx != nullptr || recv_weights != nullptr ? num_tokens * num_topk : 0;
+        const int64_t side_blocks = (side_lanes + kWave * waves - 1) / (kWave * waves);
+        if (side_lanes >= (int64_t{1} << 31) || blocks + side_blocks >= (int64_t{1} << 31))
+            return NANOEP_ERR_INVALID_ARGUMENT;
+        const FastDivisor topk_divisor = make_fast_divisor(static_cast<uint32_t>(num_topk));
+        dispatch_compact_kernel<<<dim3(static_cast<unsigned>(blocks + side_blocks)), block, 0, stream>>>(
             static_cast<const u32x4*>(x), weights, recv_metadata, dst_slots, static_cast<u32x4*>(recv_x), recv_topk_idx,
             recv_weights, static_cast<uint32_t>(num_tokens), static_cast<uint32_t>(recv_count), blocking.parts,
             parts_divisor.magic, parts_divisor.shift, blocking.chunks_per_block, blocking.rows_per_block,
-            static_cast<uint32_t>(vectors), static_cast<uint32_t>(chunks), static_cast<uint32_t>(num_topk));
+            static_cast<uint32_t>(vectors), static_cast<uint32_t>(chunks), static_cast<uint32_t>(num_topk),
+            topk_divisor.magic, topk_divisor.shift, static_cast<uint32_t>(side_blocks));
     } else {
 #define NANOEP_LAUNCH_ROWS(LOOKUP, ZERO_FILL)                                                                         \
     dispatch_rows_kernel<LOOKUP, ZERO_FILL><<<grid, block, 0, stream>>>(                                             \
