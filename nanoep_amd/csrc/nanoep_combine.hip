@@ -164,13 +164,28 @@ __global__ void __launch_bounds__(1024) combine_few_rows_kernel(const u32x4* __r
                                                                 uint32_t vectors,
                                                                 uint32_t chunks,
                                                                 uint32_t topk,
-                                                                int multiple_reduction) {
+                                                                int multiple_reduction,
+                                                                uint32_t topk_magic,  // fast divisor by K
+                                                                uint32_t topk_shift,
+                                                                uint32_t side_blocks) {
     NANOEP_FETCH_ARGS_4(y, token_slots, out_x, bias);
     NANOEP_FETCH_ARGS_4(tokens, y_rows, parts, parts_magic);
     NANOEP_FETCH_ARGS_4(parts_shift, chunks_per_block, rows_per_block, vectors);
     NANOEP_FETCH_ARGS_4(chunks, topk, multiple_reduction, out_weights);
-    const uint32_t group = fast_divide(blockIdx.x, parts_magic, parts_shift);
-    const uint32_t part = blockIdx.x - group * parts;
+    if (blockIdx.x < side_blocks) {
+        // weights back to their (token, k): one lane each, in workgroups of their own at the front
+        // of the grid (on the first payload wavefront of a row they are a second round trip)
+        const uint32_t wave = threadIdx.z * chunks_per_block + threadIdx.y;
+        const uint32_t flat = (blockIdx.x * (chunks_per_block * rows_per_block) + wave) * kWave + threadIdx.x;
+        if (fast_divide(flat, topk_magic, topk_shift) >= tokens)
+            return;
+        const int32_t slot = token_slots[flat];
+        out_weights[flat] = slot >= 0 && static_cast<uint32_t>(slot) < y_rows ? weights[slot] : 0.0f;
+        return;
+    }
+    const uint32_t payload_block = blockIdx.x - side_blocks;
+    const uint32_t group = fast_divide(payload_block, parts_magic, parts_shift);
+    const uint32_t part = payload_block - group * parts;
     const uint32_t token = group * rows_per_block + __builtin_amdgcn_readfirstlane(threadIdx.z);
     const uint32_t chunk = part * chunks_per_block + __builtin_amdgcn_readfirstlane(threadIdx.y);
     if (token >= tokens || chunk >= chunks)
@@ -217,11 +232,6 @@ __global__ void __launch_bounds__(1024) combine_few_rows_kernel(const u32x4* __r
         packed.w = bf16_round(acc[6]) | (bf16_round(acc[7]) << 16);
         store_vec<true>(out_x + static_cast<uint64_t>(token) * vectors + vector, packed);
     }
-    if (chunk == 0 && out_weights != nullptr && threadIdx.x < topk) {
-        const int32_t mine = slots[threadIdx.x];
-        const bool mine_valid = mine >= 0 && static_cast<uint32_t>(mine) < y_rows;
-        out_weights[static_cast<uint64_t>(token) * topk + threadIdx.x] = mine_valid ? weights[mine] : 0.0f;
-    }
 }
 
 // Compact layout: a token has one received row, so the combine is a row copy through fp32
@@ -243,12 +253,33 @@ __global__ void __launch_bounds__(1024) combine_compact_kernel(const u32x4* __re
                                                                uint32_t rows_per_block,    // == blockDim.z
                                                                uint32_t vectors,
                                                                uint32_t chunks,
-                                                               uint32_t topk) {
+                                                               uint32_t topk,
+                                                               uint32_t topk_magic,  // fast divisor by K
+                                                               uint32_t topk_shift,
+                                                               uint32_t side_blocks) {
     NANOEP_FETCH_ARGS_4(y, dst_slots, out_x, bias);
     NANOEP_FETCH_ARGS_4(tokens, recv_count, parts, parts_magic);
     NANOEP_FETCH_ARGS_4(parts_shift, chunks_per_block, rows_per_block, vectors);
-    const uint32_t group = fast_divide(blockIdx.x, parts_magic, parts_shift);
-    const uint32_t part = blockIdx.x - group * parts;
+    if (blockIdx.x < side_blocks) {
+        // weights back to their (token, k), zero for masked choices and tokens that were not sent: one
+        // lane each, in workgroups of their own at the front of the grid.  On the first payload wavefront
+        // of every row the two dependent lookups cost 22 us of 104 at 32768 x 4096, top-8.
+        const uint32_t wave = threadIdx.z * chunks_per_block + threadIdx.y;
+        const uint32_t flat = (blockIdx.x * (chunks_per_block * rows_per_block) + wave) * kWave + threadIdx.x;
+        const uint32_t token = fast_divide(flat, topk_magic, topk_shift);
+        if (token >= tokens)
+            return;
+        const uint32_t k = flat - token * topk;
+        const int64_t row = dst_slots[token];
+        float weight = 0.0f;
+        if (row >= 0 && row < static_cast<int64_t>(recv_count) && recv_metadata[row * (topk + 2) + 2 + k] >= 0)
+            weight = weights[row * topk + k];
+        out_weights[flat] = weight;
+        return;
+    }
+    const uint32_t payload_block = blockIdx.x - side_blocks;
+    const uint32_t group = fast_divide(payload_block, parts_magic, parts_shift);
+    const uint32_t part = payload_block - group * parts;
     const uint32_t token = group * rows_per_block + __builtin_amdgcn_readfirstlane(threadIdx.z);
     const uint32_t chunk = part * chunks_per_block + __builtin_amdgcn_readfirstlane(threadIdx.y);
     if (token >= tokens || chunk >= chunks)
@@ -272,13 +303,6 @@ __global__ void __launch_bounds__(1024) combine_compact_kernel(const u32x4* __re
         packed.z = bf16_round(acc[4]) | (bf16_round(acc[5]) << 16);
         packed.w = bf16_round(acc[6]) | (bf16_round(acc[7]) << 16);
         store_vec<true>(out_x + static_cast<uint64_t>(token) * vectors + vector, packed);
-    }
-    if (chunk == 0 && out_weights != nullptr && threadIdx.x < topk) {
-        const uint32_t lane = threadIdx.x;
-        float weight = 0.0f;
-        if (received && recv_metadata[row * (topk + 2) + 2 + lane] >= 0)
-            weight = weights[row * topk + lane];
-        out_weights[static_cast<uint64_t>(token) * topk + lane] = weight;
     }
 }
 
@@ -322,6 +346,14 @@ int nanoep_combine(const void* y, const float* weights, const void* bias, const 
         return NANOEP_ERR_INVALID_ARGUMENT;
     const dim3 grid(static_cast<unsigned>(blocks));
     const dim3 block(kWave, blocking.chunks_per_block, blocking.rows_per_block);
+    // workgroups of their own, one lane per (token, k), for the kernels that restore weights that way
+    const int64_t waves = static_cast<int64_t>(blocking.chunks_per_block) * blocking.rows_per_block;
+    const int64_t side_lanes = out_weights != nullptr ? num_tokens * num_topk : 0;
+    const int64_t side_blocks = (side_lanes + kWave * waves - 1) / (kWave * waves);
+    if (side_lanes >= (int64_t{1} << 31) || blocks + side_blocks >= (int64_t{1} << 31))
+        return NANOEP_ERR_INVALID_ARGUMENT;
+    const dim3 grid_with_side(static_cast<unsigned>(blocks + side_blocks));
+    const FastDivisor topk_divisor = make_fast_divisor(static_cast<uint32_t>(num_topk));
     auto stream = static_cast<hipStream_t>(stream_handle);
     const int gathered = expand ? num_topk : 1;
     // the slot table only helps the expanded layout, and only when something was received
@@ -329,23 +361,23 @@ int nanoep_combine(const void* y, const float* weights, const void* bias, const 
     const FastDivisor parts_divisor = make_fast_divisor(blocking.parts);
     if (!expand) {
         // y may be a null pointer when nothing was received: every token then takes the hole path
-        combine_compact_kernel<<<grid, block, 0, stream>>>(
+        combine_compact_kernel<<<grid_with_side, block, 0, stream>>>(
             static_cast<const u32x4*>(recv_count > 0 ? y : out_x), weights, static_cast<const u32x4*>(bias), recv_metadata,
             dst_slots, static_cast<u32x4*>(out_x), out_weights, static_cast<uint32_t>(num_tokens),
             static_cast<uint32_t>(recv_count), blocking.parts, parts_divisor.magic, parts_divisor.shift,
             blocking.chunks_per_block, blocking.rows_per_block, static_cast<uint32_t>(vectors), static_cast<uint32_t>(chunks),
-            static_cast<uint32_t>(num_topk));
+            static_cast<uint32_t>(num_topk), topk_divisor.magic, topk_divisor.shift, static_cast<uint32_t>(side_blocks));
         NANOEP_HIP_TRY(hipGetLastError());
         return NANOEP_OK;
     }
     if (direct && num_topk <= 4) {
 #define NANOEP_LAUNCH_FEW(TOPK)                                                                                       \
-    combine_few_rows_kernel<TOPK><<<grid, block, 0, stream>>>(                                                       \
+    combine_few_rows_kernel<TOPK><<<grid_with_side, block, 0, stream>>>(                                             \
         static_cast<const u32x4*>(y), weights, static_cast<const u32x4*>(bias), token_slots,                         \
         static_cast<u32x4*>(out_x), out_weights, static_cast<uint32_t>(num_tokens), static_cast<uint32_t>(y_rows),   \
         blocking.parts, parts_divisor.magic, parts_divisor.shift, blocking.chunks_per_block, blocking.rows_per_block, \
         static_cast<uint32_t>(vectors), static_cast<uint32_t>(chunks), static_cast<uint32_t>(num_topk),              \
-        multiple_reduction ? 1 : 0)
+        multiple_reduction ? 1 : 0, topk_divisor.magic, topk_divisor.shift, static_cast<uint32_t>(side_blocks))
         if (num_topk == 1)
             NANOEP_LAUNCH_FEW(1);
         else if (num_topk == 2)
