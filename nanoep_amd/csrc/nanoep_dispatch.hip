@@ -198,7 +198,8 @@ __global__ void __launch_bounds__(1024) dispatch_ordered_kernel(const u32x4* __r
                                                                 uint32_t vectors,
                                                                 uint32_t chunks,      // pieces of kSpan chunks in a row
                                                                 uint32_t topk_magic,  // fast divisor by K
-                                                                uint32_t topk_shift) {
+                                                                uint32_t topk_shift,
+                                                                uint32_t payload_blocks) {  // blocks behind them, if any, move the weights
     NANOEP_FETCH_ARGS_4(x, weights, recv_x, recv_weights);
     NANOEP_FETCH_ARGS_4(slot_order, entries, source_limit, out_rows);
     NANOEP_FETCH_ARGS_4(copy_blocks, copy_per_xcd, parts, parts_magic);
@@ -215,6 +216,24 @@ __global__ void __launch_bounds__(1024) dispatch_ordered_kernel(const u32x4* __r
             copy_blocks = (rows_per_block == 1 ? entries : (entries + rows_per_block - 1) / rows_per_block) * parts;
             copy_per_xcd = (copy_blocks + kNumXcds - 1) / kNumXcds;
         }
+    }
+    if (blockIdx.x >= payload_blocks) {
+        // The weights of the assignments, one lane per list entry, in workgroups of their own at the
+        // end of the grid.  The host asks for them when rows are short: hung onto the first payload
+        // wavefront of every row the weight is a second round trip in one wavefront of (at most) four
+        // (8192 x 2048, top-8: 61 -> 58 us).  With longer rows the first wavefronts are few and carry it
+        // at no measurable cost, while these extra workgroups cost 0.1 ns per assignment (4096 x 7168:
+        // +1 us, 32768 x 7168: +25 us of 700).
+        const uint32_t wave = threadIdx.z * chunks_per_block + threadIdx.y;
+        const uint32_t flat = ((blockIdx.x - payload_blocks) * (chunks_per_block * rows_per_block) + wave) * kWave + threadIdx.x;
+        if (flat >= entries)
+            return;
+        const int64_t entry = slot_order[flat];
+        const uint32_t source = static_cast<uint32_t>(entry);
+        const uint32_t out_row = static_cast<uint32_t>(static_cast<uint64_t>(entry) >> 32);
+        if (entry >= 0 && source < source_limit && out_row < out_rows)
+            recv_weights[out_row] = weights[source];
+        return;
     }
     const uint32_t index_in_xcd = blockIdx.x / kNumXcds;
     if (kZeroFill && index_in_xcd >= copy_per_xcd) {
@@ -254,7 +273,8 @@ __global__ void __launch_bounds__(1024) dispatch_ordered_kernel(const u32x4* __r
         if (at < vectors)
             store_vec<true>(recv_x + static_cast<uint64_t>(out_row) * vectors + at, data[s]);
     }
-    if (chunk == 0 && threadIdx.x == 0 && recv_weights != nullptr)
+    // no workgroups behind the payload: the row's first wavefront moves its weight
+    if (chunk == 0 && threadIdx.x == 0 && recv_weights != nullptr && payload_blocks == gridDim.x)
         recv_weights[out_row] = weights[source];
 }
 
@@ -402,7 +422,15 @@ int nanoep_dispatch(const void* x, const float* weights, const int32_t* recv_met
         for (topk_shift = 0; (1 << topk_shift) < num_topk; ++topk_shift) {
         }
 
-    const dim3 grid((copy_per_xcd + pad_per_xcd) * kNumXcds);
+    // slot-order walk over short rows (up to four chunks): one lane per list entry moves the weights,
+    // in workgroups at the end of the grid; longer rows carry the weight on their first wavefront
+    const bool side_weights = ordered && recv_weights != nullptr && chunks * span <= 4;
+    const int64_t side_lanes = side_weights ? copy_candidates : 0;
+    const int64_t side_blocks = (side_lanes + kWave * waves - 1) / (kWave * waves);
+    const int64_t payload_blocks = (int64_t{copy_per_xcd} + pad_per_xcd) * kNumXcds;
+    if (payload_blocks + side_blocks >= (int64_t{1} << 31))
+        return NANOEP_ERR_INVALID_ARGUMENT;
+    const dim3 grid(static_cast<unsigned>(payload_blocks + side_blocks));
     const dim3 block(kWave, blocking.chunks_per_block, blocking.rows_per_block);
     const FastDivisor parts_divisor = make_fast_divisor(blocking.parts);
     auto stream = static_cast<hipStream_t>(stream_handle);
@@ -417,7 +445,8 @@ int nanoep_dispatch(const void* x, const float* weights, const int32_t* recv_met
         static_cast<uint32_t>(pad_per_expert),                                                                       \
         static_cast<uint32_t>(pad_groups_per_expert > 0 ? pad_groups_per_expert : 1), blocking.parts,                \
         parts_divisor.magic, parts_divisor.shift, blocking.chunks_per_block, blocking.rows_per_block,                \
-        static_cast<uint32_t>(vectors), static_cast<uint32_t>(chunks), topk_divisor.magic, topk_divisor.shift)
+        static_cast<uint32_t>(vectors), static_cast<uint32_t>(chunks), topk_divisor.magic, topk_divisor.shift,       \
+        static_cast<uint32_t>(payload_blocks))
 #define NANOEP_LAUNCH_ORDERED(DEVICE_COUNT, ZERO_FILL)             \
     do {                                                           \
         if (span == 2)                                             \
@@ -438,17 +467,17 @@ int nanoep_dispatch(const void* x, const float* weights, const int32_t* recv_met
     } else if (!expand) {
         const int64_t blocks = (num_tokens + blocking.rows_per_block - 1) / blocking.rows_per_block * blocking.parts;
         // one lane per (token, k) for the ids and weights, when the caller wants either
-        const int64_t side_lanes = recv_topk_idx != nullptr || recv_weights != nullptr ? num_tokens * num_topk : 0;
-        const int64_t side_blocks = (side_lanes + kWave * waves - 1) / (kWave * waves);
-        if (side_lanes >= (int64_t{1} << 31) || blocks + side_blocks >= (int64_t{1} << 31))
+        const int64_t row_side_lanes = recv_topk_idx != nullptr || recv_weights != nullptr ? num_tokens * num_topk : 0;
+        const int64_t row_side_blocks = (row_side_lanes + kWave * waves - 1) / (kWave * waves);
+        if (row_side_lanes >= (int64_t{1} << 31) || blocks + row_side_blocks >= (int64_t{1} << 31))
             return NANOEP_ERR_INVALID_ARGUMENT;
         const FastDivisor topk_divisor = make_fast_divisor(static_cast<uint32_t>(num_topk));
-        dispatch_compact_kernel<<<dim3(static_cast<unsigned>(blocks + side_blocks)), block, 0, stream>>>(
+        dispatch_compact_kernel<<<dim3(static_cast<unsigned>(blocks + row_side_blocks)), block, 0, stream>>>(
             static_cast<const u32x4*>(x), weights, recv_metadata, dst_slots, static_cast<u32x4*>(recv_x), recv_topk_idx,
             recv_weights, static_cast<uint32_t>(num_tokens), static_cast<uint32_t>(recv_count), blocking.parts,
             parts_divisor.magic, parts_divisor.shift, blocking.chunks_per_block, blocking.rows_per_block,
             static_cast<uint32_t>(vectors), static_cast<uint32_t>(chunks), static_cast<uint32_t>(num_topk),
-            topk_divisor.magic, topk_divisor.shift, static_cast<uint32_t>(side_blocks));
+            topk_divisor.magic, topk_divisor.shift, static_cast<uint32_t>(row_side_blocks));
     } else {
 #define NANOEP_LAUNCH_ROWS(LOOKUP, ZERO_FILL)                                                                         \
     dispatch_rows_kernel<LOOKUP, ZERO_FILL><<<grid, block, 0, stream>>>(                                             \
