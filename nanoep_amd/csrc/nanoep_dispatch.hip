@@ -395,11 +395,14 @@ int nanoep_dispatch(const void* x, const float* weights, const int32_t* recv_met
 
     const int vectors = hidden / 8;
     int chunks = (vectors + kWave - 1) / kWave;
-    // Chunks per wavefront of the slot-order walk: two once the source outgrows the last-level cache
-    // (NANOEP_DISPATCH_SPAN=1|2 overrides).  `chunks` then counts pieces of that many chunks.
+    // Chunks per wavefront of the slot-order walk: two once the source outgrows the last-level cache,
+    // and for rows of two to four chunks, where halving the wavefronts a row takes outweighs the second
+    // store (16384 x 1024 top-4: 38 -> 33 us; 8192 x 2048 top-8: 55 -> 52 us).  NANOEP_DISPATCH_SPAN=1|2
+    // overrides.  `chunks` then counts pieces of that many chunks.
     int span = 1;
     if (ordered) {
-        span = static_cast<int64_t>(num_tokens) * hidden * 2 > kLastLevelCacheBytes ? 2 : 1;
+        const bool short_rows = chunks >= 2 && chunks <= 4;
+        span = short_rows || static_cast<int64_t>(num_tokens) * hidden * 2 > kLastLevelCacheBytes ? 2 : 1;
         const int forced_span = env_int("NANOEP_DISPATCH_SPAN", 0);
         if (forced_span == 1 || forced_span == 2)
             span = forced_span;
