@@ -219,11 +219,11 @@ __global__ void __launch_bounds__(1024) dispatch_ordered_kernel(const u32x4* __r
     }
     if (blockIdx.x >= payload_blocks) {
         // The weights of the assignments, one lane per list entry, in workgroups of their own at the
-        // end of the grid.  The host asks for them when rows are short: hung onto the first payload
-        // wavefront of every row the weight is a second round trip in one wavefront of (at most) four
-        // (8192 x 2048, top-8: 61 -> 58 us).  With longer rows the first wavefronts are few and carry it
-        // at no measurable cost, while these extra workgroups cost 0.1 ns per assignment (4096 x 7168:
-        // +1 us, 32768 x 7168: +25 us of 700).
+        // end of the grid.  The host asks for them when a row is one or two chunks: hung onto the
+        // row's first payload wavefront the weight is a second round trip in every (second) wavefront
+        // (131072 x 512 top-8: 77.5 -> 74.5 us).  With longer rows the first wavefronts are few and
+        // carry it at no measurable cost, while these extra workgroups cost 0.1 ns per assignment
+        // (4096 x 7168: +1 us, 32768 x 7168: +25 us of 700).
         const uint32_t wave = threadIdx.z * chunks_per_block + threadIdx.y;
         const uint32_t flat = ((blockIdx.x - payload_blocks) * (chunks_per_block * rows_per_block) + wave) * kWave + threadIdx.x;
         if (flat >= entries)
@@ -396,12 +396,13 @@ int nanoep_dispatch(const void* x, const float* weights, const int32_t* recv_met
     const int vectors = hidden / 8;
     int chunks = (vectors + kWave - 1) / kWave;
     // Chunks per wavefront of the slot-order walk: two once the source outgrows the last-level cache,
-    // and for rows of two to four chunks, where halving the wavefronts a row takes outweighs the second
-    // store (16384 x 1024 top-4: 38 -> 33 us; 8192 x 2048 top-8: 55 -> 52 us).  NANOEP_DISPATCH_SPAN=1|2
-    // overrides.  `chunks` then counts pieces of that many chunks.
+    // and for rows of two chunks, which then take one wavefront (16384 x 1024 top-4: 39.8 -> 35.6 us;
+    // at four chunks the gain is within +3 / -1 %).  NANOEP_DISPATCH_SPAN=1|2 overrides.  `chunks`
+    // then counts pieces of that many chunks.
+    const int row_chunks = chunks;
     int span = 1;
     if (ordered) {
-        const bool short_rows = chunks >= 2 && chunks <= 4;
+        const bool short_rows = chunks == 2;
         span = short_rows || static_cast<int64_t>(num_tokens) * hidden * 2 > kLastLevelCacheBytes ? 2 : 1;
         const int forced_span = env_int("NANOEP_DISPATCH_SPAN", 0);
         if (forced_span == 1 || forced_span == 2)
@@ -425,9 +426,11 @@ int nanoep_dispatch(const void* x, const float* weights, const int32_t* recv_met
         for (topk_shift = 0; (1 << topk_shift) < num_topk; ++topk_shift) {
         }
 
-    // slot-order walk over short rows (up to four chunks): one lane per list entry moves the weights,
-    // in workgroups at the end of the grid; longer rows carry the weight on their first wavefront
-    const bool side_weights = ordered && recv_weights != nullptr && chunks * span <= 4;
+    // slot-order walk over rows of one or two chunks: one lane per list entry moves the weights, in
+    // workgroups at the end of the grid (+3-4 %); longer rows carry the weight on their first wavefront
+    // (8192 x 2048 top-8 with alignment 128: 56.0 against 57.0 us).  NANOEP_DISPATCH_SIDE=0|1 overrides.
+    const int side_switch = env_int("NANOEP_DISPATCH_SIDE", -1);
+    const bool side_weights = ordered && recv_weights != nullptr && (side_switch < 0 ? row_chunks <= 2 : side_switch != 0);
     const int64_t side_lanes = side_weights ? copy_candidates : 0;
     const int64_t side_blocks = (side_lanes + kWave * waves - 1) / (kWave * waves);
     const int64_t payload_blocks = (int64_t{copy_per_xcd} + pad_per_xcd) * kNumXcds;
