@@ -60,11 +60,12 @@ int nanoep_window_layout(int ranks, int64_t max_tokens, int hidden, int topk, in
 /* Device scratch needed by nanoep_layout for (T, K, L). */
 size_t nanoep_layout_workspace_bytes(int64_t num_tokens, int num_topk, int64_t num_local_experts);
 
-/* Tokens per block of the routing layout for T tokens, L local experts and payload rows of
- * `hidden` bf16 elements (0: not known; the answer is 0 when L is not supported).  The slot-order
- * list is ordered block of consecutive tokens by block, and a block's rows should fit one XCD's 4 MiB
- * L2: 256 tokens up to hidden 8192 (and when hidden is not known), then 128 and 64; fewer for very
- * many experts, and for batches of 257..2047 tokens so that there are eight blocks. */
+/* Tokens of one block ("window") of the slot-order list for T tokens, L local experts and payload
+ * rows of `hidden` bf16 elements (0: not known; the answer is 0 when L is not supported).  The list
+ * is ordered window of consecutive tokens by window, and a window's rows should fit one XCD's 4 MiB
+ * L2: 512 tokens up to hidden 4096, 256 up to 8192 (and when hidden is not known), then 128 and 64;
+ * fewer for batches of 257..4095 tokens so that there are eight windows, and the layout workgroup's
+ * own token count when the layout needs its separate scan launch (more than 1024 workgroups). */
 int nanoep_layout_block_tokens(int64_t num_tokens, int64_t num_local_experts, int hidden);
 
 /* Number of int64 words of the slot-order buffer for (T, K, L): T rounded up to 256, times K
@@ -84,9 +85,8 @@ int64_t nanoep_slot_order_entries(int64_t num_tokens, int num_topk, int64_t num_
  * reference's handle tensors; nanoep_dispatch / nanoep_combine run a little faster when given it.
  * slot_order (optional, expanded only, T*K < 2^31, int64 [nanoep_slot_order_entries]) lists the A
  * valid assignments as (slot << 32) | (t * K + k), token block by token block and in ascending slot
- * (that is expert-major) order inside a block; the entries from A up to the end of the last block
- * (blocks * nanoep_layout_block_tokens * K) are -1, anything behind them is left unwritten, and the
- * last word of the buffer holds A.  Walking it makes a dispatch write runs of consecutive destination
+ * (that is expert-major) order inside a block; the entries from A on are -1 and the last word of
+ * the buffer holds A.  Walking it makes a dispatch write runs of consecutive destination
  * rows while a block's source rows stay cache resident.  Like token_slots it is private to this library.
  * hidden is the row width (bf16 elements) of the payload that will be dispatched with this handle,
  * 0 when not known: it only sizes the token blocks (nanoep_layout_block_tokens).

@@ -208,8 +208,7 @@ __global__ void __launch_bounds__(1024) dispatch_ordered_kernel(const u32x4* __r
     if (kDeviceCount) {
         // The list length was not known when the grid was sized: shrink the walk to the entries in
         // use, so that the per-XCD ranges split the real work and not its unused tail.
-        // A word that cannot be a count (the layout did not run) walks nothing: the buffer's tail
-        // behind the layout's blocks is never written.
+        // A word that cannot be a count (the layout did not run) walks nothing.
         const int64_t live = uniform_load(live_count);
         if (live != static_cast<int64_t>(entries)) {
             entries = live >= 0 && live < static_cast<int64_t>(entries) ? static_cast<uint32_t>(live) : 0u;

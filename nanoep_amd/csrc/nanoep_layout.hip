@@ -13,34 +13,62 @@ constexpr int kMaxBlockTokens = 256;
 // list block by block and wants every re-use of a source row to hit that cache.
 constexpr int64_t kXcdL2Bytes = int64_t{4} << 20;
 
-// Tokens handled by one layout workgroup = tokens of one block of the slot-order list.
-//  * `hidden` (bf16 elements of a payload row, 0 = not known) sizes the block so that its rows fit an
-//    XCD's L2: 256 tokens up to 8192 elements (and when it is not known), then 128 and 64.  (Blocks
-//    of 512 tokens for rows of up to 4096 elements make the dispatch 1-4 % faster and the layout
-//    itself 5 us slower: half as many workgroups, each with a longer chain.)
-//  * The LDS bit matrix has (L+1) rows of tokens/32 words plus a 16-bit prefix per word, so the block
-//    shrinks as the expert count grows.
-//  * The dispatch hands every XCD whole token blocks when there are at least eight of them: batches
-//    of more than 256 tokens take smaller blocks (down to 64 tokens) to get there.  A batch of up to
-//    256 tokens is one block: its whole layout is then a single launch.
-int layout_tokens_per_block(int64_t tokens_total, int64_t local_experts, int hidden) {
-    if (static_cast<size_t>(local_experts + 1) * 12 > kLayoutLdsBudget)  // three int32 arrays of the assignment kernel
-        return 0;
-    int largest = 256;
+// Most blocks for which every assignment workgroup scans the block histograms itself.
+constexpr int kFusedScanMaxBlocks = 1024;
+// Largest window: the run of consecutive tokens the slot-order list is ordered by.
+constexpr int kMaxWindowTokens = 512;
+
+// Tokens of one window of the slot-order list.
+//  * `hidden` (bf16 elements of a payload row, 0 = not known) sizes the window so that its rows fit an
+//    XCD's L2: 512 tokens up to 4096 elements, 256 up to 8192 (and when it is not known), then 128, 64.
+//  * The dispatch hands every XCD whole windows when there are at least eight of them: batches of
+//    more than 256 tokens take smaller windows (down to 64 tokens) to get there.
+int layout_window_tokens(int64_t tokens_total, int hidden) {
+    int window = 256;
     if (hidden > 0)
-        for (largest = kMaxBlockTokens; largest > 64 && static_cast<int64_t>(largest) * hidden * 2 > kXcdL2Bytes; largest /= 2) {
+        for (window = kMaxWindowTokens; window > 64 && static_cast<int64_t>(window) * hidden * 2 > kXcdL2Bytes; window /= 2) {
         }
-    int chosen = 0;
-    for (int tokens = largest; tokens >= 32; tokens /= 2) {
+    if (tokens_total <= 256 && window > 256)
+        window = 256;  // one layout block: the whole layout is then a single launch
+    while (tokens_total > 256 && window > 64 && (tokens_total + window - 1) / window < 8)
+        window /= 2;
+    return window;
+}
+
+// Tokens handled by one layout workgroup (one thread per token): the window, at most 256, fewer when
+// the LDS bit matrix ((L+1) rows of tokens/32 words plus a 16-bit prefix per word) asks for it.  A
+// window of 512 tokens is two workgroups' worth: the assignment pass orders the list by windows from
+// the block histograms (a 512-token workgroup makes the dispatch as fast and the layout 5 us slower).
+int layout_tokens_per_block(int64_t tokens_total, int64_t local_experts, int hidden) {
+    if (static_cast<size_t>(local_experts + 1) * 16 > kLayoutLdsBudget)  // four int32 arrays of the assignment kernel
+        return 0;
+    const int window = layout_window_tokens(tokens_total, hidden);
+    for (int tokens = window < kMaxBlockTokens ? window : kMaxBlockTokens; tokens >= 32; tokens /= 2) {
         const size_t words = static_cast<size_t>(tokens / 32);
-        if (static_cast<size_t>(local_experts + 1) * (words * 6 + 4) <= kLayoutLdsBudget) {
-            chosen = tokens;
-            break;
-        }
+        if (static_cast<size_t>(local_experts + 1) * (words * 6 + 4) <= kLayoutLdsBudget)
+            return tokens;
     }
-    while (tokens_total > 256 && chosen > 64 && (tokens_total + chosen - 1) / chosen < 8)
-        chosen /= 2;
-    return chosen;
+    return 0;
+}
+
+// Layout blocks per window.  Windows of several blocks need every assignment workgroup to see the
+// block histograms (the two-launch plan); with a separate scan launch the window is the block.
+int layout_window_blocks(int64_t tokens_total, int64_t local_experts, int hidden, bool fused_scan) {
+    const int per_block = layout_tokens_per_block(tokens_total, local_experts, hidden);
+    const int window = layout_window_tokens(tokens_total, hidden);
+    return per_block == 0 || !fused_scan || window <= per_block ? 1 : window / per_block;
+}
+
+// Whether the layout of this batch runs as two launches (see nanoep_layout).
+bool layout_uses_fused_scan(int64_t tokens_total, int64_t local_experts, int hidden) {
+    const int per_block = layout_tokens_per_block(tokens_total, local_experts, hidden);
+    if (per_block == 0 || tokens_total == 0)
+        return false;
+    const int64_t blocks = (tokens_total + per_block - 1) / per_block;
+    const int forced = env_int("NANOEP_LAYOUT_LAUNCHES", 0);
+    if (forced == 3)
+        return false;
+    return forced == 2 || blocks <= kFusedScanMaxBlocks;
 }
 
 // Smallest block any `hidden` can lead to for this batch: what the workspace is sized for.
@@ -82,8 +110,6 @@ LayoutWorkspace carve_layout_workspace(void* base, int64_t tokens, int topk, int
 // A (token, k) entry of the rank table packs (expert << kRankBits) | in-block rank; -1 marks a
 // masked choice.  A layout block never holds more than 256 tokens, so the rank fits 8 bits.
 constexpr int kRankBits = 8;
-// Most blocks for which every assignment workgroup scans the block histograms itself.
-constexpr int kFusedScanMaxBlocks = 1024;
 static_assert(kMaxBlockTokens <= (1 << kRankBits), "in-block ranks must fit the packed entry");
 constexpr int kRankMask = (1 << kRankBits) - 1;
 
@@ -397,6 +423,7 @@ __device__ __forceinline__ void layout_assign_block(const int32_t* block_counts,
                                                     int num_topk,
                                                     int local_experts,
                                                     int tokens_per_block,
+                                                    int window_blocks,
                                                     int threads,
                                                     int expand,
                                                     int64_t alignment,
@@ -417,11 +444,16 @@ __device__ __forceinline__ void layout_assign_block(const int32_t* block_counts,
     __shared__ int64_t wave_assigned[kMaxBlockTokens / kWave];
     __shared__ int32_t wave_own[kMaxBlockTokens / kWave];
     __shared__ int32_t wave_before[kMaxBlockTokens / kWave];
+    __shared__ int32_t wave_window_before[kMaxBlockTokens / kWave];
     __shared__ int status_bits;
+    __shared__ int own_assignments;
     const int rows = local_experts + 1;
     int32_t* column_total = assign_lds;         // [L+1] totals over all blocks (fused scan only)
     int32_t* slot_base = assign_lds + rows;     // [L+1] assignments before this block -> first slot per expert
-    int32_t* order_base = assign_lds + 2 * rows;  // [L+1] this block's histogram -> its exclusive scan
+    // [L+1] histogram of this block's window (window_blocks consecutive blocks: the unit the slot-order
+    // list is ordered by) -> where an expert's run starts inside the window's part of the list
+    int32_t* order_base = assign_lds + 2 * rows;
+    int32_t* window_before = assign_lds + 3 * rows;  // [L+1] the window's assignments in the blocks before this one
 
     const int tid = threadIdx.x;
     const int block = blockIdx.x;
@@ -435,11 +467,15 @@ __device__ __forceinline__ void layout_assign_block(const int32_t* block_counts,
         packed[k] = live ? packed_rank[token * num_topk + (k < num_topk ? k : 0)] : -1;
 
     if (kFusedScan) {
-        for (int i = tid; i < 2 * rows; i += threads)
+        for (int i = tid; i < 4 * rows; i += threads)
             assign_lds[i] = 0;
-        if (tid == 0)
+        if (tid == 0) {
             status_bits = 0;
+            own_assignments = 0;
+        }
         __syncthreads();
+        const int window_first = block / window_blocks * window_blocks;
+        const int window_end = window_first + window_blocks;
 
         const int columns_per_pass = rows < threads ? rows : threads;
         const int segments = threads / columns_per_pass;
@@ -455,18 +491,23 @@ __device__ __forceinline__ void layout_assign_block(const int32_t* block_counts,
             const int second = column + columns_per_pass;
             const bool active = segment < segments && column < rows;
             const bool active_second = segment < segments && second < rows;
-            int total[2] = {0, 0}, before[2] = {0, 0}, own[2] = {0, 0};
+            int total[2] = {0, 0}, before[2] = {0, 0}, own[2] = {0, 0}, window[2] = {0, 0}, earlier[2] = {0, 0};
             if (active) {
 #pragma unroll 8
                 for (int b = begin; b < end; ++b) {
                     const int count = block_counts[static_cast<int64_t>(b) * rows + column];
                     const int count_second = active_second ? block_counts[static_cast<int64_t>(b) * rows + second] : 0;
+                    const bool in_window = b >= window_first && b < window_end;
                     total[0] += count;
                     total[1] += count_second;
                     before[0] += b < block ? count : 0;
                     before[1] += b < block ? count_second : 0;
                     own[0] = b == block ? count : own[0];
                     own[1] = b == block ? count_second : own[1];
+                    window[0] += in_window ? count : 0;
+                    window[1] += in_window ? count_second : 0;
+                    earlier[0] += in_window && b < block ? count : 0;
+                    earlier[1] += in_window && b < block ? count_second : 0;
                 }
             }
             for (int i = 0; i < 2; ++i) {
@@ -476,12 +517,18 @@ __device__ __forceinline__ void layout_assign_block(const int32_t* block_counts,
                 if (segments == 1) {
                     column_total[at] = total[i];
                     slot_base[at] = before[i];
+                    order_base[at] = window[i];
+                    window_before[at] = earlier[i];
                 } else {
                     atomicAdd(&column_total[at], total[i]);
                     atomicAdd(&slot_base[at], before[i]);
+                    if (window[i] != 0)
+                        atomicAdd(&order_base[at], window[i]);
+                    if (earlier[i] != 0)
+                        atomicAdd(&window_before[at], earlier[i]);
                 }
-                if (block >= begin && block < end)
-                    order_base[at] = own[i];
+                if (at < local_experts && own[i] != 0)
+                    atomicAdd(&own_assignments, own[i]);
             }
         }
         if (block == 0) {
@@ -502,6 +549,7 @@ __device__ __forceinline__ void layout_assign_block(const int32_t* block_counts,
             else
                 next = static_cast<int32_t>(column < local_experts ? expert_counts[column] : send_counts[0]);
             order_base[column] = next - before;
+            window_before[column] = 0;  // the window is this block alone
             slot_base[column] = before;
         }
     }
@@ -511,7 +559,7 @@ __device__ __forceinline__ void layout_assign_block(const int32_t* block_counts,
     const int first = tid * per_thread < local_experts ? tid * per_thread : local_experts;
     const int last = first + per_thread < local_experts ? first + per_thread : local_experts;
     int64_t padded_sum = 0, count_sum = 0;
-    int own_sum = 0, before_sum = 0;
+    int own_sum = 0, before_sum = 0, window_before_sum = 0;  // own_sum: the window's assignments (see order_base)
     for (int e = first; e < last; ++e) {
         if (kFusedScan) {
             const int64_t count = column_total[e];
@@ -520,11 +568,13 @@ __device__ __forceinline__ void layout_assign_block(const int32_t* block_counts,
         }
         own_sum += order_base[e];
         before_sum += slot_base[e];
+        window_before_sum += window_before[e];
     }
     const int64_t padded_scan = kFusedScan ? wave_inclusive_scan(padded_sum) : 0;
     const int64_t assigned_scan = kFusedScan ? wave_inclusive_scan(count_sum) : 0;
     const int own_scan = static_cast<int>(wave_inclusive_scan(own_sum));
     const int before_scan = static_cast<int>(wave_inclusive_scan(before_sum));
+    const int window_before_scan = static_cast<int>(wave_inclusive_scan(window_before_sum));
     const int wave = tid / kWave;
     const int waves = threads / kWave;
     if ((tid & (kWave - 1)) == kWave - 1) {
@@ -532,20 +582,25 @@ __device__ __forceinline__ void layout_assign_block(const int32_t* block_counts,
         wave_assigned[wave] = assigned_scan;
         wave_own[wave] = own_scan;
         wave_before[wave] = before_scan;
+        wave_window_before[wave] = window_before_scan;
     }
     __syncthreads();
     int64_t running = padded_scan - padded_sum;
     int running_own = own_scan - own_sum;
     int64_t capacity = 0, assigned = 0;
-    int own_total = 0, assigned_before = 0;  // this block's assignments, and those of the blocks before it
+    // the window's assignments, those of all blocks before this one, and the window's share of the latter
+    int window_total = 0, assigned_before = 0, window_earlier = 0;
     for (int w = 0; w < waves; ++w) {
         running += w < wave ? wave_padded[w] : 0;
         running_own += w < wave ? wave_own[w] : 0;
         capacity += wave_padded[w];
         assigned += wave_assigned[w];
-        own_total += wave_own[w];
+        window_total += wave_own[w];
         assigned_before += wave_before[w];
+        window_earlier += wave_window_before[w];
     }
+    // this block's own assignments: the window's when the window is the block
+    const int own_total = kFusedScan ? own_assignments : window_total;
     if (!kFusedScan)
         assigned = totals[0];
     for (int e = first; e < last; ++e) {
@@ -560,9 +615,9 @@ __device__ __forceinline__ void layout_assign_block(const int32_t* block_counts,
         } else {
             slot_base[e] += static_cast<int32_t>(expert_offsets[e]);
         }
-        const int own = order_base[e];
-        order_base[e] = running_own;
-        running_own += own;
+        const int in_window = order_base[e];
+        order_base[e] = running_own + window_before[e];  // behind the expert's entries of the window's earlier blocks
+        running_own += in_window;
     }
     if (kFusedScan && block == 0 && tid == 0) {
         const int64_t received = column_total[local_experts];
@@ -576,19 +631,25 @@ __device__ __forceinline__ void layout_assign_block(const int32_t* block_counts,
         __hip_atomic_store(&host_counts[0], received, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_SYSTEM);
     }
     __syncthreads();
-    // The list is dense: this block's run starts where the earlier blocks' assignments end.  Every
-    // block also clears as many entries of the unused tail [A, entries) as it has masked choices.
+    // The list is dense: a window's part starts where the assignments of the blocks before the window
+    // end.  Every block also clears as many entries of the unused tail as it has masked choices.
     int64_t* order = nullptr;
     if (slot_order != nullptr) {
-        order = slot_order + assigned_before;
+        order = slot_order + (assigned_before - window_earlier);
         const int64_t block_entries = static_cast<int64_t>(tokens_per_block) * num_topk;
         int64_t* tail = slot_order + assigned + (block * block_entries - assigned_before);
         const int holes = static_cast<int>(block_entries) - own_total;
         for (int i = tid; i < holes; i += threads)
             tail[i] = -1;
+        // The buffer's size does not depend on the block size: (T rounded up to 256) * K entries, then
+        // the count word.  The last block (the one with the fewest tokens) clears what lies behind
+        // the blocks' own entries, so that everything from entry A to the count word reads -1.
+        const int64_t capacity_entries = (num_tokens + kMaxBlockTokens - 1) / kMaxBlockTokens * kMaxBlockTokens * num_topk;
+        if (block == num_blocks - 1)
+            for (int64_t i = num_blocks * block_entries + tid; i < capacity_entries; i += threads)
+                slot_order[i] = -1;
         if (block == 0 && tid == 0)
-            // count word: last word of the buffer, whose size does not depend on the block size
-            slot_order[(num_tokens + kMaxBlockTokens - 1) / kMaxBlockTokens * kMaxBlockTokens * num_topk] = assigned;
+            slot_order[capacity_entries] = assigned;
     }
     if (live)
         assign_token_slots<kCap>(token, num_topk, expand, row_in_block, slot_base[local_experts], slot_base, order_base,
@@ -603,6 +664,7 @@ __global__ void __launch_bounds__(kMaxBlockTokens) layout_assign_kernel(const in
                                                             int num_topk,
                                                             int local_experts,
                                                             int tokens_per_block,
+                                                            int window_blocks,
                                                             int threads,
                                                             int expand,
                                                             int64_t alignment,
@@ -619,7 +681,7 @@ __global__ void __launch_bounds__(kMaxBlockTokens) layout_assign_kernel(const in
                                                             int32_t* token_slots,
                                                             int64_t* slot_order) {
     layout_assign_block<kCap, kFusedScan>(block_counts, block_status, num_blocks, num_tokens, num_topk, local_experts,
-                                          tokens_per_block, threads, expand, alignment, packed_rank, local_row, expert_counts,
+                                          tokens_per_block, window_blocks, threads, expand, alignment, packed_rank, local_row, expert_counts,
                                           expert_offsets, send_counts, recv_rank_prefix, totals, host_counts, recv_metadata,
                                           dst_slots, token_slots, slot_order);
 }
@@ -653,7 +715,7 @@ __global__ void __launch_bounds__(kMaxBlockTokens) layout_single_block_kernel(co
                              block_status, packed_rank, local_row);
     __threadfence();
     __syncthreads();
-    layout_assign_block<kCap, true>(block_counts, block_status, 1, num_tokens, num_topk, local_experts, words * 32, threads,
+    layout_assign_block<kCap, true>(block_counts, block_status, 1, num_tokens, num_topk, local_experts, words * 32, 1, threads,
                                     expand, alignment, packed_rank, local_row, expert_counts, expert_offsets, send_counts,
                                     recv_rank_prefix, nullptr, host_counts, recv_metadata, dst_slots, token_slots, slot_order);
 }
@@ -673,7 +735,12 @@ size_t nanoep_layout_workspace_bytes(int64_t num_tokens, int num_topk, int64_t n
 }
 
 int nanoep_layout_block_tokens(int64_t num_tokens, int64_t num_local_experts, int hidden) {
-    return num_local_experts <= 0 || num_tokens < 0 || hidden < 0 ? 0 : layout_tokens_per_block(num_tokens, num_local_experts, hidden);
+    if (num_local_experts <= 0 || num_tokens < 0 || hidden < 0)
+        return 0;
+    // tokens the slot-order list is ordered by: the layout workgroup's tokens times the blocks of a window
+    const int per_block = layout_tokens_per_block(num_tokens, num_local_experts, hidden);
+    const bool fused = layout_uses_fused_scan(num_tokens, num_local_experts, hidden);
+    return per_block * layout_window_blocks(num_tokens, num_local_experts, hidden, fused);
 }
 
 int64_t nanoep_slot_order_entries(int64_t num_tokens, int num_topk, int64_t num_local_experts) {
@@ -720,18 +787,15 @@ int nanoep_layout(const int64_t* topk_idx, int64_t num_tokens, int num_topk, int
     // 1024 blocks whatever the expert count (8192 tokens, 256 experts: 21 against 27 us; 262144
     // tokens: 159 against 198 us).  Beyond, the blocks^2 loads lose (2^20 tokens, 8 experts: 124
     // against 67 us) and a third launch does the scan once.
-    bool fused_scan = blocks > 0 && blocks <= kFusedScanMaxBlocks;
+    const bool fused_scan = layout_uses_fused_scan(num_tokens, num_local_experts, hidden);
     const int forced_launches = env_int("NANOEP_LAYOUT_LAUNCHES", 0);
-    if (forced_launches == 3)
-        fused_scan = false;
-    else if (forced_launches == 2 && blocks > 0)
-        fused_scan = true;
+    const int window_blocks = layout_window_blocks(num_tokens, num_local_experts, hidden, fused_scan);
     hipError_t launch_status = hipSuccess;
     with_topk_cap(num_topk, [&](auto cap) {
         constexpr int kCap = decltype(cap)::value;
         if (blocks == 1 && forced_launches == 0) {
             const size_t count_lds = static_cast<size_t>(experts + 1) * (words * 6 + 4);
-            const size_t assign_lds = static_cast<size_t>(experts + 1) * 12;
+            const size_t assign_lds = static_cast<size_t>(experts + 1) * 16;
             layout_single_block_kernel<kCap><<<1, count_threads, count_lds > assign_lds ? count_lds : assign_lds, stream>>>(
                 topk_idx, num_tokens, num_topk, experts, words, count_threads, expand, alignment, topk_snapshot,
                 ws.block_counts, ws.block_status, ws.packed_rank, ws.local_row, expert_counts, expert_offsets, send_counts,
@@ -747,11 +811,11 @@ int nanoep_layout(const int64_t* topk_idx, int64_t num_tokens, int num_topk, int
             if ((launch_status = hipGetLastError()) != hipSuccess)
                 return;
         }
-        const size_t assign_lds = static_cast<size_t>(experts + 1) * 12;
+        const size_t assign_lds = static_cast<size_t>(experts + 1) * 16;
         if (fused_scan) {
             layout_assign_kernel<kCap, true><<<blocks, count_threads, assign_lds, stream>>>(
-                ws.block_counts, ws.block_status, blocks, num_tokens, num_topk, experts, tokens_per_block, count_threads,
-                expand, alignment, ws.packed_rank, ws.local_row, expert_counts, expert_offsets, send_counts,
+                ws.block_counts, ws.block_status, blocks, num_tokens, num_topk, experts, tokens_per_block, window_blocks,
+                count_threads, expand, alignment, ws.packed_rank, ws.local_row, expert_counts, expert_offsets, send_counts,
                 recv_rank_prefix, ws.totals, host_counts, recv_metadata, dst_slots, token_slots, slot_order);
             launch_status = hipGetLastError();
             return;
@@ -763,7 +827,7 @@ int nanoep_layout(const int64_t* topk_idx, int64_t num_tokens, int num_topk, int
             return;
         if (blocks > 0) {
             layout_assign_kernel<kCap, false><<<blocks, count_threads, assign_lds, stream>>>(
-                ws.block_counts, ws.block_status, blocks, num_tokens, num_topk, experts, tokens_per_block, count_threads,
+                ws.block_counts, ws.block_status, blocks, num_tokens, num_topk, experts, tokens_per_block, 1, count_threads,
                 expand, alignment, ws.packed_rank, ws.local_row, expert_counts, expert_offsets, send_counts,
                 recv_rank_prefix, ws.totals, host_counts, recv_metadata, dst_slots, token_slots, slot_order);
             launch_status = hipGetLastError();

@@ -72,11 +72,14 @@ def test_argument_checks_come_before_any_device_work():
     assert library.nanoep_slot_order_entries(100, 3, 8) == 256 * 3 + 1 and library.nanoep_slot_order_entries(0, 3, 8) == 0
     assert library.nanoep_layout_block_tokens(4096, 6000, 0) == 0 and library.nanoep_layout_block_tokens(4096, 0, 0) == 0
     sizes = (1, 256, 257, 512, 1024, 1536, 1792, 1793, 2048, 4095, 4096, 100000)
-    for hidden in (0, 2048, 7168):
+    for hidden in (0, 7168):
         assert [library.nanoep_layout_block_tokens(t, 256, hidden) for t in sizes] == [256, 256, 64, 64, 128, 128, 128, 256, 256, 256, 256, 256]
-    # a block's rows fit an XCD's 4 MiB L2
-    assert [library.nanoep_layout_block_tokens(100000, 256, h) for h in (8, 8192, 8200, 16384, 16392, 1 << 20)] == [256, 256, 128, 128, 64, 64]
-    assert library.nanoep_layout_block_tokens(100000, 1400, 2048) == 128  # 256-token blocks of 1401 LDS rows do not fit
+    # rows of up to 4096 elements: windows of 512 tokens (two layout blocks) once there are eight of them
+    assert [library.nanoep_layout_block_tokens(t, 256, 2048) for t in sizes] == [256, 256, 64, 64, 128, 128, 128, 256, 256, 512, 512, 512]
+    # a window's rows fit an XCD's 4 MiB L2
+    assert [library.nanoep_layout_block_tokens(100000, 256, h) for h in (8, 4096, 4104, 8192, 8200, 16384, 16392, 1 << 20)] == [512, 512, 256, 256, 128, 128, 64, 64]
+    assert library.nanoep_layout_block_tokens(100000, 1400, 2048) == 512  # four layout blocks of 128 tokens (1401 LDS rows)
+    assert library.nanoep_layout_block_tokens(300000, 256, 2048) == 256  # separate scan launch: the window is the layout block
     assert library.nanoep_layout_block_tokens(4096, 256, -1) == 0
     out = (ctypes.c_int64 * 4)()
     assert library.nanoep_wait_counts(null, null, 0.0, out) == 1
