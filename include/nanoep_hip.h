@@ -63,8 +63,9 @@ size_t nanoep_layout_workspace_bytes(int64_t num_tokens, int num_topk, int64_t n
 /* Tokens of one block ("window") of the slot-order list for T tokens, L local experts and payload
  * rows of `hidden` bf16 elements (0: not known; the answer is 0 when L is not supported).  The list
  * is ordered window of consecutive tokens by window, and a window's rows should fit one XCD's 4 MiB
- * L2: 512 tokens up to hidden 4096, 256 up to 8192 (and when hidden is not known), then 128 and 64;
- * fewer for batches of 257..4095 tokens so that there are eight windows, and the layout workgroup's
+ * L2: 512 tokens up to hidden 4096 (1024 tokens up to hidden 1024), 256 up to 8192 (and when hidden
+ * is not known), then 128 and 64; fewer for batches of 257..4095 tokens so that there are eight
+ * windows (sixteen before a window takes 1024 tokens), and the layout workgroup's
  * own token count when the layout needs its separate scan launch (more than 1024 workgroups). */
 int nanoep_layout_block_tokens(int64_t num_tokens, int64_t num_local_experts, int hidden);
 

@@ -16,21 +16,25 @@ constexpr int64_t kXcdL2Bytes = int64_t{4} << 20;
 // Most blocks for which every assignment workgroup scans the block histograms itself.
 constexpr int kFusedScanMaxBlocks = 1024;
 // Largest window: the run of consecutive tokens the slot-order list is ordered by.
-constexpr int kMaxWindowTokens = 512;
+constexpr int kMaxWindowTokens = 1024;
 
 // Tokens of one window of the slot-order list.
 //  * `hidden` (bf16 elements of a payload row, 0 = not known) sizes the window so that its rows fit an
 //    XCD's L2: 512 tokens up to 4096 elements, 256 up to 8192 (and when it is not known), then 128, 64.
-//  * The dispatch hands every XCD whole windows when there are at least eight of them: batches of
-//    more than 256 tokens take smaller windows (down to 64 tokens) to get there.
+//    Rows of up to 1024 elements take 1024 tokens (half the L2: at 2048 elements a 1024-token window
+//    measured 8 % slower than a 512-token one, at 1024 and 512 elements 5 and 7 % faster).
+//  * The dispatch hands every XCD whole windows when there are at least eight of them (sixteen for
+//    1024-token windows): batches of more than 256 tokens take smaller windows (down to 64 tokens)
+//    to get there.
 int layout_window_tokens(int64_t tokens_total, int hidden) {
     int window = 256;
     if (hidden > 0)
-        for (window = kMaxWindowTokens; window > 64 && static_cast<int64_t>(window) * hidden * 2 > kXcdL2Bytes; window /= 2) {
+        for (window = kMaxWindowTokens;
+             window > 64 && static_cast<int64_t>(window) * hidden * 2 > (window > 512 ? kXcdL2Bytes / 2 : kXcdL2Bytes); window /= 2) {
         }
     if (tokens_total <= 256 && window > 256)
         window = 256;  // one layout block: the whole layout is then a single launch
-    while (tokens_total > 256 && window > 64 && (tokens_total + window - 1) / window < 8)
+    while (tokens_total > 256 && window > 64 && (tokens_total + window - 1) / window < (window > 512 ? 16 : 8))
         window /= 2;
     return window;
 }

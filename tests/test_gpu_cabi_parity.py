@@ -353,6 +353,16 @@ def test_both_layout_launch_plans(device, monkeypatch, hidden, launches, tokens,
     assert_layout(metadata, counts, oracle.layout(idx, experts, alignment), expand, hidden)
 
 
+@pytest.mark.parametrize("tokens,experts,topk,hidden", [(16400, 64, 4, 1024), (15500, 1400, 3, 256), (20001, 8, 2, 512)])
+def test_windows_of_1024_tokens(device, tokens, experts, topk, hidden):
+    """Rows of up to 1024 elements in batches of more than 15 360 tokens: the slot-order list is
+    ordered by windows of 1024 tokens, four layout blocks each (eight when 1400 experts shrink the
+    blocks); ragged last window."""
+    assert cabi.lib().nanoep_layout_block_tokens(tokens, experts, hidden) == 1024
+    idx = cases.routing("dropout", tokens, experts, topk, seed=tokens)
+    run_dispatch_combine(device, idx, hidden, experts, 8, True, True, True, seed=3)
+
+
 @pytest.mark.parametrize("seed", range(24))
 def test_randomized_shapes(device, seed):
     """Seeded random geometries: ragged token counts, hidden sizes that are not multiples of 512 or
