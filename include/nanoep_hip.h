@@ -80,6 +80,8 @@ int64_t nanoep_slot_order_entries(int64_t num_tokens, int num_topk, int64_t num_
  * build_receive_metadata_row (csrc/dispatch_epilogue.cuh:20-47); results follow
  * reference_layout (nano_ep/testing/oracle.py:70-104) with rows and slots in token order.
  *
+ * Limits: T <= 2^31 - 1, K <= 32, L <= 3839 (the assignment kernel keeps four int32 per expert in
+ * LDS), alignment <= 2^31; anything beyond returns NANOEP_ERR_INVALID_ARGUMENT.
  * recv_metadata must have room for T rows; the first N are written.
  * token_slots (optional, int32 [T, K]) receives slot[t,k] (or the local id when !expand), -1 when
  * masked: the same information as dst_slots + recv_metadata in one lookup.  It is not one of the

@@ -444,6 +444,8 @@ DispatchResult dispatch(PeerRuntime& runtime,
         const int64_t count32 = tokens * (topk + 2) + (expand ? tokens * topk : 0);
         const size_t workspace_bytes = nanoep_layout_workspace_bytes(tokens, static_cast<int>(topk), local_experts);
         TORCH_CHECK(workspace_bytes > 0, "unsupported routing geometry for the layout kernels");
+        TORCH_CHECK(nanoep_layout_block_tokens(tokens, local_experts, static_cast<int>(hidden)) > 0,
+                    "the layout kernels take at most 3839 local experts, got ", local_experts);
         torch::Tensor arena64, arena32;
         allocate_for_consumer([&] {
             arena64 = torch::empty({count64}, int64_options);

@@ -71,6 +71,8 @@ def test_argument_checks_come_before_any_device_work():
     assert library.nanoep_slot_order_entries(4096, 8, 256) == 4096 * 8 + 1 and library.nanoep_layout_block_tokens(4096, 256, 0) == 256
     assert library.nanoep_slot_order_entries(100, 3, 8) == 256 * 3 + 1 and library.nanoep_slot_order_entries(0, 3, 8) == 0
     assert library.nanoep_layout_block_tokens(4096, 6000, 0) == 0 and library.nanoep_layout_block_tokens(4096, 0, 0) == 0
+    # most local experts: four int32 per expert (and one more row) in 60 KiB of LDS
+    assert library.nanoep_layout_block_tokens(4096, 3839, 0) == 256 and library.nanoep_layout_block_tokens(4096, 3840, 0) == 0
     sizes = (1, 256, 257, 512, 1024, 1536, 1792, 1793, 2048, 4095, 4096, 100000)
     for hidden in (0, 7168):
         assert [library.nanoep_layout_block_tokens(t, 256, hidden) for t in sizes] == [256, 256, 64, 64, 128, 128, 128, 256, 256, 256, 256, 256]

@@ -363,6 +363,16 @@ def test_windows_of_1024_tokens(device, tokens, experts, topk, hidden):
     run_dispatch_combine(device, idx, hidden, experts, 8, True, True, True, seed=3)
 
 
+@pytest.mark.parametrize("tokens", [300, 5000])
+def test_most_local_experts(device, tokens):
+    """3839 local experts, the most the assignment kernel's LDS arrays take: layout workgroups of
+    32 tokens, eight to a window."""
+    experts = 3839
+    assert cabi.lib().nanoep_layout_block_tokens(tokens, experts, 0) > 0 and cabi.lib().nanoep_layout_block_tokens(tokens, experts + 1, 0) == 0
+    idx = cases.routing("dropout", tokens, experts, 5, seed=tokens)
+    run_dispatch_combine(device, idx, 512, experts, 3, True, True, True, seed=tokens)
+
+
 @pytest.mark.parametrize("seed", range(24))
 def test_randomized_shapes(device, seed):
     """Seeded random geometries: ragged token counts, hidden sizes that are not multiples of 512 or
