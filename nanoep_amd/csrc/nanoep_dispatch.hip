@@ -166,13 +166,16 @@ __global__ void __launch_bounds__(1024) dispatch_rows_kernel(const u32x4* __rest
 
 // The slot-order walk, stripped to what its wavefronts need: a wavefront lives about a microsecond,
 // most of it waiting in a chain of scalar work -> list entry -> source load -> store, so every
-// scalar instruction and branch ahead of the source load is throughput.  Validity is folded into
-// one flag and the load is issued unconditionally (row 0 stands in).  kZeroFill is false when the
-// launch has no gap rows to clear: the copy path then carries none of that bookkeeping.
+// scalar instruction and branch ahead of the source load is throughput (ten more scalar
+// instructions and three taken branches there measured +6 % on the whole kernel).  kZeroFill is
+// false when the launch has no gap rows to clear: the copy path then carries none of that
+// bookkeeping.  kWholeRows is the launch with one workgroup a list entry and one wavefront a piece
+// of the row (rows of 5 to 16 pieces, no side workgroups): block index and wavefront index are
+// the entry and the piece, with no division and no taken branch on the way to the load.
 // kSpan is the number of consecutive 1 KiB chunks a wavefront moves (loads issued back to back,
 // then the stores).  One is best while the source fits the last-level cache; beyond that size the
 // single-chunk walk loses a quarter of its rate and two chunks a wavefront win it back.
-template <bool kDeviceCount, bool kZeroFill, int kSpan>
+template <bool kDeviceCount, bool kZeroFill, int kSpan, bool kWholeRows>
 __global__ void __launch_bounds__(1024) dispatch_ordered_kernel(const u32x4* __restrict__ x,              // [T][vectors]
                                                                 const float* __restrict__ weights,       // [T][K] or null
                                                                 const int64_t* __restrict__ slot_order,  // [entries]
@@ -216,7 +219,7 @@ __global__ void __launch_bounds__(1024) dispatch_ordered_kernel(const u32x4* __r
             copy_per_xcd = (copy_blocks + kNumXcds - 1) / kNumXcds;
         }
     }
-    if (blockIdx.x >= payload_blocks) {
+    if (!kWholeRows && blockIdx.x >= payload_blocks) {
         // The weights of the assignments, one lane per list entry, in workgroups of their own at the
         // end of the grid.  The host asks for them when a row is one or two chunks: hung onto the
         // row's first payload wavefront the weight is a second round trip in every (second) wavefront
@@ -244,19 +247,29 @@ __global__ void __launch_bounds__(1024) dispatch_ordered_kernel(const u32x4* __r
         return;
     }
     const uint32_t block = (blockIdx.x % kNumXcds) * copy_per_xcd + index_in_xcd;
-    if (index_in_xcd >= copy_per_xcd || block >= copy_blocks)
-        return;
-    const uint32_t group = fast_divide(block, parts_magic, parts_shift);
-    const uint32_t part = block - group * parts;
-    const uint32_t candidate = group * rows_per_block + __builtin_amdgcn_readfirstlane(threadIdx.z);
-    const uint32_t chunk = part * chunks_per_block + __builtin_amdgcn_readfirstlane(threadIdx.y);
-    if (candidate >= entries || chunk >= chunks)
-        return;
+    uint32_t candidate, chunk;
+    if (kWholeRows) {
+        // one workgroup a row, as many wavefronts as the row has pieces: the block is the list entry
+        if (index_in_xcd >= copy_per_xcd || block >= entries)
+            return;
+        candidate = block;
+        chunk = __builtin_amdgcn_readfirstlane(threadIdx.y);
+    } else {
+        if (index_in_xcd >= copy_per_xcd || block >= copy_blocks)
+            return;
+        const uint32_t group = fast_divide(block, parts_magic, parts_shift);
+        const uint32_t part = block - group * parts;
+        candidate = group * rows_per_block + __builtin_amdgcn_readfirstlane(threadIdx.z);
+        chunk = part * chunks_per_block + __builtin_amdgcn_readfirstlane(threadIdx.y);
+        if (candidate >= entries || chunk >= chunks)
+            return;
+    }
     const int64_t entry = uniform_load(slot_order + candidate);
     const uint32_t source = static_cast<uint32_t>(entry);
     const uint32_t out_row = static_cast<uint32_t>(static_cast<uint64_t>(entry) >> 32);
-    const bool valid = entry >= 0 && source < source_limit && out_row < out_rows;
-    const uint32_t token = valid ? fast_divide(source, topk_magic, topk_shift) : 0u;
+    if (!(entry >= 0 && source < source_limit && out_row < out_rows))
+        return;
+    const uint32_t token = fast_divide(source, topk_magic, topk_shift);
     const uint32_t vector = chunk * (kSpan * kWave) + threadIdx.x;
     u32x4 data[kSpan];
 #pragma unroll
@@ -264,8 +277,6 @@ __global__ void __launch_bounds__(1024) dispatch_ordered_kernel(const u32x4* __r
         const uint32_t at = vector + s * kWave;
         data[s] = x[static_cast<uint64_t>(token) * vectors + (at < vectors ? at : 0u)];
     }
-    if (!valid)
-        return;
 #pragma unroll
     for (int s = 0; s < kSpan; ++s) {
         const uint32_t at = vector + s * kWave;
@@ -273,7 +284,7 @@ __global__ void __launch_bounds__(1024) dispatch_ordered_kernel(const u32x4* __r
             store_vec<true>(recv_x + static_cast<uint64_t>(out_row) * vectors + at, data[s]);
     }
     // no workgroups behind the payload: the row's first wavefront moves its weight
-    if (chunk == 0 && threadIdx.x == 0 && recv_weights != nullptr && payload_blocks == gridDim.x)
+    if (chunk == 0 && threadIdx.x == 0 && recv_weights != nullptr && (kWholeRows || payload_blocks == gridDim.x))
         recv_weights[out_row] = weights[source];
 }
 
@@ -443,8 +454,8 @@ int nanoep_dispatch(const void* x, const float* weights, const int32_t* recv_met
     auto stream = static_cast<hipStream_t>(stream_handle);
     if (ordered) {
         const FastDivisor topk_divisor = make_fast_divisor(static_cast<uint32_t>(num_topk));
-#define NANOEP_LAUNCH_ORDERED_SPAN(DEVICE_COUNT, ZERO_FILL, SPAN)                                                     \
-    dispatch_ordered_kernel<DEVICE_COUNT, ZERO_FILL, SPAN><<<grid, block, 0, stream>>>(                              \
+#define NANOEP_LAUNCH_ORDERED_ROWS(DEVICE_COUNT, ZERO_FILL, SPAN, WHOLE_ROWS)                                         \
+    dispatch_ordered_kernel<DEVICE_COUNT, ZERO_FILL, SPAN, WHOLE_ROWS><<<grid, block, 0, stream>>>(                  \
         static_cast<const u32x4*>(x), weights, slot_order, live_count, expert_counts, expert_offsets,                \
         static_cast<u32x4*>(recv_x), recv_weights, static_cast<uint32_t>(copy_candidates),                           \
         static_cast<uint32_t>(num_tokens * num_topk), static_cast<uint32_t>(out_rows),                               \
@@ -454,6 +465,13 @@ int nanoep_dispatch(const void* x, const float* weights, const int32_t* recv_met
         parts_divisor.magic, parts_divisor.shift, blocking.chunks_per_block, blocking.rows_per_block,                \
         static_cast<uint32_t>(vectors), static_cast<uint32_t>(chunks), topk_divisor.magic, topk_divisor.shift,       \
         static_cast<uint32_t>(payload_blocks))
+#define NANOEP_LAUNCH_ORDERED_SPAN(DEVICE_COUNT, ZERO_FILL, SPAN)             \
+    do {                                                                      \
+        if (whole_rows)                                                       \
+            NANOEP_LAUNCH_ORDERED_ROWS(DEVICE_COUNT, ZERO_FILL, SPAN, true);  \
+        else                                                                  \
+            NANOEP_LAUNCH_ORDERED_ROWS(DEVICE_COUNT, ZERO_FILL, SPAN, false); \
+    } while (0)
 #define NANOEP_LAUNCH_ORDERED(DEVICE_COUNT, ZERO_FILL)             \
     do {                                                           \
         if (span == 2)                                             \
@@ -461,6 +479,14 @@ int nanoep_dispatch(const void* x, const float* weights, const int32_t* recv_met
         else                                                       \
             NANOEP_LAUNCH_ORDERED_SPAN(DEVICE_COUNT, ZERO_FILL, 1); \
     } while (0)
+        // a workgroup per list entry with a wavefront per piece of the row: the kernel then needs no
+        // division to find its entry and piece (4096 x 7168: 81.5 -> 80.4 us, with alignment 128
+        // 100.6 -> 96.9 us, 8192 x 5120: 123.1 -> 120.3 us).  Rows of four pieces are better off
+        // with the general path (8192 x 2048 with cache-resident sources: 37.6 against 38.3 us).
+        const int whole_rows_switch = env_int("NANOEP_DISPATCH_WHOLE_ROWS", -1);
+        const bool whole_rows = blocking.parts == 1 && blocking.rows_per_block == 1 &&
+                                blocking.chunks_per_block == static_cast<unsigned>(chunks) && side_blocks == 0 &&
+                                (whole_rows_switch < 0 ? chunks >= 5 : whole_rows_switch != 0);
         if (live_count != nullptr && pad_blocks > 0)
             NANOEP_LAUNCH_ORDERED(true, true);
         else if (live_count != nullptr)
@@ -471,6 +497,7 @@ int nanoep_dispatch(const void* x, const float* weights, const int32_t* recv_met
             NANOEP_LAUNCH_ORDERED(false, false);
 #undef NANOEP_LAUNCH_ORDERED
 #undef NANOEP_LAUNCH_ORDERED_SPAN
+#undef NANOEP_LAUNCH_ORDERED_ROWS
     } else if (!expand) {
         const int64_t blocks = (num_tokens + blocking.rows_per_block - 1) / blocking.rows_per_block * blocking.parts;
         // one lane per (token, k) for the ids and weights, when the caller wants either

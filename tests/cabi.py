@@ -130,12 +130,14 @@ def slot_order_of(metadata, use_order=True):
 
 
 def dispatch(x, weights, metadata, counts, num_local_experts, alignment, expand, zero_padding, *, num_cus=0, poison=None,
-             use_table=True, use_order=True, order_count="exact", walk="forced", span=None):
+             use_table=True, use_order=True, order_count="exact", walk="forced", span=None, whole_rows=None):
     """Returns (recv_x, recv_topk_idx | None, recv_weights | None) through nanoep_dispatch.
 
     walk="forced" sets the library's switch for the slot-order walk explicitly, walk="auto" leaves
     the environment alone (the library then walks the list whenever it is given one).  span=1|2
     forces the number of chunks a wavefront of that walk moves (the library picks it by source size).
+    whole_rows=0|1 forces or forbids that walk's kernel variant for one workgroup a list entry (the
+    library takes it for rows of five pieces and more whose workgroup covers the row).
     """
     recv_metadata, expert_counts, expert_offsets, dst_slots = metadata[0], metadata[1], metadata[2], metadata[3]
     received, capacity = counts[0], counts[1]
@@ -158,6 +160,9 @@ def dispatch(x, weights, metadata, counts, num_local_experts, alignment, expand,
     order_entries = 0 if order is None else (counts[2] if order_count == "exact" else -1)
     previous = os.environ.pop("NANOEP_DISPATCH_ORDER", None)
     previous_span = os.environ.pop("NANOEP_DISPATCH_SPAN", None)
+    previous_rows = os.environ.pop("NANOEP_DISPATCH_WHOLE_ROWS", None)
+    if whole_rows is not None:
+        os.environ["NANOEP_DISPATCH_WHOLE_ROWS"] = str(int(whole_rows))
     if walk == "forced":
         os.environ["NANOEP_DISPATCH_ORDER"] = "1"
     if span is not None:
@@ -172,6 +177,9 @@ def dispatch(x, weights, metadata, counts, num_local_experts, alignment, expand,
     finally:
         os.environ.pop("NANOEP_DISPATCH_ORDER", None)
         os.environ.pop("NANOEP_DISPATCH_SPAN", None)
+        os.environ.pop("NANOEP_DISPATCH_WHOLE_ROWS", None)
+        if previous_rows is not None:
+            os.environ["NANOEP_DISPATCH_WHOLE_ROWS"] = previous_rows
         if previous is not None:
             os.environ["NANOEP_DISPATCH_ORDER"] = previous
         if previous_span is not None:

@@ -100,6 +100,16 @@ def run_dispatch_combine(device, idx, hidden, experts, alignment, expand, zero_p
             )
             assert torch.equal(wide_x.view(torch.int16), got_x.view(torch.int16))
             assert wide_w is None or torch.equal(wide_w.view(torch.int32), got_w.view(torch.int32))
+        # ... so must both kernel variants of that walk (one workgroup a list entry without any
+        # division, and the general one), with either entry count and either width
+        for whole_rows in (0, 1):
+            for order_count, span in (("exact", 1), ("device", 1), ("exact", 2)):
+                rows_x, _, rows_w = cabi.dispatch(
+                    x.to(device), None if w is None else w.to(device), metadata, counts, experts, alignment, expand, zero_padding,
+                    num_cus=num_cus, poison=POISON, order_count=order_count, span=span, whole_rows=whole_rows,
+                )
+                assert torch.equal(rows_x.view(torch.int16), got_x.view(torch.int16))
+                assert rows_w is None or torch.equal(rows_w.view(torch.int32), got_w.view(torch.int32))
         # ... so must the same call with the library's switches left alone
         auto_x, _, auto_w = cabi.dispatch(
             x.to(device), None if w is None else w.to(device), metadata, counts, experts, alignment, expand, zero_padding,
