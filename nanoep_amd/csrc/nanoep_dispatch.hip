@@ -271,6 +271,12 @@ __global__ void __launch_bounds__(1024) dispatch_ordered_kernel(const u32x4* __r
         return;
     const uint32_t token = fast_divide(source, topk_magic, topk_shift);
     const uint32_t vector = chunk * (kSpan * kWave) + threadIdx.x;
+    // no workgroups behind the payload: the row's first wavefront moves its weight, fetched through
+    // the scalar path while the payload load is in flight
+    const bool carries_weight = chunk == 0 && recv_weights != nullptr && (kWholeRows || payload_blocks == gridDim.x);
+    float weight = 0.0f;
+    if (carries_weight)
+        weight = uniform_load(weights + source);
     u32x4 data[kSpan];
 #pragma unroll
     for (int s = 0; s < kSpan; ++s) {
@@ -283,9 +289,8 @@ __global__ void __launch_bounds__(1024) dispatch_ordered_kernel(const u32x4* __r
         if (at < vectors)
             store_vec<true>(recv_x + static_cast<uint64_t>(out_row) * vectors + at, data[s]);
     }
-    // no workgroups behind the payload: the row's first wavefront moves its weight
-    if (chunk == 0 && threadIdx.x == 0 && recv_weights != nullptr && (kWholeRows || payload_blocks == gridDim.x))
-        recv_weights[out_row] = weights[source];
+    if (carries_weight && threadIdx.x == 0)
+        recv_weights[out_row] = weight;
 }
 
 // Compact layout: receive row r holds source token src_token(r), in token order, so the dispatch is
