@@ -486,11 +486,11 @@ DispatchResult dispatch(PeerRuntime& runtime,
         // them before launching the permute would leave the GPU idle for a host round trip, so the
         // outputs are allocated at their upper bound (every choice valid plus every expert's worst
         // alignment gap), the permute is enqueued right behind the layout, and the results are
-        // narrowed to the exact shapes afterwards.  When the bound is far above what routing can
-        // need (huge alignments) the exact-allocation order is kept.
+        // narrowed to the exact shapes afterwards.  When the gaps alone could exceed the assignments
+        // (the bound is then more than twice what routing can fill) the exact-allocation order is kept.
         const int64_t gap_bound = expand ? local_experts * (alignment - 1) : 0;
         const int64_t row_bound = expand ? tokens * topk + gap_bound : tokens;
-        const bool speculative = tokens > 0 && gap_bound <= tokens * topk / 4 + 1024 && row_bound <= std::numeric_limits<int32_t>::max();
+        const bool speculative = tokens > 0 && gap_bound <= tokens * topk + 1024 && row_bound <= std::numeric_limits<int32_t>::max();
         if (speculative) {
             allocate_outputs(row_bound, tokens);
             launch_permute(metadata, tokens, row_bound, /*count_on_device=*/true);
