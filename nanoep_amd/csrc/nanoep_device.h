@@ -160,7 +160,6 @@ struct RowBlocking {
 enum WalkShape {
     kTokenOrderWalk,  // two-wavefront workgroups: best or within noise of best for the expanded token-order walks
     kSlotOrderWalk,   // one workgroup a row up to 16 wavefronts, an even split beyond
-    kSlotOrderWalkDeviceCount,  // the same walk when the kernel reads its entry count: up to 8 wavefronts
     kRowCopyWalk,     // compact layouts (plain row copies): single-wavefront workgroups
 };
 
@@ -169,12 +168,13 @@ inline RowBlocking pick_row_blocking(int chunks, WalkShape shape) {
     int per_block = env_int("NANOEP_CHUNKS_PER_BLOCK", 0);
     if (per_block < 1 || per_block > kMaxWavesPerBlock) {
         per_block = kDefaultChunksPerBlock;
-        if (shape == kSlotOrderWalk || shape == kSlotOrderWalkDeviceCount) {
+        if (shape == kSlotOrderWalk) {
             // measured on long timed regions: one 14-wavefront workgroup a row against two of 7:
             // 4096 x 7168: 83.7 -> 81.7 us, 8192 x 6144: 145.7 -> 139.7 us (2-wavefront workgroups: 91 us).
-            // A fresh dispatch, whose grid is sized for every choice being valid, is better off
-            // with the smaller workgroups: 100 against 104 us on the device at 4096 x 7168.
-            const int most = shape == kSlotOrderWalk ? kMaxWavesPerBlock : 8;
+            // The same holds for a fresh dispatch, whose grid is sized for every choice being valid
+            // (host-visible, cold sources, 4096 x 7168: 125.0 -> 118.6 us; no difference with
+            // alignment 128 or with cache-resident sources).
+            const int most = kMaxWavesPerBlock;
             const int pieces = (chunks + most - 1) / most;
             per_block = (chunks + pieces - 1) / pieces;
         } else if (shape == kRowCopyWalk) {

@@ -424,8 +424,7 @@ int nanoep_dispatch(const void* x, const float* weights, const int32_t* recv_met
             span = forced_span;
         chunks = (chunks + span - 1) / span;
     }
-    const WalkShape walk = !ordered ? (expand ? kTokenOrderWalk : kRowCopyWalk)
-                           : live_count != nullptr ? kSlotOrderWalkDeviceCount : kSlotOrderWalk;
+    const WalkShape walk = ordered ? kSlotOrderWalk : expand ? kTokenOrderWalk : kRowCopyWalk;
     const RowBlocking blocking = pick_row_blocking(chunks, walk);
     const int64_t waves = static_cast<int64_t>(blocking.chunks_per_block) * blocking.rows_per_block;
     const int64_t copy_candidates = ordered ? slot_order_entries : expand ? num_tokens * num_topk : num_tokens;
