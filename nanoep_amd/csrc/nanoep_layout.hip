@@ -497,7 +497,7 @@ __device__ __forceinline__ void layout_assign_block(const int32_t* block_counts,
             const bool active_second = segment < segments && second < rows;
             int total[2] = {0, 0}, before[2] = {0, 0}, own[2] = {0, 0}, window[2] = {0, 0}, earlier[2] = {0, 0};
             if (active) {
-#pragma unroll 8
+#pragma unroll 16
                 for (int b = begin; b < end; ++b) {
                     const int count = block_counts[static_cast<int64_t>(b) * rows + column];
                     const int count_second = active_second ? block_counts[static_cast<int64_t>(b) * rows + second] : 0;
