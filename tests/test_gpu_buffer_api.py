@@ -153,6 +153,31 @@ def test_fresh_and_cached_replay(device, monkeypatch, walk, expand, zero_padding
         buffer.close()
 
 
+@pytest.mark.parametrize("alignment,at_bound", [(16, True), (19, True), (20, False), (64, False)])
+def test_fresh_dispatch_allocation_orders(device, alignment, at_bound):
+    """A fresh dispatch allocates its outputs at their upper bound and narrows them while the
+    alignment gaps cannot exceed the assignments by more than 1024 rows (the permute then runs
+    right behind the layout), and exactly, after the host has the counts, beyond: same results."""
+    tokens, experts, topk, hidden = 40, 64, 4, 512
+    assert (experts * (alignment - 1) <= tokens * topk + 1024) == at_bound
+    idx = cases.routing("dropout", tokens, experts, topk, seed=alignment)
+    x = cases.payload(tokens, hidden)
+    w = cases.gate_weights(tokens, topk)
+    with Buffer(None, EPConfig(experts, topk, hidden, tokens)) as buffer:
+        fresh = buffer.dispatch(x.to(device), topk_idx=idx.to(device), weights=w.to(device), do_expand=True,
+                                alignment=alignment, zero_padding=True)
+        lay = assert_dispatch_result(fresh, x, idx, w, experts, True, alignment, True)
+        assert_handle(fresh.handle, lay, True, alignment, buffer)
+        held_rows = fresh.x.untyped_storage().nbytes() // (2 * hidden)
+        if at_bound:
+            assert held_rows >= tokens * topk + experts * (alignment - 1) > fresh.x.shape[0]
+        else:
+            assert held_rows < tokens * topk + experts * (alignment - 1)
+        replay = buffer.dispatch(x.to(device), weights=w.to(device), handle=fresh.handle, zero_padding=True)
+        assert torch.equal(replay.x.view(torch.int16), fresh.x.view(torch.int16))
+        assert torch.equal(replay.topk_weights, fresh.topk_weights)
+
+
 @pytest.mark.parametrize(
     "tokens,hidden,switch",
     [
