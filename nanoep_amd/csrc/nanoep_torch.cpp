@@ -19,6 +19,7 @@
 #include <cstdlib>
 #include <limits>
 #include <memory>
+#include <optional>
 #include <string>
 #include <tuple>
 #include <vector>
@@ -116,6 +117,50 @@ class PeerRuntime {
     // already, and a word they store late must not be taken for the answer to a fresh dispatch.
     int64_t* unread_counts() const { return host_counts() + NANOEP_HOST_COUNT_WORDS; }
 
+    // The private handle tensors (slot table, slot-order list) of the latest fresh expanded dispatch.
+    // A caller that keeps only the reference's seven handle tensors gets them back on a replay of
+    // that same handle: the entry is recognised by the identity of the handle's routing snapshot
+    // (the tensor object, its data pointer and version) and of its recv_metadata storage.  The two
+    // tensors are views of the allocations that back the seven public ones.
+    void remember_private(const std::vector<torch::Tensor>& metadata, int64_t alignment) {
+        forget_private();
+        if (metadata.size() < 9 || !metadata[7].defined() || !metadata[8].defined())
+            return;
+        remembered_snapshot_.emplace(metadata[5].getIntrusivePtr());
+        remembered_version_ = tensor_version(metadata[5]);
+        remembered_snapshot_data_ = metadata[5].data_ptr();
+        remembered_metadata_data_ = metadata[0].data_ptr();
+        remembered_rows_ = metadata[0].size(0);
+        remembered_alignment_ = alignment;
+        remembered_table_ = metadata[7];
+        remembered_order_ = metadata[8];
+    }
+
+    // Appends the remembered private tensors to a seven-tensor handle when it is the remembered one
+    // (alignment < 0: the caller does not know the handle's alignment, the identity decides).
+    bool recall_private(std::vector<torch::Tensor>& metadata, int64_t alignment) const {
+        if (closed_ || !remembered_snapshot_.has_value() || metadata.size() != 7)
+            return false;
+        const auto alive = remembered_snapshot_->lock();
+        if (!alive || alive.get() != metadata[5].unsafeGetTensorImpl() || metadata[5].data_ptr() != remembered_snapshot_data_ ||
+            tensor_version(metadata[5]) != remembered_version_ || metadata[0].data_ptr() != remembered_metadata_data_ ||
+            metadata[0].size(0) != remembered_rows_ || (alignment >= 0 && alignment != remembered_alignment_))
+            return false;
+        metadata.push_back(remembered_table_);
+        metadata.push_back(remembered_order_);
+        ++private_recalls_;
+        return true;
+    }
+
+    // number of seven-tensor handles that got their private tensors back (for tests)
+    int64_t private_recalls() const { return private_recalls_; }
+
+    void forget_private() {
+        remembered_snapshot_.reset();
+        remembered_table_ = torch::Tensor();
+        remembered_order_ = torch::Tensor();
+    }
+
     py::bytes export_local_handle() const {
         std::string tag(64, '\0');
         tag.replace(0, 9, "nanoep-r1");
@@ -159,14 +204,28 @@ class PeerRuntime {
             return;
         TORCH_CHECK(!mappings_open_, "close_peer_mappings must run before close");
         window_ = torch::Tensor();
+        forget_private();
         closed_ = true;
     }
 
    private:
+    // in-place edits through torch bump the version; inference tensors have none
+    static uint32_t tensor_version(const torch::Tensor& tensor) {
+        return tensor.is_inference() ? 0u : tensor.unsafeGetTensorImpl()->version_counter().current_version();
+    }
+
     int device_ = 0;
     int64_t num_bytes_ = 0;
     int64_t* host_counts_ = nullptr;
     torch::Tensor window_;
+    std::optional<c10::weak_intrusive_ptr<c10::TensorImpl>> remembered_snapshot_;
+    uint32_t remembered_version_ = 0;
+    const void* remembered_snapshot_data_ = nullptr;
+    const void* remembered_metadata_data_ = nullptr;
+    int64_t remembered_rows_ = 0;
+    int64_t remembered_alignment_ = 0;
+    torch::Tensor remembered_table_, remembered_order_;
+    mutable int64_t private_recalls_ = 0;
     bool mappings_open_ = false;
     bool closed_ = false;
 };
@@ -399,8 +458,12 @@ DispatchResult dispatch(PeerRuntime& runtime,
         // reference only.  The layout is a pure function of the routing snapshot, so the private
         // slot-order list is made again on the device (two small launches, no host wait) and the
         // payload takes the fast walk: 4096 x 7168 top-8 with cold sources 144 -> 99 us.
+        // ... unless the handle is the one of the latest fresh dispatch, whose private tensors
+        // the runtime still has (NANOEP_RECALL_ORDER=0 switches that off).
+        if (expand && recv_count > 0 && env_switch("NANOEP_RECALL_ORDER") != 0)
+            runtime.recall_private(metadata, alignment);
         const int rebuild_switch = env_switch("NANOEP_REBUILD_ORDER");
-        const bool rebuild = expand && recv_count > 0 && cached_metadata.size() == 7 && tokens * topk < (int64_t{1} << 31) &&
+        const bool rebuild = expand && recv_count > 0 && metadata.size() == 7 && tokens * topk < (int64_t{1} << 31) &&
                              (rebuild_switch == 1 || (rebuild_switch != 0 && tokens * hidden * 2 >= kRebuildOrderMinBytes));
         if (rebuild) {
             const int64_t order_entries = nanoep_slot_order_entries(tokens, static_cast<int>(topk), local_experts);
@@ -526,6 +589,8 @@ DispatchResult dispatch(PeerRuntime& runtime,
             if (recv_count > 0)
                 launch_permute(metadata, recv_count, expanded_capacity);
         }
+        if (expand)
+            runtime.remember_private(metadata, alignment);
     }
 
     std::vector<torch::Tensor> outputs{out_x, out_indices, out_weights};
@@ -614,9 +679,16 @@ CombineResult combine(PeerRuntime& runtime,
                                         x.options().dtype(torch::kFloat32));
     }
     if (source_tokens > 0) {
+        // a seven-tensor handle of the latest fresh dispatch gets its slot table back from the runtime
+        std::vector<torch::Tensor> handle;
+        if (expand && metadata.size() == 7 && env_switch("NANOEP_RECALL_ORDER") != 0) {
+            handle = metadata;
+            runtime.recall_private(handle, -1);
+        }
+        const auto& lookup = handle.size() > 7 ? handle : metadata;
         check_status(nanoep_combine(x.data_ptr(), weights.has_value() ? weights->data_ptr<float>() : nullptr,
                                     bias.has_value() ? bias->data_ptr() : nullptr, metadata[0].data_ptr<int32_t>(),
-                                    metadata[3].data_ptr<int64_t>(), slot_table(metadata, source_tokens, topk, expand), recv_count,
+                                    metadata[3].data_ptr<int64_t>(), slot_table(lookup, source_tokens, topk, expand), recv_count,
                                     x.size(0), source_tokens, static_cast<int>(hidden),
                                     static_cast<int>(topk), expand ? 1 : 0, allow_multiple_reduction ? 1 : 0, combined_x.data_ptr(),
                                     weights.has_value() ? combined_weights.data_ptr<float>() : nullptr, cu_budget, comm.stream()),
@@ -678,6 +750,7 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, module) {
         .def("barrier", &nanoep::PeerRuntime::barrier)
         .def("barrier", &nanoep::PeerRuntime::barrier_at)
         .def("close_peer_mappings", &nanoep::PeerRuntime::close_peer_mappings)
+        .def("private_recalls", &nanoep::PeerRuntime::private_recalls)
         .def("close", &nanoep::PeerRuntime::close);
     py::class_<nanoep::CompletionEvent, std::shared_ptr<nanoep::CompletionEvent>>(module, "CompletionEvent")
         .def("current_stream_wait", &nanoep::CompletionEvent::current_stream_wait);

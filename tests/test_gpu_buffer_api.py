@@ -186,12 +186,17 @@ def test_fresh_dispatch_allocation_orders(device, alignment, at_bound):
         pytest.param(2048, 4096, "0", id="16MiB-token-order-forced"),
     ],
 )
-def test_replay_with_only_the_reference_handle_tensors(device, monkeypatch, tokens, hidden, switch):
+@pytest.mark.parametrize("recall", [False, True], ids=["no-recall", "recall"])
+def test_replay_with_only_the_reference_handle_tensors(device, monkeypatch, tokens, hidden, switch, recall):
     """A handle that carries just the reference's seven tensors (as one that went through the
-    reference's own Python class would) replays to the same bytes: the extension makes the private
-    slot-order list again on the device for large payloads, or walks in token order."""
+    reference's own Python class would) replays to the same bytes.  While it is the handle of the
+    buffer's latest fresh dispatch the runtime hands its private tensors back (recall); otherwise
+    the extension makes the slot-order list again on the device for large payloads, or walks in
+    token order."""
     if switch is not None:
         monkeypatch.setenv("NANOEP_REBUILD_ORDER", switch)
+    if not recall:
+        monkeypatch.setenv("NANOEP_RECALL_ORDER", "0")
     experts, topk, alignment = 16, 4, 8
     idx = cases.routing("dropout", tokens, experts, topk, seed=9)
     x, w = cases.payload(tokens, hidden, seed=4), cases.gate_weights(tokens, topk)
@@ -208,14 +213,30 @@ def test_replay_with_only_the_reference_handle_tensors(device, monkeypatch, toke
             full = buffer.dispatch(new_x.to(device), weights=new_w.to(device), handle=fresh.handle, zero_padding=True)
             assert torch.equal(replay.x.view(torch.int16), full.x.view(torch.int16))
             assert torch.equal(replay.topk_weights.view(torch.int32), full.topk_weights.view(torch.int32))
+            assert buffer._runtime.private_recalls() == (step if recall else 0)
         # a fresh dispatch after such replays still reads its own counts
         again = buffer.dispatch(x.to(device), topk_idx=idx.flip(0).contiguous().to(device), do_expand=True, alignment=alignment)
         lay = oracle.layout(idx.flip(0).contiguous(), experts, alignment)
         assert again.handle.layout.recv_count == lay.recv_count and again.handle.layout.expanded_capacity == lay.expanded_capacity
+        # ... and the runtime now remembers that dispatch: the older handle is no longer recalled
+        recalls = buffer._runtime.private_recalls()
         combined = buffer.combine(full.x, bare)
         want, _ = oracle.combine(full.x.cpu(), oracle.layout(idx, experts, alignment).recv_metadata(True),
                                  oracle.layout(idx, experts, alignment).dst_slots, do_expand=True)
         assert_same_bits(combined.x, want, "combine through the bare handle")
+        late = buffer.dispatch(x.to(device), weights=w.to(device), handle=bare, zero_padding=True)
+        assert_dispatch_result(late, x, idx, w, experts, True, alignment, True)
+        assert buffer._runtime.private_recalls() == recalls
+        # the latest one is, by dispatch and by combine
+        newest = dataclasses.replace(again.handle, token_slots=None, slot_order=None)
+        newest_replay = buffer.dispatch(x.to(device), handle=newest)
+        assert_dispatch_result(newest_replay, x, idx.flip(0).contiguous(), None, experts, True, alignment, False)
+        rows = again.handle.layout.expanded_capacity
+        y = cases.payload(rows, hidden, seed=12)
+        flipped = oracle.layout(idx.flip(0).contiguous(), experts, alignment)
+        want_newest, _ = oracle.combine(y, flipped.recv_metadata(True), flipped.dst_slots, do_expand=True)
+        assert_same_bits(buffer.combine(y.to(device), newest).x, want_newest, "combine through the newest bare handle")
+        assert buffer._runtime.private_recalls() == recalls + (2 if recall else 0)
     finally:
         buffer.close()
 
