@@ -19,6 +19,7 @@
 #include <cstdlib>
 #include <limits>
 #include <memory>
+#include <mutex>
 #include <optional>
 #include <string>
 #include <tuple>
@@ -123,7 +124,8 @@ class PeerRuntime {
     // (the tensor object, its data pointer and version) and of its recv_metadata storage.  The two
     // tensors are views of the allocations that back the seven public ones.
     void remember_private(const std::vector<torch::Tensor>& metadata, int64_t alignment) {
-        forget_private();
+        std::lock_guard<std::mutex> lock(private_mutex_);
+        drop_private();
         if (metadata.size() < 9 || !metadata[7].defined() || !metadata[8].defined())
             return;
         remembered_snapshot_.emplace(metadata[5].getIntrusivePtr());
@@ -139,6 +141,7 @@ class PeerRuntime {
     // Appends the remembered private tensors to a seven-tensor handle when it is the remembered one
     // (alignment < 0: the caller does not know the handle's alignment, the identity decides).
     bool recall_private(std::vector<torch::Tensor>& metadata, int64_t alignment) const {
+        std::lock_guard<std::mutex> lock(private_mutex_);
         if (closed_ || !remembered_snapshot_.has_value() || metadata.size() != 7)
             return false;
         const auto alive = remembered_snapshot_->lock();
@@ -156,9 +159,8 @@ class PeerRuntime {
     int64_t private_recalls() const { return private_recalls_; }
 
     void forget_private() {
-        remembered_snapshot_.reset();
-        remembered_table_ = torch::Tensor();
-        remembered_order_ = torch::Tensor();
+        std::lock_guard<std::mutex> lock(private_mutex_);
+        drop_private();
     }
 
     py::bytes export_local_handle() const {
@@ -209,6 +211,12 @@ class PeerRuntime {
     }
 
    private:
+    void drop_private() {
+        remembered_snapshot_.reset();
+        remembered_table_ = torch::Tensor();
+        remembered_order_ = torch::Tensor();
+    }
+
     // in-place edits through torch bump the version; inference tensors have none
     static uint32_t tensor_version(const torch::Tensor& tensor) {
         return tensor.is_inference() ? 0u : tensor.unsafeGetTensorImpl()->version_counter().current_version();
@@ -226,6 +234,7 @@ class PeerRuntime {
     int64_t remembered_alignment_ = 0;
     torch::Tensor remembered_table_, remembered_order_;
     mutable int64_t private_recalls_ = 0;
+    mutable std::mutex private_mutex_;  // dispatch and combine run without the interpreter lock
     bool mappings_open_ = false;
     bool closed_ = false;
 };
