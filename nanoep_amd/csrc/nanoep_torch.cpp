@@ -124,8 +124,9 @@ class PeerRuntime {
     // (the tensor object, its data pointer and version) and of its recv_metadata storage.  The two
     // tensors are views of the allocations that back the seven public ones.
     void remember_private(const std::vector<torch::Tensor>& metadata, int64_t alignment) {
+        torch::Tensor old_table, old_order;  // released after the lock: a tensor's release may want the interpreter lock
         std::lock_guard<std::mutex> lock(private_mutex_);
-        drop_private();
+        drop_private(old_table, old_order);
         if (metadata.size() < 9 || !metadata[7].defined() || !metadata[8].defined())
             return;
         remembered_snapshot_.emplace(metadata[5].getIntrusivePtr());
@@ -159,8 +160,9 @@ class PeerRuntime {
     int64_t private_recalls() const { return private_recalls_; }
 
     void forget_private() {
+        torch::Tensor old_table, old_order;
         std::lock_guard<std::mutex> lock(private_mutex_);
-        drop_private();
+        drop_private(old_table, old_order);
     }
 
     py::bytes export_local_handle() const {
@@ -211,8 +213,10 @@ class PeerRuntime {
     }
 
    private:
-    void drop_private() {
+    void drop_private(torch::Tensor& old_table, torch::Tensor& old_order) {
         remembered_snapshot_.reset();
+        old_table = std::move(remembered_table_);
+        old_order = std::move(remembered_order_);
         remembered_table_ = torch::Tensor();
         remembered_order_ = torch::Tensor();
     }
