@@ -208,12 +208,12 @@ def main():
     with torch.cuda.stream(stream):
         # fresh dispatch: layout kernels + host wait for N/C + permute, as seen by the caller
         fresh_times, fresh_gpu_times = [], []
-        for _ in range(10):
+        for call in range(2 * rotation, -1, -1):  # rotating sources like the timed steps; the last call takes xs[0]
             begin, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
             torch.cuda.synchronize()
             t0 = time.perf_counter()
             begin.record(stream)
-            received = buffer.dispatch(xs[0], topk_idx=idx, weights=weights, do_expand=workload.expand,
+            received = buffer.dispatch(xs[call % rotation], topk_idx=idx, weights=weights, do_expand=workload.expand,
                                        alignment=workload.alignment, zero_padding=workload.zero_padding)
             end.record(stream)
             torch.cuda.synchronize()
