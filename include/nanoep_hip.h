@@ -34,6 +34,7 @@ extern "C" {
 #define NANOEP_ERR_WORKSPACE 3        /* workspace too small */
 #define NANOEP_ERR_TIMEOUT 4          /* host wait for the layout counts timed out */
 #define NANOEP_ERR_ROUTING 5          /* layout kernel saw an expert id outside [-1, L) or a duplicate */
+#define NANOEP_ERR_SCRATCH_LIMIT 6    /* nanoep_layout_static: (T, K, L) needs more than NANOEP_STATIC_SCRATCH_BYTES */
 
 /* Bits of the routing status word the layout kernels publish (host_counts[3]). */
 #define NANOEP_ROUTING_BAD_EXPERT 1
@@ -102,6 +103,27 @@ int nanoep_layout(const int64_t* topk_idx, int64_t num_tokens, int num_topk, int
                   int64_t* expert_offsets, int64_t* dst_slots, int64_t* send_counts, int64_t* topk_snapshot,
                   int64_t* recv_rank_prefix, int32_t* token_slots, int64_t* slot_order, void* workspace,
                   size_t workspace_bytes, int64_t* host_counts, void* stream);
+
+/* Size of the device array behind nanoep_layout_static (4 MiB on every GPU the library runs on). */
+#define NANOEP_STATIC_SCRATCH_BYTES (4u << 20)
+
+/*
+ * nanoep_layout without the workspace arguments, for callers that cannot allocate device memory
+ * (code under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc).  It has
+ * no counterpart in the reference.  The kernels' workspace is a file-scope device array of
+ * NANOEP_STATIC_SCRATCH_BYTES that each GPU holds until the process ends; the call allocates
+ * and frees nothing (its first call on a device looks the array's address up once).  Inputs, outputs
+ * and results are those of nanoep_layout.  A geometry whose workspace
+ * (nanoep_layout_workspace_bytes) exceeds the array returns NANOEP_ERR_SCRATCH_LIMIT before anything
+ * is enqueued: 4096 tokens x top-8 x 256 experts need 0.2 MiB, 32768 tokens 1.7 MiB.
+ * All calls on one GPU share the one array: two calls whose kernels can overlap in time (different
+ * streams, or different threads) race and must be serialized by the caller.
+ */
+int nanoep_layout_static(const int64_t* topk_idx, int64_t num_tokens, int num_topk, int64_t num_local_experts,
+                         int64_t alignment, int expand, int hidden, int32_t* recv_metadata, int64_t* expert_counts,
+                         int64_t* expert_offsets, int64_t* dst_slots, int64_t* send_counts, int64_t* topk_snapshot,
+                         int64_t* recv_rank_prefix, int32_t* token_slots, int64_t* slot_order, int64_t* host_counts,
+                         void* stream);
 
 /* Spin on the mailbox until the layout enqueued on `stream` has published its counts
  * (the reference's wait_dispatch_counts, csrc/peer.cu:198-227).  out = {N, C, A, status}. */

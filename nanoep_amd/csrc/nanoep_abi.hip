@@ -24,7 +24,7 @@ using namespace nanoep;
 
 extern "C" {
 
-int nanoep_abi_version(void) { return 3; }
+int nanoep_abi_version(void) { return 4; }
 
 const char* nanoep_status_string(int status) {
     switch (status) {
@@ -40,6 +40,8 @@ const char* nanoep_status_string(int status) {
             return "timed out waiting for the layout counts";
         case NANOEP_ERR_ROUTING:
             return "routing ids must be -1 or distinct expert ids in [0, num_local_experts)";
+        case NANOEP_ERR_SCRATCH_LIMIT:
+            return "routing geometry needs more layout workspace than the static scratch of nanoep_layout_static holds (4 MiB)";
         default:
             return "unknown status";
     }

@@ -2,7 +2,15 @@
 
 #include <ctime>
 
+#include <mutex>
+
 #include "nanoep_device.h"
+
+// Device memory of nanoep_layout_static: the layout kernels' workspace (block histograms, in-block
+// ranks, receive rows) for callers that cannot allocate.  Every GPU holds its own copy of the array
+// at its own address until the process ends; host code only ever uses the address that
+// hipGetSymbolAddress returns for the current device, never the array's name.
+static __device__ __align__(256) unsigned char scratch[NANOEP_STATIC_SCRATCH_BYTES];
 
 namespace nanoep {
 namespace {
@@ -725,59 +733,35 @@ __global__ void __launch_bounds__(kMaxBlockTokens) layout_single_block_kernel(co
 }
 
 
-}  // namespace
-}  // namespace nanoep
-
-using namespace nanoep;
-
-extern "C" {
-
-size_t nanoep_layout_workspace_bytes(int64_t num_tokens, int num_topk, int64_t num_local_experts) {
-    if (num_tokens < 0 || num_topk <= 0 || num_local_experts <= 0)
-        return 0;
-    return carve_layout_workspace(nullptr, num_tokens, num_topk, num_local_experts).bytes;
-}
-
-int nanoep_layout_block_tokens(int64_t num_tokens, int64_t num_local_experts, int hidden) {
-    if (num_local_experts <= 0 || num_tokens < 0 || hidden < 0)
-        return 0;
-    // tokens the slot-order list is ordered by: the layout workgroup's tokens times the blocks of a window
-    const int per_block = layout_tokens_per_block(num_tokens, num_local_experts, hidden);
-    const bool fused = layout_uses_fused_scan(num_tokens, num_local_experts, hidden);
-    return per_block * layout_window_blocks(num_tokens, num_local_experts, hidden, fused);
-}
-
-int64_t nanoep_slot_order_entries(int64_t num_tokens, int num_topk, int64_t num_local_experts) {
-    if (num_tokens < 0 || num_topk <= 0 || num_local_experts <= 0)
-        return 0;
-    if (layout_smallest_block(num_tokens, num_local_experts) == 0 || num_tokens == 0)
-        return 0;
-    // whole blocks of any size the layout may take, then the count word
-    return (num_tokens + kMaxBlockTokens - 1) / kMaxBlockTokens * kMaxBlockTokens * num_topk + 1;
-}
-
-int nanoep_layout(const int64_t* topk_idx, int64_t num_tokens, int num_topk, int64_t num_local_experts,
-                  int64_t alignment, int expand, int hidden, int32_t* recv_metadata, int64_t* expert_counts,
-                  int64_t* expert_offsets, int64_t* dst_slots, int64_t* send_counts, int64_t* topk_snapshot,
-                  int64_t* recv_rank_prefix, int32_t* token_slots, int64_t* slot_order, void* workspace,
-                  size_t workspace_bytes, int64_t* host_counts, void* stream_handle) {
+// Argument checks shared by the two layout entry points (everything but the workspace).
+int check_layout_arguments(const int64_t* topk_idx, int64_t num_tokens, int num_topk, int64_t num_local_experts, int64_t alignment,
+                           int expand, int hidden, const int32_t* recv_metadata, const int64_t* expert_counts,
+                           const int64_t* expert_offsets, const int64_t* dst_slots, const int64_t* send_counts,
+                           const int64_t* topk_snapshot, const int64_t* recv_rank_prefix, const int64_t* slot_order,
+                           const int64_t* host_counts) {
     if (num_tokens < 0 || num_tokens > INT32_MAX || num_topk <= 0 || num_topk > kMaxTopk || num_local_experts <= 0 ||
         num_local_experts >= (int64_t{1} << (31 - kRankBits)) || alignment <= 0 || alignment > (int64_t{1} << 31) || hidden < 0)
         return NANOEP_ERR_INVALID_ARGUMENT;
     if (expert_counts == nullptr || expert_offsets == nullptr || send_counts == nullptr || recv_rank_prefix == nullptr ||
-        host_counts == nullptr || workspace == nullptr)
+        host_counts == nullptr)
         return NANOEP_ERR_INVALID_ARGUMENT;
     if (num_tokens > 0 && (topk_idx == nullptr || recv_metadata == nullptr || dst_slots == nullptr || topk_snapshot == nullptr))
         return NANOEP_ERR_INVALID_ARGUMENT;
     // the slot-order list packs token * K + k into 32 bits and only exists for the expanded layout
     if (slot_order != nullptr && (!expand || num_tokens * num_topk >= (int64_t{1} << 31)))
         return NANOEP_ERR_INVALID_ARGUMENT;
-    const int tokens_per_block = layout_tokens_per_block(num_tokens, num_local_experts, hidden);
-    if (tokens_per_block == 0)
+    if (layout_tokens_per_block(num_tokens, num_local_experts, hidden) == 0)
         return NANOEP_ERR_INVALID_ARGUMENT;
-    const LayoutWorkspace ws = carve_layout_workspace(workspace, num_tokens, num_topk, num_local_experts);
-    if (ws.bytes > workspace_bytes)
-        return NANOEP_ERR_WORKSPACE;
+    return NANOEP_OK;
+}
+
+// Enqueues the layout launches over a carved workspace; the arguments have been checked.
+int enqueue_layout(const int64_t* topk_idx, int64_t num_tokens, int num_topk, int64_t num_local_experts, int64_t alignment,
+                   int expand, int hidden, int32_t* recv_metadata, int64_t* expert_counts, int64_t* expert_offsets,
+                   int64_t* dst_slots, int64_t* send_counts, int64_t* topk_snapshot, int64_t* recv_rank_prefix,
+                   int32_t* token_slots, int64_t* slot_order, const LayoutWorkspace& ws, int64_t* host_counts,
+                   void* stream_handle) {
+    const int tokens_per_block = layout_tokens_per_block(num_tokens, num_local_experts, hidden);
     const int64_t blocks64 = (num_tokens + tokens_per_block - 1) / tokens_per_block;
     const int blocks = static_cast<int>(blocks64);
     const int experts = static_cast<int>(num_local_experts);
@@ -839,6 +823,105 @@ int nanoep_layout(const int64_t* topk_idx, int64_t num_tokens, int num_topk, int
     });
     NANOEP_HIP_TRY(launch_status);
     return NANOEP_OK;
+}
+
+// Address of this file's `scratch` array on the current device, resolved once per device (each GPU
+// holds its own copy at its own address).
+constexpr int kMaxDevices = 64;
+std::mutex g_static_scratch_mutex;
+void* g_static_scratch[kMaxDevices] = {};
+
+int static_scratch_of_current_device(void** out) {
+    int device = -1;
+    NANOEP_HIP_TRY(hipGetDevice(&device));
+    if (device < 0 || device >= kMaxDevices)
+        return NANOEP_ERR_INVALID_ARGUMENT;
+    std::lock_guard<std::mutex> lock(g_static_scratch_mutex);
+    if (g_static_scratch[device] == nullptr) {
+        void* address = nullptr;
+        NANOEP_HIP_TRY(hipGetSymbolAddress(&address, HIP_SYMBOL(scratch)));
+        if (address == nullptr)
+            return NANOEP_ERR_HIP;
+        g_static_scratch[device] = address;
+    }
+    *out = g_static_scratch[device];
+    return NANOEP_OK;
+}
+
+}  // namespace
+}  // namespace nanoep
+
+using namespace nanoep;
+
+extern "C" {
+
+size_t nanoep_layout_workspace_bytes(int64_t num_tokens, int num_topk, int64_t num_local_experts) {
+    if (num_tokens < 0 || num_topk <= 0 || num_local_experts <= 0)
+        return 0;
+    return carve_layout_workspace(nullptr, num_tokens, num_topk, num_local_experts).bytes;
+}
+
+int nanoep_layout_block_tokens(int64_t num_tokens, int64_t num_local_experts, int hidden) {
+    if (num_local_experts <= 0 || num_tokens < 0 || hidden < 0)
+        return 0;
+    // tokens the slot-order list is ordered by: the layout workgroup's tokens times the blocks of a window
+    const int per_block = layout_tokens_per_block(num_tokens, num_local_experts, hidden);
+    const bool fused = layout_uses_fused_scan(num_tokens, num_local_experts, hidden);
+    return per_block * layout_window_blocks(num_tokens, num_local_experts, hidden, fused);
+}
+
+int64_t nanoep_slot_order_entries(int64_t num_tokens, int num_topk, int64_t num_local_experts) {
+    if (num_tokens < 0 || num_topk <= 0 || num_local_experts <= 0)
+        return 0;
+    if (layout_smallest_block(num_tokens, num_local_experts) == 0 || num_tokens == 0)
+        return 0;
+    // whole blocks of any size the layout may take, then the count word
+    return (num_tokens + kMaxBlockTokens - 1) / kMaxBlockTokens * kMaxBlockTokens * num_topk + 1;
+}
+
+int nanoep_layout(const int64_t* topk_idx, int64_t num_tokens, int num_topk, int64_t num_local_experts,
+                  int64_t alignment, int expand, int hidden, int32_t* recv_metadata, int64_t* expert_counts,
+                  int64_t* expert_offsets, int64_t* dst_slots, int64_t* send_counts, int64_t* topk_snapshot,
+                  int64_t* recv_rank_prefix, int32_t* token_slots, int64_t* slot_order, void* workspace,
+                  size_t workspace_bytes, int64_t* host_counts, void* stream_handle) {
+    const int status = check_layout_arguments(topk_idx, num_tokens, num_topk, num_local_experts, alignment, expand, hidden,
+                                              recv_metadata, expert_counts, expert_offsets, dst_slots, send_counts, topk_snapshot,
+                                              recv_rank_prefix, slot_order, host_counts);
+    if (status != NANOEP_OK)
+        return status;
+    if (workspace == nullptr)
+        return NANOEP_ERR_INVALID_ARGUMENT;
+    const LayoutWorkspace ws = carve_layout_workspace(workspace, num_tokens, num_topk, num_local_experts);
+    if (ws.bytes > workspace_bytes)
+        return NANOEP_ERR_WORKSPACE;
+    return enqueue_layout(topk_idx, num_tokens, num_topk, num_local_experts, alignment, expand, hidden, recv_metadata, expert_counts,
+                          expert_offsets, dst_slots, send_counts, topk_snapshot, recv_rank_prefix, token_slots, slot_order, ws,
+                          host_counts, stream_handle);
+}
+
+int nanoep_layout_static(const int64_t* topk_idx, int64_t num_tokens, int num_topk, int64_t num_local_experts,
+                         int64_t alignment, int expand, int hidden, int32_t* recv_metadata, int64_t* expert_counts,
+                         int64_t* expert_offsets, int64_t* dst_slots, int64_t* send_counts, int64_t* topk_snapshot,
+                         int64_t* recv_rank_prefix, int32_t* token_slots, int64_t* slot_order, int64_t* host_counts,
+                         void* stream_handle) {
+    const int status = check_layout_arguments(topk_idx, num_tokens, num_topk, num_local_experts, alignment, expand, hidden,
+                                              recv_metadata, expert_counts, expert_offsets, dst_slots, send_counts, topk_snapshot,
+                                              recv_rank_prefix, slot_order, host_counts);
+    if (status != NANOEP_OK)
+        return status;
+    // the size is checked before any device is touched
+    if (carve_layout_workspace(nullptr, num_tokens, num_topk, num_local_experts).bytes > NANOEP_STATIC_SCRATCH_BYTES)
+        return NANOEP_ERR_SCRATCH_LIMIT;
+    void* base = nullptr;
+    const int scratch_status = static_scratch_of_current_device(&base);
+    if (scratch_status != NANOEP_OK)
+        return scratch_status;
+    // Nothing in the workspace has to start at zero: the count pass writes every histogram row, status
+    // word, rank entry and receive row that the later passes of the same call read.
+    const LayoutWorkspace ws = carve_layout_workspace(base, num_tokens, num_topk, num_local_experts);
+    return enqueue_layout(topk_idx, num_tokens, num_topk, num_local_experts, alignment, expand, hidden, recv_metadata, expert_counts,
+                          expert_offsets, dst_slots, send_counts, topk_snapshot, recv_rank_prefix, token_slots, slot_order, ws,
+                          host_counts, stream_handle);
 }
 
 int nanoep_wait_counts(int64_t* host_counts, void* stream_handle, double timeout_seconds,

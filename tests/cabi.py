@@ -46,6 +46,7 @@ def lib() -> ctypes.CDLL:
         handle.nanoep_slot_order_entries.restype = i64
         handle.nanoep_slot_order_entries.argtypes = [i64, i, i64]
         handle.nanoep_layout.argtypes = [p, i64, i, i64, i64, i, i, p, p, p, p, p, p, p, p, p, p, sz, p, p]
+        handle.nanoep_layout_static.argtypes = [p, i64, i, i64, i64, i, i, p, p, p, p, p, p, p, p, p, p, p]
         handle.nanoep_wait_counts.argtypes = [p, p, dbl, ctypes.POINTER(i64)]
         handle.nanoep_dispatch.argtypes = [p, p, p, p, p, p, i64, p, p, i64, i64, i64, i, i, i64, i64, i, i, p, p, p, i, p]
         handle.nanoep_combine.argtypes = [p, p, p, p, p, p, i64, i64, i64, i, i, i, i, p, p, i, p]
@@ -80,9 +81,11 @@ def window_layout(ranks, tokens, hidden, topk, experts, multi=False) -> list[int
     return list(out)
 
 
-def layout(topk_idx: torch.Tensor, num_local_experts: int, alignment: int, expand: bool, *, raise_on_routing=True, hidden=0):
+def layout(topk_idx: torch.Tensor, num_local_experts: int, alignment: int, expand: bool, *, raise_on_routing=True, hidden=0,
+           static_scratch=False):
     """Runs the layout kernels and returns (metadata list of 7, or 9 when expanded, (N, C, A, status)).
-    hidden is the row width the handle will be used with (0: not known); it sizes the token blocks."""
+    hidden is the row width the handle will be used with (0: not known); it sizes the token blocks.
+    static_scratch takes nanoep_layout_static (the library's own device array) instead of nanoep_layout."""
     device = topk_idx.device
     tokens, topk = topk_idx.shape
     i64 = dict(dtype=torch.int64, device=device)
@@ -98,16 +101,25 @@ def layout(topk_idx: torch.Tensor, num_local_experts: int, alignment: int, expan
     if expand:
         entries = lib().nanoep_slot_order_entries(tokens, topk, num_local_experts)
         slot_order = torch.full((entries,), -7, dtype=torch.int64, device=device)
-    ws_bytes = lib().nanoep_layout_workspace_bytes(tokens, topk, num_local_experts)
-    workspace = torch.empty(ws_bytes, dtype=torch.uint8, device=device)
     mailbox = torch.empty(HOST_COUNT_WORDS, dtype=torch.int64, pin_memory=True)
-    check(
-        lib().nanoep_layout(
-            ptr(topk_idx), tokens, topk, num_local_experts, alignment, int(expand), hidden, ptr(recv_metadata),
-            ptr(expert_counts), ptr(expert_offsets), ptr(dst_slots), ptr(send_counts), ptr(snapshot), ptr(prefix),
-            ptr(token_slots), ptr(slot_order), ptr(workspace), ws_bytes, mailbox.data_ptr(), stream_handle(),
+    if static_scratch:
+        check(
+            lib().nanoep_layout_static(
+                ptr(topk_idx), tokens, topk, num_local_experts, alignment, int(expand), hidden, ptr(recv_metadata),
+                ptr(expert_counts), ptr(expert_offsets), ptr(dst_slots), ptr(send_counts), ptr(snapshot), ptr(prefix),
+                ptr(token_slots), ptr(slot_order), mailbox.data_ptr(), stream_handle(),
+            )
         )
-    )
+    else:
+        ws_bytes = lib().nanoep_layout_workspace_bytes(tokens, topk, num_local_experts)
+        workspace = torch.empty(ws_bytes, dtype=torch.uint8, device=device)
+        check(
+            lib().nanoep_layout(
+                ptr(topk_idx), tokens, topk, num_local_experts, alignment, int(expand), hidden, ptr(recv_metadata),
+                ptr(expert_counts), ptr(expert_offsets), ptr(dst_slots), ptr(send_counts), ptr(snapshot), ptr(prefix),
+                ptr(token_slots), ptr(slot_order), ptr(workspace), ws_bytes, mailbox.data_ptr(), stream_handle(),
+            )
+        )
     out = (ctypes.c_int64 * HOST_COUNT_WORDS)()
     status = lib().nanoep_wait_counts(mailbox.data_ptr(), stream_handle(), 30.0, out)
     if status != 0 and (raise_on_routing or status != 5):

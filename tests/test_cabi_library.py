@@ -23,9 +23,10 @@ def test_every_declared_symbol_is_exported():
 
 def test_version_and_status_strings():
     library = cabi.lib()
-    assert library.nanoep_abi_version() == 3
-    texts = [library.nanoep_status_string(code).decode() for code in range(0, 7)]
-    assert texts[0] == "ok" and len(set(texts[:6])) == 6 and texts[6] == "unknown status"
+    assert library.nanoep_abi_version() == 4
+    texts = [library.nanoep_status_string(code).decode() for code in range(0, 8)]
+    assert texts[0] == "ok" and len(set(texts[:7])) == 7 and texts[7] == "unknown status"
+    assert "static scratch" in texts[6] and "4 MiB" in texts[6]
     assert library.nanoep_last_hip_error().decode() == ""
 
 
@@ -90,6 +91,17 @@ def test_argument_checks_come_before_any_device_work():
     assert library.nanoep_wait_counts(null, null, 0.0, out) == 1
 
 
+def test_static_layout_checks_arguments_and_its_size_limit_before_any_device_work():
+    library = cabi.lib()
+    null = None
+    assert library.nanoep_layout_static(null, -1, 2, 4, 1, 0, 0, null, null, null, null, null, null, null, null, null, null, null) == 1
+    assert library.nanoep_layout_static(null, 4, 2, 4, 1, 0, 0, null, 8, 8, null, 8, null, 8, null, 8, 8, null) == 1
+    # 4 MiB of static scratch: the headline batch needs 0.2 MiB, 32768 tokens 1.7 MiB, 131072 tokens x top-8 more than 4
+    assert library.nanoep_layout_workspace_bytes(4096, 8, 256) < library.nanoep_layout_workspace_bytes(32768, 8, 256) < (4 << 20)
+    assert library.nanoep_layout_workspace_bytes(131072, 8, 256) > (4 << 20)
+    assert library.nanoep_layout_static(8, 131072, 8, 256, 1, 1, 0, 8, 8, 8, 8, 8, 8, 8, 8, 8, 8, null) == 6
+
+
 @pytest.mark.skipif(shutil.which("gcc") is None, reason="no C compiler")
 def test_plain_c_client_compiles_links_and_runs(tmp_path):
     """The header is C99 and the library links from C without HIP or torch on the include path."""
@@ -102,6 +114,6 @@ def test_plain_c_client_compiles_links_and_runs(tmp_path):
         check=True, capture_output=True, text=True,
     )
     out = subprocess.run([str(binary)], check=True, capture_output=True, text=True, timeout=60).stdout.splitlines()
-    assert out[0] == "abi 3 status 0 window 0 96 160 160 9888"
+    assert out[0] == "abi 4 status 0 window 0 96 160 160 9888"
     assert out[1].startswith("invalid 1 '") and "invalid" in out[1].lower()
     assert out[2] == "sizes 32769 256 1"
