@@ -28,15 +28,15 @@ __device__ __forceinline__ void accumulate(float (&acc)[8], const u32x4 v) {
     acc[7] += bf16_high(v.w);
 }
 
-// One wavefront produces one 1 KiB chunk of one source token's output row.  A workgroup is
-// (64, chunks_per_block, tokens_per_block).  Lane k fetches the token's k-th slot (from
+// Expanded layout.  One wavefront produces one 1 KiB chunk of one source token's output row.  A
+// workgroup is (64, chunks_per_block, tokens_per_block).  Lane k fetches the token's k-th slot (from
 // token_slots[t][k], or dst_slots[t] -> recv_metadata[row][2+k]); the slots are broadcast to
 // scalars, the kGroup rows are fetched with back-to-back nontemporal 128-bit loads (a masked k
 // re-reads row 0 so that the loads stay unconditional) and the valid ones are added in ascending k
 // starting from +0.0f; the optional bias is added once and the sum is rounded to bf16 once.
 template <int kGroup, bool kDirectSlots>
-__global__ void __launch_bounds__(1024) combine_rows_kernel(const u32x4* __restrict__ y,                // [rows][vectors]
-                                                            const float* __restrict__ weights,         // [C] / [N][K] or null
+__global__ void __launch_bounds__(1024) combine_rows_kernel(const u32x4* __restrict__ y,                // [C][vectors]
+                                                            const float* __restrict__ weights,         // [C] or null
                                                             const u32x4* __restrict__ bias,            // [T][vectors] or null
                                                             const int32_t* __restrict__ recv_metadata,  // [N][K+2]
                                                             const int64_t* __restrict__ dst_slots,     // [T]
@@ -54,13 +54,12 @@ __global__ void __launch_bounds__(1024) combine_rows_kernel(const u32x4* __restr
                                                             int vectors,
                                                             int chunks,
                                                             int num_topk,
-                                                            int expand,
                                                             int multiple_reduction) {
     NANOEP_FETCH_ARGS_4(y, weights, bias, out_x);
     NANOEP_FETCH_ARGS_4(recv_metadata, dst_slots, token_slots, out_weights);
     NANOEP_FETCH_ARGS_4(recv_count, y_rows, num_tokens, parts);
     NANOEP_FETCH_ARGS_4(parts_magic, parts_shift, chunks_per_block, tokens_per_block);
-    NANOEP_FETCH_ARGS_4(vectors, chunks, num_topk, expand);
+    NANOEP_FETCH_ARGS_4(vectors, chunks, num_topk, multiple_reduction);
     const int lane = threadIdx.x;
     const uint32_t wave_y = __builtin_amdgcn_readfirstlane(threadIdx.y);
     const uint32_t wave_z = __builtin_amdgcn_readfirstlane(threadIdx.z);
@@ -75,28 +74,22 @@ __global__ void __launch_bounds__(1024) combine_rows_kernel(const u32x4* __restr
     // lanes past the end of a short row re-read vector 0 instead of branching around the loads
     const int load_vector = in_row ? vector : 0;
 
-    // field: expanded slot (or local expert id when compact) of this token's k = lane, -1 when masked
-    int64_t row = -1;
+    // slot: expanded slot of this token's k = lane, -1 when masked
     bool received = true;
-    const int32_t* fields;
+    const int32_t* slots;
     if (kDirectSlots) {
-        fields = token_slots + static_cast<int64_t>(token) * num_topk;
+        slots = token_slots + static_cast<int64_t>(token) * num_topk;
     } else {
-        row = uniform_load(dst_slots + token);
+        const int64_t row = uniform_load(dst_slots + token);
         received = row >= 0 && row < recv_count;
-        fields = recv_metadata + (received ? row : 0) * (num_topk + 2) + 2;
+        slots = recv_metadata + (received ? row : 0) * (num_topk + 2) + 2;
     }
-    // Compact rows need their per-k fields only to return weights: a received row always carries
-    // at least one valid choice, so the payload path skips that dependent load.
-    const bool need_fields = expand || (chunk == 0 && out_weights != nullptr);
-    int field = -1;
-    if (need_fields && received && lane < num_topk)
-        field = fields[lane];
-    const bool valid = expand ? (field >= 0 && field < y_rows) : field >= 0;
+    int slot = -1;
+    if (received && lane < num_topk)
+        slot = slots[lane];
+    const bool valid = slot >= 0 && slot < y_rows;
     const uint64_t valid_mask = __ballot(valid);
-    // compact: the token's single received row stands in for k = 0
-    const uint64_t gather_mask = expand ? valid_mask : ((received && row < y_rows) ? 1ull : 0ull);
-    const int gathered = gather_mask == 0 ? 0 : (expand ? num_topk : 1);
+    const int gathered = valid_mask == 0 ? 0 : num_topk;
 
     u32x4 bias_data = {0u, 0u, 0u, 0u};
     if (bias != nullptr)
@@ -107,18 +100,18 @@ __global__ void __launch_bounds__(1024) combine_rows_kernel(const u32x4* __restr
         u32x4 data[kGroup];
 #pragma unroll
         for (int k = 0; k < kGroup; ++k) {
-            const bool live = (gather_mask >> (base + k)) & 1;
+            const bool live = (valid_mask >> (base + k)) & 1;
             int64_t source_row = 0;
             if (live)
-                source_row = expand ? static_cast<int64_t>(__builtin_amdgcn_readlane(field, (base + k) & (kWave - 1))) : row;
+                source_row = static_cast<int64_t>(__builtin_amdgcn_readlane(slot, (base + k) & (kWave - 1)));
             data[k] = load_vec<true>(y + source_row * vectors + load_vector);
         }
 #pragma unroll
         for (int k = 0; k < kGroup; ++k)
-            if ((gather_mask >> (base + k)) & 1)
+            if ((valid_mask >> (base + k)) & 1)
                 accumulate(acc, data[k]);
     }
-    if (multiple_reduction && expand && __popcll(valid_mask) >= 2) {
+    if (multiple_reduction && __popcll(valid_mask) >= 2) {
 #pragma unroll
         for (int j = 0; j < 8; ++j)
             acc[j] = 0.0f + __uint_as_float(bf16_round(acc[j]) << 16);
@@ -134,12 +127,8 @@ __global__ void __launch_bounds__(1024) combine_rows_kernel(const u32x4* __restr
         store_vec<true>(out_x + static_cast<int64_t>(token) * vectors + vector, packed);
     }
 
-    if (chunk == 0 && out_weights != nullptr && lane < num_topk) {
-        float weight = 0.0f;
-        if (valid)
-            weight = expand ? weights[field] : weights[row * num_topk + lane];
-        out_weights[static_cast<int64_t>(token) * num_topk + lane] = weight;
-    }
+    if (chunk == 0 && out_weights != nullptr && lane < num_topk)
+        out_weights[static_cast<int64_t>(token) * num_topk + lane] = valid ? weights[slot] : 0.0f;
 }
 
 // Expanded layout with at most kTopk <= 4 rows per token and the slot table at hand: the same
@@ -355,7 +344,6 @@ int nanoep_combine(const void* y, const float* weights, const void* bias, const 
     const dim3 grid_with_side(static_cast<unsigned>(blocks + side_blocks));
     const FastDivisor topk_divisor = make_fast_divisor(static_cast<uint32_t>(num_topk));
     auto stream = static_cast<hipStream_t>(stream_handle);
-    const int gathered = expand ? num_topk : 1;
     // the slot table only helps the expanded layout, and only when something was received
     const bool direct = token_slots != nullptr && expand && recv_count > 0;
     const FastDivisor parts_divisor = make_fast_divisor(blocking.parts);
@@ -393,8 +381,7 @@ int nanoep_combine(const void* y, const float* weights, const void* bias, const 
         static_cast<const u32x4*>(y), weights, static_cast<const u32x4*>(bias), recv_metadata, dst_slots,          \
         token_slots, static_cast<u32x4*>(out_x), out_weights, recv_count, y_rows, static_cast<uint32_t>(num_tokens), \
         blocking.parts, parts_divisor.magic, parts_divisor.shift, blocking.chunks_per_block, blocking.rows_per_block,  \
-        vectors, chunks, num_topk, expand ? 1 : 0,                                                                   \
-        multiple_reduction ? 1 : 0)
+        vectors, chunks, num_topk, multiple_reduction ? 1 : 0)
 #define NANOEP_LAUNCH_COMBINE_GROUP(GROUP)    \
     do {                                     \
         if (direct)                          \
@@ -403,13 +390,13 @@ int nanoep_combine(const void* y, const float* weights, const void* bias, const 
             NANOEP_LAUNCH_COMBINE(GROUP, false); \
     } while (0)
     // the group size is the number of rows fetched per pass: the smallest of 1, 2, 4, 8, 16 covering K
-    if (gathered <= 1)
+    if (num_topk <= 1)
         NANOEP_LAUNCH_COMBINE_GROUP(1);
-    else if (gathered <= 2)
+    else if (num_topk <= 2)
         NANOEP_LAUNCH_COMBINE_GROUP(2);
-    else if (gathered <= 4)
+    else if (num_topk <= 4)
         NANOEP_LAUNCH_COMBINE_GROUP(4);
-    else if (gathered <= 8)
+    else if (num_topk <= 8)
         NANOEP_LAUNCH_COMBINE_GROUP(8);
     else
         NANOEP_LAUNCH_COMBINE_GROUP(16);

@@ -10,8 +10,8 @@ namespace {
 // a single store and retires sustains more HBM write bandwidth than one that issues several.
 //
 // A workgroup is (64, chunks_per_block, rows_per_block): threadIdx.y is the chunk, threadIdx.z the
-// destination candidate, so no per-wave division by the chunk count is needed.  Candidates are
-// ordered (source token, k): the K destinations of a token are handled by consecutive workgroups
+// destination candidate, so no per-wave division by the chunk count is needed.  In the token-order
+// walk of the expanded layout (dispatch_rows_kernel) candidates are ordered (source token, k): the K destinations of a token are handled by consecutive workgroups
 // behind one XCD's L2, so only the first read of a source row goes to HBM, and every destination
 // row is written as one contiguous run by the wavefronts of one workgroup.  The source address
 // depends only on the block index, so its load is in flight while the wave-uniform lookups
@@ -68,12 +68,11 @@ __global__ void __launch_bounds__(1024) dispatch_rows_kernel(const u32x4* __rest
                                                              const int32_t* __restrict__ token_slots,   // [T][K] or null
                                                              const int64_t* __restrict__ expert_counts,
                                                              const int64_t* __restrict__ expert_offsets,
-                                                             u32x4* __restrict__ recv_x,                // [C or N][vectors]
-                                                             int64_t* __restrict__ recv_topk_idx,       // compact [N][K] or null
-                                                             float* __restrict__ recv_weights,          // [C] / [N][K] or null
+                                                             u32x4* __restrict__ recv_x,                // [C][vectors]
+                                                             float* __restrict__ recv_weights,          // [C] or null
                                                              int64_t recv_count,
                                                              int64_t out_rows,
-                                                             uint32_t copy_candidates,  // T*K expanded, T compact
+                                                             uint32_t copy_candidates,  // T*K
                                                              uint32_t copy_blocks,
                                                              uint32_t copy_per_xcd,  // ceil(copy_blocks / 8)
                                                              uint32_t pad_blocks,
@@ -88,13 +87,12 @@ __global__ void __launch_bounds__(1024) dispatch_rows_kernel(const u32x4* __rest
                                                              int vectors,
                                                              int chunks,
                                                              int num_topk,
-                                                             int topk_shift,  // log2(K) when K is a power of two, else -1
-                                                             int expand) {
+                                                             int topk_shift) {  // log2(K) when K is a power of two, else -1
     NANOEP_FETCH_ARGS_4(x, weights, recv_x, recv_weights);
     NANOEP_FETCH_ARGS_4(token_slots, copy_blocks, dst_slots, recv_metadata);
     NANOEP_FETCH_ARGS_4(out_rows, recv_count, copy_candidates, copy_per_xcd);
     NANOEP_FETCH_ARGS_4(parts_magic, parts_shift, vectors, chunks);
-    NANOEP_FETCH_ARGS_4(num_topk, topk_shift, expand, chunks_per_block);
+    NANOEP_FETCH_ARGS_4(num_topk, topk_shift, rows_per_block, chunks_per_block);
     // Workgroups are handed to the XCDs round-robin.  Each XCD takes one contiguous range of the
     // copy work followed by one contiguous range of the zero-fill work, so neighbouring work items
     // (which share their source rows) stay behind one L2 and every XCD gets its share of both.
@@ -122,42 +120,28 @@ __global__ void __launch_bounds__(1024) dispatch_rows_kernel(const u32x4* __rest
             return;
         const int vector = chunk * kWave + lane;
         const bool in_row = vector < vectors;
-        uint32_t token = candidate;
-        int k = 0;
-        int64_t out_row;
-        const int32_t* fields = nullptr;
-        if (expand) {
-            token = topk_shift >= 0 ? candidate >> topk_shift : candidate / static_cast<uint32_t>(num_topk);
-            k = static_cast<int>(candidate - token * num_topk);
-        }
+        // candidates are (source token, k) pairs in token order
+        uint32_t token = topk_shift >= 0 ? candidate >> topk_shift : candidate / static_cast<uint32_t>(num_topk);
+        int k = static_cast<int>(candidate - token * num_topk);
         token = __builtin_amdgcn_readfirstlane(token);
         k = __builtin_amdgcn_readfirstlane(k);
         // lanes past the end of a short row re-read vector 0 instead of branching around the load
         const u32x4 data = x[static_cast<int64_t>(token) * vectors + (in_row ? vector : 0)];
-        if (kLookup == kLookupTable && expand) {
+        int64_t out_row;
+        if (kLookup == kLookupTable) {
             out_row = uniform_load(token_slots + static_cast<int64_t>(token) * num_topk + k);
         } else {
             const int64_t row = uniform_load(dst_slots + token);
             if (row < 0 || row >= recv_count)
                 return;
-            fields = recv_metadata + row * (num_topk + 2);
-            out_row = expand ? static_cast<int64_t>(uniform_load(fields + 2 + k)) : row;
+            out_row = static_cast<int64_t>(uniform_load(recv_metadata + row * (num_topk + 2) + 2 + k));
         }
         if (out_row < 0 || out_row >= out_rows)
             return;
         if (in_row)
             store_vec<true>(recv_x + out_row * vectors + vector, data);
-        if (chunk != 0)
-            return;
-        if (expand) {
-            if (lane == 0 && recv_weights != nullptr)
-                recv_weights[out_row] = weights[static_cast<int64_t>(token) * num_topk + k];
-        } else if (lane < num_topk) {
-            if (recv_topk_idx != nullptr)
-                recv_topk_idx[out_row * num_topk + lane] = fields[2 + lane];
-            if (recv_weights != nullptr)
-                recv_weights[out_row * num_topk + lane] = weights[static_cast<int64_t>(token) * num_topk + lane];
-        }
+        if (chunk == 0 && lane == 0 && recv_weights != nullptr)
+            recv_weights[out_row] = weights[static_cast<int64_t>(token) * num_topk + k];
     } else {
         zero_fill_gap_rows(block, pad_per_expert, pad_groups_per_expert, chunks_per_block, rows_per_block, expert_counts,
                            expert_offsets, recv_x, recv_weights, out_rows, vectors);
@@ -520,13 +504,13 @@ int nanoep_dispatch(const void* x, const float* weights, const int32_t* recv_met
 #define NANOEP_LAUNCH_ROWS(LOOKUP, ZERO_FILL)                                                                         \
     dispatch_rows_kernel<LOOKUP, ZERO_FILL><<<grid, block, 0, stream>>>(                                             \
         static_cast<const u32x4*>(x), weights, recv_metadata, dst_slots, token_slots, expert_counts, expert_offsets, \
-        static_cast<u32x4*>(recv_x), recv_topk_idx, recv_weights, recv_count, out_rows,                              \
+        static_cast<u32x4*>(recv_x), recv_weights, recv_count, out_rows,                                             \
         static_cast<uint32_t>(copy_candidates), static_cast<uint32_t>(copy_blocks), copy_per_xcd,                    \
         static_cast<uint32_t>(pad_blocks), pad_per_xcd, blocking.parts, parts_divisor.magic, parts_divisor.shift,    \
         blocking.chunks_per_block, blocking.rows_per_block, static_cast<uint32_t>(pad_per_expert),                   \
         static_cast<uint32_t>(pad_groups_per_expert > 0 ? pad_groups_per_expert : 1), vectors, chunks, num_topk,     \
-        topk_shift, expand ? 1 : 0)
-        const bool table = token_slots != nullptr && expand;
+        topk_shift)
+        const bool table = token_slots != nullptr;
         if (table && pad_blocks > 0)
             NANOEP_LAUNCH_ROWS(kLookupTable, true);
         else if (table)

@@ -35,6 +35,10 @@ constexpr int kMaxWindowTokens = 1024;
 //    1024-token windows): batches of more than 256 tokens take smaller windows (down to 64 tokens)
 //    to get there.
 int layout_window_tokens(int64_t tokens_total, int hidden) {
+    // NANOEP_WINDOW_TOKENS forces a window: any multiple of 32 up to 256 (one layout workgroup), or 512 / 1024
+    const int forced = env_int("NANOEP_WINDOW_TOKENS", 0);
+    if (forced >= 32 && forced % 32 == 0 && (forced <= 256 || forced == 512 || forced == 1024) && tokens_total > 256)
+        return forced;
     int window = 256;
     if (hidden > 0)
         for (window = kMaxWindowTokens;
@@ -55,7 +59,7 @@ int layout_tokens_per_block(int64_t tokens_total, int64_t local_experts, int hid
     if (static_cast<size_t>(local_experts + 1) * 16 > kLayoutLdsBudget)  // four int32 arrays of the assignment kernel
         return 0;
     const int window = layout_window_tokens(tokens_total, hidden);
-    for (int tokens = window < kMaxBlockTokens ? window : kMaxBlockTokens; tokens >= 32; tokens /= 2) {
+    for (int tokens = window < kMaxBlockTokens ? window : kMaxBlockTokens; tokens >= 32; tokens = tokens / 2 / 32 * 32) {
         const size_t words = static_cast<size_t>(tokens / 32);
         if (static_cast<size_t>(local_experts + 1) * (words * 6 + 4) <= kLayoutLdsBudget)
             return tokens;
@@ -648,9 +652,12 @@ __device__ __forceinline__ void layout_assign_block(const int32_t* block_counts,
     int64_t* order = nullptr;
     if (slot_order != nullptr) {
         order = slot_order + (assigned_before - window_earlier);
+        // every block before the last one is full; the last one holds what is left of the batch
         const int64_t block_entries = static_cast<int64_t>(tokens_per_block) * num_topk;
+        const int64_t tokens_left = num_tokens - static_cast<int64_t>(block) * tokens_per_block;
+        const int64_t own_entries = (tokens_left < tokens_per_block ? tokens_left : tokens_per_block) * num_topk;
         int64_t* tail = slot_order + assigned + (block * block_entries - assigned_before);
-        const int holes = static_cast<int>(block_entries) - own_total;
+        const int holes = static_cast<int>(own_entries) - own_total;
         for (int i = tid; i < holes; i += threads)
             tail[i] = -1;
         // The buffer's size does not depend on the block size: (T rounded up to 256) * K entries, then
@@ -658,7 +665,7 @@ __device__ __forceinline__ void layout_assign_block(const int32_t* block_counts,
         // the blocks' own entries, so that everything from entry A to the count word reads -1.
         const int64_t capacity_entries = (num_tokens + kMaxBlockTokens - 1) / kMaxBlockTokens * kMaxBlockTokens * num_topk;
         if (block == num_blocks - 1)
-            for (int64_t i = num_blocks * block_entries + tid; i < capacity_entries; i += threads)
+            for (int64_t i = num_tokens * num_topk + tid; i < capacity_entries; i += threads)
                 slot_order[i] = -1;
         if (block == 0 && tid == 0)
             slot_order[capacity_entries] = assigned;
@@ -937,6 +944,12 @@ int nanoep_wait_counts(int64_t* host_counts, void* stream_handle, double timeout
         if (received >= 0)
             break;
         if ((++spins & 0x3ff) == 0) {
+            // the clock first: a caller with no patience left is answered without touching the stream
+            timespec now{};
+            clock_gettime(CLOCK_MONOTONIC, &now);
+            const double elapsed = (now.tv_sec - start.tv_sec) + 1e-9 * (now.tv_nsec - start.tv_nsec);
+            if (elapsed > timeout_seconds)
+                return NANOEP_ERR_TIMEOUT;
             // A finished (or failed) stream with no published count means the layout never ran.
             const hipError_t state = hipStreamQuery(stream);
             if (state != hipErrorNotReady) {
@@ -948,11 +961,6 @@ int nanoep_wait_counts(int64_t* host_counts, void* stream_handle, double timeout
                     break;
                 return NANOEP_ERR_TIMEOUT;
             }
-            timespec now{};
-            clock_gettime(CLOCK_MONOTONIC, &now);
-            const double elapsed = (now.tv_sec - start.tv_sec) + 1e-9 * (now.tv_nsec - start.tv_nsec);
-            if (elapsed > timeout_seconds)
-                return NANOEP_ERR_TIMEOUT;
         }
     }
     for (int i = 0; i < NANOEP_HOST_COUNT_WORDS; ++i)

@@ -16,7 +16,9 @@
 #include <torch/extension.h>
 
 #include <array>
+#include <atomic>
 #include <cstdlib>
+#include <deque>
 #include <limits>
 #include <memory>
 #include <mutex>
@@ -40,9 +42,9 @@ namespace {
 
 constexpr int64_t kHiddenAlignment = 256;  // the reference's H % 256 == 0 contract
 constexpr double kCountTimeoutSeconds = 60.0;
-// A replay with only the reference's seven handle tensors re-runs the layout for the slot-order
-// list once the payload is at least this large (below, the token-order walk is as fast).
-constexpr int64_t kRebuildOrderMinBytes = int64_t{16} << 20;
+// Fresh expanded dispatches whose private handle tensors the runtime keeps for callers that hand
+// back only the reference's seven.
+constexpr size_t kRememberedHandles = 4;
 
 int env_switch(const char* name) {  // -1: not set
     const char* text = std::getenv(name);
@@ -83,6 +85,11 @@ int resolve_cu_budget(int num_sms, c10::DeviceIndex device) {
 // kernels publish N / C into, and (only if somebody asks for it) a window-sized byte tensor.
 // It keeps the reference's PeerRuntime method set (csrc/bindings.cpp:59-83) so setup code written
 // for the reference runs; there are no peers, so handles are opaque tags and barriers are no-ops.
+//
+// dispatch and combine run without the interpreter lock, so everything here that several Python
+// threads can reach at once is guarded: the mailbox by `counts_mutex_` (held by a fresh dispatch
+// from the enqueue of its layout until it has read the counts), the remembered handle tensors by
+// `private_mutex_`, the state flags by being atomic.
 class PeerRuntime {
    public:
     PeerRuntime(int rank, int world_size, int64_t num_bytes) : num_bytes_(num_bytes) {
@@ -91,11 +98,10 @@ class PeerRuntime {
         TORCH_CHECK(num_bytes >= 0, "window size must be non-negative");
         check_hip(hipGetDevice(&device_), "hipGetDevice");
         void* mailbox = nullptr;
-        // two mailboxes: the one fresh dispatches wait on, and one for layouts nobody waits for
-        check_hip(hipHostMalloc(&mailbox, 2 * NANOEP_HOST_COUNT_WORDS * sizeof(int64_t), hipHostMallocMapped | hipHostMallocCoherent),
+        check_hip(hipHostMalloc(&mailbox, NANOEP_HOST_COUNT_WORDS * sizeof(int64_t), hipHostMallocMapped | hipHostMallocCoherent),
                   "hipHostMalloc");
         host_counts_ = static_cast<int64_t*>(mailbox);
-        for (int i = 0; i < 2 * NANOEP_HOST_COUNT_WORDS; ++i)
+        for (int i = 0; i < NANOEP_HOST_COUNT_WORDS; ++i)
             host_counts_[i] = -1;
     }
 
@@ -110,59 +116,140 @@ class PeerRuntime {
     int rank() const { return 0; }
     int world_size() const { return 1; }
     int device() const { return device_; }
-    int64_t* host_counts() const {
-        TORCH_CHECK(!closed_, "PeerRuntime is closed");
-        return host_counts_;
-    }
-    // Mailbox of layouts that are re-run on the device for a cached handle: their counts are known
-    // already, and a word they store late must not be taken for the answer to a fresh dispatch.
-    int64_t* unread_counts() const { return host_counts() + NANOEP_HOST_COUNT_WORDS; }
 
-    // The private handle tensors (slot table, slot-order list) of the latest fresh expanded dispatch.
-    // A caller that keeps only the reference's seven handle tensors gets them back on a replay of
-    // that same handle: the entry is recognised by the identity of the handle's routing snapshot
-    // (the tensor object, its data pointer and version) and of its recv_metadata storage.  The two
-    // tensors are views of the allocations that back the seven public ones.
+    // Every operation starts here (the reference's reserve_barrier_epochs, csrc/peer.cu:171-175):
+    // a closed runtime, and one whose last fresh dispatch never got its counts, serve nothing.
+    void require_usable() const {
+        TORCH_CHECK(!closed_.load(), "PeerRuntime is closed");
+        TORCH_CHECK(!counts_failed_.load(), "A fresh dispatch on this runtime failed while waiting for its counts; the runtime is unusable");
+    }
+
+    // One fresh dispatch's use of the mailbox, from before its layout is enqueued until the host has
+    // read N and C (the reference's prepare_dispatch_counts / wait_dispatch_counts /
+    // fail_dispatch_counts, csrc/peer.cu:187-232).  Fresh dispatches of other threads wait their
+    // turn at the constructor.  A turn that ends without `wait` having delivered the counts (a
+    // timeout, a HIP error, an exception in between) leaves the runtime failed for good: a word the
+    // device stores late must never answer a later call.
+    class CountsTurn {
+       public:
+        explicit CountsTurn(PeerRuntime& runtime) : runtime_(runtime), lock_(runtime.counts_mutex_) {
+            runtime_.require_usable();
+            TORCH_CHECK(!runtime_.counts_pending_.load(), "A fresh dispatch is waiting for counts or has failed");
+            runtime_.counts_pending_.store(true);
+        }
+        CountsTurn(const CountsTurn&) = delete;
+        CountsTurn& operator=(const CountsTurn&) = delete;
+        ~CountsTurn() {
+            if (!settled_)
+                runtime_.counts_failed_.store(true);
+            runtime_.counts_pending_.store(false);
+        }
+
+        int64_t* mailbox() const { return runtime_.host_counts_; }
+
+        // Nothing was enqueued that could still write the mailbox: the turn ends without a verdict.
+        void abandon() { settled_ = true; }
+
+        // Spins until the layout enqueued on `stream` has published {N, C, A, status}.  Returns
+        // NANOEP_OK or NANOEP_ERR_ROUTING (the words are complete either way); anything else throws
+        // and latches the failure.
+        int wait(hipStream_t stream, double timeout_seconds, int64_t (&counts)[NANOEP_HOST_COUNT_WORDS]) {
+            const int status = nanoep_wait_counts(mailbox(), stream, timeout_seconds, counts);
+            if (status == NANOEP_OK || status == NANOEP_ERR_ROUTING) {
+                settled_ = true;
+                return status;
+            }
+            check_status(status, "wait_counts");
+            return status;
+        }
+
+       private:
+        PeerRuntime& runtime_;
+        std::unique_lock<std::mutex> lock_;
+        bool settled_ = false;
+    };
+
+    bool counts_failed() const { return counts_failed_.load(); }
+
+    // What a fresh dispatch whose counts never arrive leaves behind, without making a GPU misbehave:
+    // a turn at the mailbox that ends with no verdict.  For tests of the failure latch.
+    void lose_counts_for_test() { CountsTurn lost(*this); }
+
+    // Whether fresh dispatches should allocate their outputs after the counts are known: set when a
+    // call that allocated at the upper bound turned out to hold over 1.25 times what it used (many
+    // masked choices), cleared when an exact call shows that the bound would have been close enough.
+    bool prefers_exact_outputs() const { return prefers_exact_outputs_.load(); }
+    void note_output_fill(bool bound_was_close) { prefers_exact_outputs_.store(!bound_was_close); }
+
+    // The private handle tensors (slot table, slot-order list) of the latest few fresh expanded
+    // dispatches.  A caller that keeps only the reference's seven handle tensors gets them back on
+    // a replay of one of those handles: an entry is recognised by the identity of the handle's
+    // routing snapshot (the tensor object, its data pointer and version) and of its recv_metadata
+    // storage.  The two tensors are views of the allocations that back the seven public ones.
+    // Handles this runtime did not make, or made too long ago, are never matched: their replays
+    // follow the handle's own recv_metadata and dst_slots in token order.
     void remember_private(const std::vector<torch::Tensor>& metadata, int64_t alignment) {
-        torch::Tensor old_table, old_order;  // released after the lock: a tensor's release may want the interpreter lock
-        std::lock_guard<std::mutex> lock(private_mutex_);
-        drop_private(old_table, old_order);
         if (metadata.size() < 9 || !metadata[7].defined() || !metadata[8].defined())
             return;
-        remembered_snapshot_.emplace(metadata[5].getIntrusivePtr());
-        remembered_version_ = tensor_version(metadata[5]);
-        remembered_snapshot_data_ = metadata[5].data_ptr();
-        remembered_metadata_data_ = metadata[0].data_ptr();
-        remembered_rows_ = metadata[0].size(0);
-        remembered_alignment_ = alignment;
-        remembered_table_ = metadata[7];
-        remembered_order_ = metadata[8];
+        RememberedHandle entry;
+        entry.snapshot.emplace(metadata[5].getIntrusivePtr());
+        entry.version = tensor_version(metadata[5]);
+        entry.snapshot_data = metadata[5].data_ptr();
+        entry.metadata_data = metadata[0].data_ptr();
+        entry.rows = metadata[0].size(0);
+        entry.alignment = alignment;
+        entry.table = metadata[7];
+        entry.order = metadata[8];
+        std::vector<RememberedHandle> retired;  // released after the lock: a tensor's release may want the interpreter lock
+        {
+            std::lock_guard<std::mutex> lock(private_mutex_);
+            // handles whose routing snapshot is gone can never come back
+            for (auto it = remembered_.begin(); it != remembered_.end();) {
+                if (it->snapshot->expired()) {
+                    retired.push_back(std::move(*it));
+                    it = remembered_.erase(it);
+                } else {
+                    ++it;
+                }
+            }
+            remembered_.push_front(std::move(entry));
+            while (remembered_.size() > kRememberedHandles) {
+                retired.push_back(std::move(remembered_.back()));
+                remembered_.pop_back();
+            }
+        }
     }
 
-    // Appends the remembered private tensors to a seven-tensor handle when it is the remembered one
+    // Appends the remembered private tensors to a seven-tensor handle when it is a remembered one
     // (alignment < 0: the caller does not know the handle's alignment, the identity decides).
     bool recall_private(std::vector<torch::Tensor>& metadata, int64_t alignment) const {
         std::lock_guard<std::mutex> lock(private_mutex_);
-        if (closed_ || !remembered_snapshot_.has_value() || metadata.size() != 7)
+        if (closed_.load() || metadata.size() != 7)
             return false;
-        const auto alive = remembered_snapshot_->lock();
-        if (!alive || alive.get() != metadata[5].unsafeGetTensorImpl() || metadata[5].data_ptr() != remembered_snapshot_data_ ||
-            tensor_version(metadata[5]) != remembered_version_ || metadata[0].data_ptr() != remembered_metadata_data_ ||
-            metadata[0].size(0) != remembered_rows_ || (alignment >= 0 && alignment != remembered_alignment_))
-            return false;
-        metadata.push_back(remembered_table_);
-        metadata.push_back(remembered_order_);
-        ++private_recalls_;
-        return true;
+        for (const auto& entry : remembered_) {
+            const auto alive = entry.snapshot->lock();
+            if (!alive || alive.get() != metadata[5].unsafeGetTensorImpl() || metadata[5].data_ptr() != entry.snapshot_data ||
+                tensor_version(metadata[5]) != entry.version || metadata[0].data_ptr() != entry.metadata_data ||
+                metadata[0].size(0) != entry.rows || (alignment >= 0 && alignment != entry.alignment))
+                continue;
+            metadata.push_back(entry.table);
+            metadata.push_back(entry.order);
+            ++private_recalls_;
+            return true;
+        }
+        return false;
     }
 
     // number of seven-tensor handles that got their private tensors back (for tests)
-    int64_t private_recalls() const { return private_recalls_; }
+    int64_t private_recalls() const {
+        std::lock_guard<std::mutex> lock(private_mutex_);
+        return private_recalls_;
+    }
 
     void forget_private() {
-        torch::Tensor old_table, old_order;
+        std::deque<RememberedHandle> retired;
         std::lock_guard<std::mutex> lock(private_mutex_);
-        drop_private(old_table, old_order);
+        retired.swap(remembered_);
     }
 
     py::bytes export_local_handle() const {
@@ -172,17 +259,17 @@ class PeerRuntime {
     }
 
     void import_peer_handles(const std::vector<py::bytes>& handles) {
-        TORCH_CHECK(!closed_, "PeerRuntime is closed");
+        TORCH_CHECK(!closed_.load(), "PeerRuntime is closed");
         if (handles.size() != 1)
             throw py::value_error("expected exactly one handle (world_size == 1)");
         for (const auto& handle : handles)
             if (py::len(handle) != 64)
                 throw py::value_error("Each IPC handle must contain exactly 64 bytes");
-        mappings_open_ = true;
+        mappings_closed_ = false;
     }
 
     torch::Tensor local_window() {
-        TORCH_CHECK(!closed_, "PeerRuntime is closed");
+        TORCH_CHECK(!closed_.load(), "PeerRuntime is closed");
         if (!window_.defined()) {
             DeviceGuard guard(static_cast<c10::DeviceIndex>(device_));
             window_ = torch::zeros({num_bytes_}, torch::dtype(torch::kUInt8).device(torch::kCUDA, device_));
@@ -197,29 +284,44 @@ class PeerRuntime {
         return addresses.to(window.device());
     }
 
-    // No peers: an epoch barrier has nobody to meet.
-    void barrier(int64_t) const { TORCH_CHECK(!closed_, "PeerRuntime is closed"); }
-    void barrier_at(int64_t, int64_t) const { TORCH_CHECK(!closed_, "PeerRuntime is closed"); }
+    // No peers: an epoch barrier has nobody to meet.  Epochs still have to increase, as in the
+    // reference (csrc/peer.cu:234-237).
+    void barrier(int64_t) {
+        require_usable();
+        ++last_barrier_epoch_;
+    }
+    void barrier_at(int64_t, int64_t epoch) {
+        require_usable();
+        TORCH_CHECK(epoch > last_barrier_epoch_, "Barrier epoch must strictly increase");
+        last_barrier_epoch_ = epoch;
+    }
 
-    void close_peer_mappings() { mappings_open_ = false; }
+    void close_peer_mappings() {
+        if (closed_.load() || mappings_closed_)
+            return;
+        TORCH_CHECK(!counts_pending_.load(), "Cannot close while a fresh dispatch is waiting for counts");
+        mappings_closed_ = true;
+    }
 
     void close() {
-        if (closed_)
+        if (closed_.load())
             return;
-        TORCH_CHECK(!mappings_open_, "close_peer_mappings must run before close");
+        TORCH_CHECK(mappings_closed_, "Call close_peer_mappings() before close()");
         window_ = torch::Tensor();
         forget_private();
-        closed_ = true;
+        closed_.store(true);
     }
 
    private:
-    void drop_private(torch::Tensor& old_table, torch::Tensor& old_order) {
-        remembered_snapshot_.reset();
-        old_table = std::move(remembered_table_);
-        old_order = std::move(remembered_order_);
-        remembered_table_ = torch::Tensor();
-        remembered_order_ = torch::Tensor();
-    }
+    struct RememberedHandle {
+        std::optional<c10::weak_intrusive_ptr<c10::TensorImpl>> snapshot;
+        uint32_t version = 0;
+        const void* snapshot_data = nullptr;
+        const void* metadata_data = nullptr;
+        int64_t rows = 0;
+        int64_t alignment = 0;
+        torch::Tensor table, order;
+    };
 
     // in-place edits through torch bump the version; inference tensors have none
     static uint32_t tensor_version(const torch::Tensor& tensor) {
@@ -230,88 +332,118 @@ class PeerRuntime {
     int64_t num_bytes_ = 0;
     int64_t* host_counts_ = nullptr;
     torch::Tensor window_;
-    std::optional<c10::weak_intrusive_ptr<c10::TensorImpl>> remembered_snapshot_;
-    uint32_t remembered_version_ = 0;
-    const void* remembered_snapshot_data_ = nullptr;
-    const void* remembered_metadata_data_ = nullptr;
-    int64_t remembered_rows_ = 0;
-    int64_t remembered_alignment_ = 0;
-    torch::Tensor remembered_table_, remembered_order_;
+    std::mutex counts_mutex_;
+    std::atomic<bool> counts_pending_{false};
+    std::atomic<bool> counts_failed_{false};
+    std::atomic<bool> prefers_exact_outputs_{false};
+    std::deque<RememberedHandle> remembered_;  // newest first
     mutable int64_t private_recalls_ = 0;
-    mutable std::mutex private_mutex_;  // dispatch and combine run without the interpreter lock
-    bool mappings_open_ = false;
-    bool closed_ = false;
+    mutable std::mutex private_mutex_;
+    int64_t last_barrier_epoch_ = 0;
+    bool mappings_closed_ = false;
+    std::atomic<bool> closed_{false};
 };
 
-// Recorded on the communication stream; waiting orders the consumer stream after it and tells
-// the caching allocator that the protected tensors are used there
-// (csrc/include/nano_ep/event.hpp:12-28 in the reference).
-struct CompletionEvent {
-    std::shared_ptr<c10::Event> event;
-    std::vector<torch::Tensor> tensors;
-
-    CompletionEvent(const Stream& stream, std::vector<torch::Tensor> outputs)
-        : event(std::make_shared<c10::Event>(c10::DeviceType::CUDA)), tensors(std::move(outputs)) {
-        event->record(stream.unwrap());
+// What a caller gets back from an asynchronous call: a marker on the communication stream behind
+// the call's kernels, and the tensors those kernels write.  Waiting puts the consumer's stream
+// behind the marker and tells the caching allocator that the tensors are in use there, so that
+// freeing them on the consumer's side cannot hand their memory out while that stream still reads
+// it (the role of csrc/include/nano_ep/event.hpp:12-28 in the reference).
+class CompletionEvent {
+   public:
+    static std::shared_ptr<CompletionEvent> record_behind(const Stream& producer, std::vector<torch::Tensor> written) {
+        auto marker = std::make_shared<CompletionEvent>();
+        marker->written_ = std::move(written);
+        marker->done_.record(producer.unwrap());
+        return marker;
     }
 
-    void wait(const Stream& stream) const {
-        stream.unwrap().wait(*event);
-        for (const auto& tensor : tensors)
+    void order_after(const Stream& consumer) const {
+        consumer.unwrap().wait(done_);
+        for (const auto& tensor : written_)
             if (tensor.defined() && tensor.numel() > 0)
-                tensor.record_stream(stream.unwrap());
+                tensor.record_stream(consumer.unwrap());
     }
 
-    void current_stream_wait() const { wait(c10::hip::getCurrentHIPStreamMasqueradingAsCUDA()); }
+    void current_stream_wait() const { order_after(c10::hip::getCurrentHIPStreamMasqueradingAsCUDA()); }
+
+    CompletionEvent() : done_(c10::DeviceType::CUDA) {}
+
+   private:
+    c10::Event done_;
+    std::vector<torch::Tensor> written_;
 };
 
 namespace {
 
-void check_payload_inputs(const torch::Tensor& x,
-                          const torch::Tensor& indices,
-                          const c10::optional<torch::Tensor>& weights,
-                          int device,
-                          int64_t num_experts,
-                          int64_t max_tokens) {
-    TORCH_CHECK(x.is_cuda() && x.get_device() == device && x.dim() == 2 && x.is_contiguous(),
+// What a tensor argument has to look like: where it lives, its element type and its extents
+// (-1 leaves an extent open).  Every tensor check of dispatch, combine and the cached handle is one
+// `require` against such a description; the message is the caller-visible part.
+struct TensorSpec {
+    c10::Device device;
+    at::ScalarType dtype;
+    std::vector<int64_t> extents;
+
+    bool describes(const torch::Tensor& tensor) const {
+        if (!tensor.defined() || tensor.device() != device || tensor.scalar_type() != dtype || !tensor.is_contiguous() ||
+            tensor.dim() != static_cast<int64_t>(extents.size()))
+            return false;
+        for (size_t axis = 0; axis < extents.size(); ++axis)
+            if (extents[axis] >= 0 && tensor.size(static_cast<int64_t>(axis)) != extents[axis])
+                return false;
+        return true;
+    }
+};
+
+template <class... Message>
+void require(const torch::Tensor& tensor, const TensorSpec& spec, const Message&... message) {
+    TORCH_CHECK(spec.describes(tensor), message...);
+}
+
+bool vector_aligned(const torch::Tensor& tensor) {
+    return tensor.numel() == 0 || reinterpret_cast<uintptr_t>(tensor.data_ptr()) % 16 == 0;
+}
+
+// The payload, its routing ids and its weights, as the reference's host pipeline insists on them
+// (csrc/pipeline.cu:26-60): same limits, same wording of what is wrong.
+void require_dispatch_inputs(const torch::Tensor& x, const torch::Tensor& routing, const c10::optional<torch::Tensor>& weights,
+                             int device, int64_t num_experts, int64_t max_tokens) {
+    const c10::Device here(c10::DeviceType::CUDA, static_cast<c10::DeviceIndex>(device));
+    TORCH_CHECK(x.defined() && x.is_cuda() && x.device() == here && x.dim() == 2 && x.is_contiguous(),
                 "x must be contiguous CUDA [T,H] on the runtime device");
-    TORCH_CHECK(x.scalar_type() == torch::kBFloat16, "dispatch x must be bfloat16");
-    TORCH_CHECK(x.size(1) > 0 && x.size(1) % kHiddenAlignment == 0, "dispatch hidden must be a positive multiple of 256");
-    TORCH_CHECK(x.numel() == 0 || reinterpret_cast<uintptr_t>(x.data_ptr()) % 16 == 0,
-                "dispatch x data pointer must be 16-byte aligned");
-    TORCH_CHECK(indices.device() == x.device() && indices.scalar_type() == torch::kInt64 && indices.dim() == 2 &&
-                    indices.size(0) == x.size(0) && indices.is_contiguous(),
-                "indices must be contiguous CUDA int64 [T,K] on the x device");
-    TORCH_CHECK(indices.size(1) > 0 && indices.size(1) <= 32, "num_topk must be in [1, 32]");
+    require(x, {here, torch::kBFloat16, {-1, -1}}, "dispatch x must be bfloat16");
+    const int64_t tokens = x.size(0), hidden = x.size(1);
+    TORCH_CHECK(hidden > 0 && hidden % kHiddenAlignment == 0, "dispatch hidden must be a positive multiple of 256");
+    TORCH_CHECK(vector_aligned(x), "dispatch x data pointer must be 16-byte aligned");
+    require(routing, {here, torch::kInt64, {tokens, -1}}, "indices must be contiguous CUDA int64 [T,K] on the x device");
+    const int64_t topk = routing.size(1);
+    TORCH_CHECK(topk >= 1 && topk <= 32, "num_topk must be in [1, 32]");
     TORCH_CHECK(num_experts > 0, "num_experts must be positive and divisible by world_size");
     TORCH_CHECK(max_tokens <= std::numeric_limits<int32_t>::max(), "max_tokens exceeds int32 metadata range");
-    TORCH_CHECK(max_tokens > 0 && x.size(0) <= max_tokens, "source token count exceeds max_tokens");
-    if (weights.has_value()) {
-        TORCH_CHECK(weights->device() == x.device() && weights->scalar_type() == torch::kFloat32 &&
-                        weights->sizes() == indices.sizes() && weights->is_contiguous(),
-                    "weights must be contiguous CUDA float32 [T,K] on the x device");
-    }
+    TORCH_CHECK(max_tokens > 0 && tokens <= max_tokens, "source token count exceeds max_tokens");
+    if (weights.has_value())
+        require(*weights, {here, torch::kFloat32, {tokens, topk}}, "weights must be contiguous CUDA float32 [T,K] on the x device");
 }
 
-void check_cached_tensor(const torch::Tensor& tensor,
-                         const torch::Tensor& reference,
-                         at::IntArrayRef shape,
-                         const char* name,
-                         at::ScalarType dtype = torch::kInt64) {
-    TORCH_CHECK(tensor.device() == reference.device() && tensor.scalar_type() == dtype && tensor.sizes() == shape && tensor.is_contiguous(),
-                "cached ", name, " has invalid CUDA storage or shape");
-}
-
-void check_handle_metadata(const std::vector<torch::Tensor>& metadata, const torch::Tensor& x, int64_t source_tokens, int64_t topk,
-                           int64_t local_experts) {
-    const int64_t recv_count = metadata[0].dim() == 2 ? metadata[0].size(0) : -1;
-    check_cached_tensor(metadata[0], x, {recv_count, topk + 2}, "recv_metadata", torch::kInt32);
-    check_cached_tensor(metadata[1], x, {local_experts}, "expert_counts");
-    check_cached_tensor(metadata[2], x, {local_experts + 1}, "expert_offsets");
-    check_cached_tensor(metadata[3], x, {source_tokens, 1}, "dst_slots");
-    check_cached_tensor(metadata[4], x, {1}, "send_counts");
-    check_cached_tensor(metadata[5], x, {source_tokens, topk}, "source_topk_snapshot");
-    check_cached_tensor(metadata[6], x, {1}, "recv_rank_prefix");
+// The seven handle tensors of a cached call against the geometry they must describe.
+void require_handle_tensors(const std::vector<torch::Tensor>& metadata, const c10::Device& here, int64_t source_tokens, int64_t topk,
+                            int64_t local_experts) {
+    struct Field {
+        const char* name;
+        at::ScalarType dtype;
+        std::vector<int64_t> extents;
+    };
+    const Field fields[7] = {
+        {"recv_metadata", torch::kInt32, {-1, topk + 2}},
+        {"expert_counts", torch::kInt64, {local_experts}},
+        {"expert_offsets", torch::kInt64, {local_experts + 1}},
+        {"dst_slots", torch::kInt64, {source_tokens, 1}},
+        {"send_counts", torch::kInt64, {1}},
+        {"source_topk_snapshot", torch::kInt64, {source_tokens, topk}},
+        {"recv_rank_prefix", torch::kInt64, {1}},
+    };
+    for (int i = 0; i < 7; ++i)
+        require(metadata[i], {here, fields[i].dtype, fields[i].extents}, "cached ", fields[i].name, " has invalid CUDA storage or shape");
 }
 
 // The optional eighth handle tensor: int32 [T,K] slot table written by the layout kernels.
@@ -399,8 +531,8 @@ DispatchResult dispatch(PeerRuntime& runtime,
     TORCH_CHECK(!cached || (cached_metadata.size() >= 7 && cached_metadata.size() <= 9),
                 "cached metadata must contain the seven prepared tensors from dispatch (plus the optional slot table and slot-order list)");
     const auto& routing = cached ? cached_metadata[5] : indices;
-    int64_t* host_counts = runtime.host_counts();
-    check_payload_inputs(x, routing, weights, runtime.device(), num_experts, max_tokens);
+    runtime.require_usable();
+    require_dispatch_inputs(x, routing, weights, runtime.device(), num_experts, max_tokens);
     TORCH_CHECK(alignment > 0, "alignment must be positive");
     const auto device = static_cast<c10::DeviceIndex>(runtime.device());
     DeviceGuard device_guard(device);
@@ -459,7 +591,7 @@ DispatchResult dispatch(PeerRuntime& runtime,
     int64_t recv_count = 0;
     int64_t expanded_capacity = 0;
     if (cached) {
-        check_handle_metadata(cached_metadata, x, tokens, topk, local_experts);
+        require_handle_tensors(cached_metadata, x.device(), tokens, topk, local_experts);
         metadata = cached_metadata;
         recv_count = cached_metadata[0].size(0);
         expanded_capacity = cached_expanded_capacity;
@@ -468,40 +600,15 @@ DispatchResult dispatch(PeerRuntime& runtime,
                     "expanded capacity exceeds int32 metadata range");
         allocate_outputs(expand ? expanded_capacity : recv_count, recv_count);
         // A handle that went through the reference's Python class carries the seven tensors of the
-        // reference only.  The layout is a pure function of the routing snapshot, so the private
-        // slot-order list is made again on the device (two small launches, no host wait) and the
-        // payload takes the fast walk: 4096 x 7168 top-8 with cold sources 144 -> 99 us.
-        // ... unless the handle is the one of the latest fresh dispatch, whose private tensors
-        // the runtime still has (NANOEP_RECALL_ORDER=0 switches that off).
+        // reference only.  If it is one of this runtime's latest fresh dispatches, the runtime still
+        // has its private tensors and the payload takes the slot-order walk
+        // (NANOEP_RECALL_ORDER=0 switches that off).  Any other seven-tensor handle is followed as it
+        // is written, in token order through its own dst_slots and recv_metadata: whatever row and
+        // slot order it describes is the order the rows land in.
         if (expand && recv_count > 0 && env_switch("NANOEP_RECALL_ORDER") != 0)
             runtime.recall_private(metadata, alignment);
-        const int rebuild_switch = env_switch("NANOEP_REBUILD_ORDER");
-        const bool rebuild = expand && recv_count > 0 && metadata.size() == 7 && tokens * topk < (int64_t{1} << 31) &&
-                             (rebuild_switch == 1 || (rebuild_switch != 0 && tokens * hidden * 2 >= kRebuildOrderMinBytes));
-        if (rebuild) {
-            const int64_t order_entries = nanoep_slot_order_entries(tokens, static_cast<int>(topk), local_experts);
-            const size_t workspace_bytes = nanoep_layout_workspace_bytes(tokens, static_cast<int>(topk), local_experts);
-            TORCH_CHECK(order_entries > 0 && workspace_bytes > 0, "unsupported routing geometry for the layout kernels");
-            // scratch of this call (stream-ordered: the allocator hands it out again only to later work of this stream)
-            const int64_t at_offsets = local_experts, at_send = 2 * local_experts + 1, at_prefix = at_send + 1, at_dst = at_prefix + 1;
-            const int64_t at_snapshot = at_dst + tokens, at_order = at_snapshot + tokens * topk, at_table = tokens * (topk + 2);
-            auto scratch64 = torch::empty({at_order + order_entries}, routing.options());
-            auto scratch32 = torch::empty({at_table + tokens * topk}, routing.options().dtype(torch::kInt32));
-            auto workspace = torch::empty({static_cast<int64_t>(workspace_bytes)}, routing.options().dtype(torch::kUInt8));
-            int64_t* base64 = scratch64.data_ptr<int64_t>();
-            int32_t* base32 = scratch32.data_ptr<int32_t>();
-            check_status(nanoep_layout(routing.data_ptr<int64_t>(), tokens, static_cast<int>(topk), local_experts, alignment, 1,
-                                       static_cast<int>(hidden), base32, base64, base64 + at_offsets, base64 + at_dst, base64 + at_send,
-                                       base64 + at_snapshot, base64 + at_prefix, base32 + at_table, base64 + at_order,
-                                       workspace.data_ptr(), workspace_bytes, runtime.unread_counts(), comm.stream()),
-                         "layout");
-            auto handle = metadata;
-            handle.push_back(scratch32.narrow(0, at_table, tokens * topk).view({tokens, topk}));
-            handle.push_back(scratch64.narrow(0, at_order, order_entries));
-            launch_permute(handle, recv_count, expanded_capacity, /*count_on_device=*/true);
-        } else if (recv_count > 0) {
+        if (recv_count > 0)
             launch_permute(metadata, recv_count, expanded_capacity);
-        }
     } else {
         hipStreamCaptureStatus capture = hipStreamCaptureStatusNone;
         check_hip(hipStreamIsCapturing(comm.stream(), &capture), "hipStreamIsCapturing");
@@ -535,12 +642,18 @@ DispatchResult dispatch(PeerRuntime& runtime,
         const int64_t at_snapshot = at_dst + tokens, at_order = at_snapshot + tokens * topk, at_table = tokens * (topk + 2);
         int64_t* base64 = arena64.data_ptr<int64_t>();
         int32_t* base32 = arena32.data_ptr<int32_t>();
-        check_status(nanoep_layout(routing.data_ptr<int64_t>(), tokens, static_cast<int>(topk), local_experts, alignment, expand ? 1 : 0,
-                                   static_cast<int>(hidden), base32, base64, base64 + at_offsets, base64 + at_dst, base64 + at_send, base64 + at_snapshot,
-                                   base64 + at_prefix, expand ? base32 + at_table : nullptr,
-                                   order_entries > 0 ? base64 + at_order : nullptr, workspace.data_ptr(), workspace_bytes,
-                                   host_counts, comm.stream()),
-                     "layout");
+
+        // From here until the counts have been read this call owns the runtime's mailbox; a fresh
+        // dispatch of another thread on the same runtime waits here for its turn.
+        PeerRuntime::CountsTurn turn(runtime);
+        const int layout_status =
+            nanoep_layout(routing.data_ptr<int64_t>(), tokens, static_cast<int>(topk), local_experts, alignment, expand ? 1 : 0,
+                          static_cast<int>(hidden), base32, base64, base64 + at_offsets, base64 + at_dst, base64 + at_send, base64 + at_snapshot,
+                          base64 + at_prefix, expand ? base32 + at_table : nullptr, order_entries > 0 ? base64 + at_order : nullptr,
+                          workspace.data_ptr(), workspace_bytes, turn.mailbox(), comm.stream());
+        if (layout_status != NANOEP_OK && layout_status != NANOEP_ERR_HIP)
+            turn.abandon();  // refused before anything was enqueued
+        check_status(layout_status, "layout");
         expert_counts = arena64.narrow(0, 0, local_experts);
         expert_offsets = arena64.narrow(0, at_offsets, local_experts + 1);
         send_counts = arena64.narrow(0, at_send, 1);
@@ -559,27 +672,32 @@ DispatchResult dispatch(PeerRuntime& runtime,
         }
 
         // The exact shapes (N, C) are only known once the layout kernels have run.  Waiting for
-        // them before launching the permute would leave the GPU idle for a host round trip, so the
-        // outputs are allocated at their upper bound (every choice valid plus every expert's worst
-        // alignment gap), the permute is enqueued right behind the layout, and the results are
-        // narrowed to the exact shapes afterwards.  When the gaps alone could exceed the assignments
-        // (the bound is then more than twice what routing can fill) the exact-allocation order is kept.
+        // them before launching the permute leaves the GPU idle for a host round trip, so where the
+        // upper bound of the shapes (every choice valid plus every expert's worst alignment gap) is
+        // close to what routing will fill, the outputs are allocated at that bound, the permute is
+        // enqueued right behind the layout and the results are narrowed afterwards.  "Close" is
+        // kept honest in both directions: the gaps may add at most an eighth to the bound, and a call
+        // that still ends up holding more than 1.25 times the rows it uses (many masked choices)
+        // permutes again into exact outputs and turns the runtime to the exact order, in which the
+        // outputs are allocated after the counts are known, until a call shows the bound close again.
+        const int64_t choice_bound = expand ? tokens * topk : tokens;
         const int64_t gap_bound = expand ? local_experts * (alignment - 1) : 0;
-        const int64_t row_bound = expand ? tokens * topk + gap_bound : tokens;
-        const bool speculative = tokens > 0 && gap_bound <= tokens * topk + 1024 && row_bound <= std::numeric_limits<int32_t>::max();
+        const int64_t row_bound = choice_bound + gap_bound;
+        const int order_switch = env_switch("NANOEP_FRESH_OUTPUTS");  // 0: always exact, 1: at the bound whenever the rule allows
+        const bool speculative = tokens > 0 && gap_bound * 8 <= choice_bound && row_bound <= std::numeric_limits<int32_t>::max() &&
+                                 order_switch != 0 && (order_switch == 1 || !runtime.prefers_exact_outputs());
         if (speculative) {
             allocate_outputs(row_bound, tokens);
             launch_permute(metadata, tokens, row_bound, /*count_on_device=*/true);
         }
 
         int64_t counts[NANOEP_HOST_COUNT_WORDS] = {0, 0, 0, 0};
-        const int status = nanoep_wait_counts(host_counts, comm.stream(), kCountTimeoutSeconds, counts);
+        const int status = turn.wait(comm.stream(), kCountTimeoutSeconds, counts);
         if (status == NANOEP_ERR_ROUTING) {
             TORCH_CHECK(false, "dispatch routing ids must be -1 or distinct expert ids in [0, ", local_experts, ")",
                         (counts[3] & NANOEP_ROUTING_BAD_EXPERT) ? "; found an id out of range" : "",
                         (counts[3] & NANOEP_ROUTING_DUPLICATE) ? "; found a duplicate expert within a token" : "");
         }
-        check_status(status, "wait_counts");
         recv_count = counts[0];
         expanded_capacity = counts[1];
         TORCH_CHECK(recv_count >= 0 && recv_count <= tokens, "dispatch receive count exceeds the source token count");
@@ -590,18 +708,22 @@ DispatchResult dispatch(PeerRuntime& runtime,
             TORCH_CHECK(counts[2] >= 0 && counts[2] <= slot_order.size(0), "assignment count exceeds the slot-order list");
             metadata[8] = slot_order.narrow(0, 0, counts[2]);  // replays walk the A assignments only
         }
-        if (speculative) {
-            TORCH_CHECK(!expand || expanded_capacity <= row_bound, "expanded capacity exceeds its upper bound");
-            out_x = out_x.narrow(0, 0, expand ? expanded_capacity : recv_count);
+        const int64_t used_rows = expand ? expanded_capacity : recv_count;
+        const bool bound_is_close = used_rows * 5 >= row_bound * 4;  // the bound holds at most 1.25 x the rows in use
+        TORCH_CHECK(used_rows <= row_bound, "receive rows exceed their upper bound");
+        if (speculative && bound_is_close) {
+            out_x = out_x.narrow(0, 0, used_rows);
             if (!expand)
                 out_indices = out_indices.narrow(0, 0, recv_count);
             if (weights.has_value())
-                out_weights = out_weights.narrow(0, 0, expand ? expanded_capacity : recv_count);
+                out_weights = out_weights.narrow(0, 0, used_rows);
         } else {
-            allocate_outputs(expand ? expanded_capacity : recv_count, recv_count);
+            allocate_outputs(used_rows, recv_count);
             if (recv_count > 0)
                 launch_permute(metadata, recv_count, expanded_capacity);
         }
+        if (tokens > 0 && gap_bound * 8 <= choice_bound)
+            runtime.note_output_fill(bound_is_close);
         if (expand)
             runtime.remember_private(metadata, alignment);
     }
@@ -620,7 +742,7 @@ DispatchResult dispatch(PeerRuntime& runtime,
                 tensor.record_stream(comm.unwrap());
         auto protected_tensors = outputs;
         protected_tensors.insert(protected_tensors.end(), metadata.begin(), metadata.end());
-        event = std::make_shared<CompletionEvent>(comm, std::move(protected_tensors));
+        event = CompletionEvent::record_behind(comm, std::move(protected_tensors));
     } else if (!same_queue(comm, compute)) {
         wait_on(compute, comm);
     }
@@ -641,14 +763,15 @@ CombineResult combine(PeerRuntime& runtime,
                       int64_t comm_stream,
                       int64_t previous_event,
                       bool async_op) {
-    TORCH_CHECK(metadata.size() >= 7 && metadata.size() <= 9 && x.dim() == 2 && metadata[5].dim() == 2,
+    TORCH_CHECK(metadata.size() >= 7 && metadata.size() <= 9 && x.defined() && x.dim() == 2 && metadata[5].dim() == 2,
                 "combine requires a 2D payload and seven prepared metadata tensors");
-    (void)runtime.host_counts();  // rejects a closed runtime
+    runtime.require_usable();
     const auto device = static_cast<c10::DeviceIndex>(runtime.device());
     DeviceGuard device_guard(device);
-    TORCH_CHECK(x.is_cuda() && x.get_device() == device && x.is_contiguous() && x.size(1) > 0,
+    const c10::Device here(c10::DeviceType::CUDA, device);
+    TORCH_CHECK(x.is_cuda() && x.device() == here && x.is_contiguous() && x.size(1) > 0,
                 "combine x must be contiguous CUDA [N,H] or [C,H] on the runtime device");
-    TORCH_CHECK(x.scalar_type() == torch::kBFloat16, "combine x must be bfloat16");
+    require(x, {here, torch::kBFloat16, {-1, -1}}, "combine x must be bfloat16");
     TORCH_CHECK(reinterpret_cast<uintptr_t>(x.data_ptr()) % 16 == 0, "combine x data pointer must be 16-byte aligned");
     TORCH_CHECK(x.size(1) % kHiddenAlignment == 0, "combine hidden must be a positive multiple of 256");
     TORCH_CHECK(metadata[1].dim() == 1 && metadata[1].numel() > 0,
@@ -661,20 +784,15 @@ CombineResult combine(PeerRuntime& runtime,
     const int64_t local_experts = metadata[1].numel();
     TORCH_CHECK(topk > 0 && topk <= 32 && topk <= local_experts && source_tokens <= max_tokens && recv_count <= max_tokens,
                 "combine routing geometry exceeds expert/token capacity");
-    check_handle_metadata(metadata, x, source_tokens, topk, local_experts);
+    require_handle_tensors(metadata, here, source_tokens, topk, local_experts);
     TORCH_CHECK(expand ? (x.size(0) >= recv_count && (recv_count != 0 || x.size(0) == 0)) : x.size(0) == recv_count,
                 "combine x rows do not match the receive layout");
-    if (weights.has_value()) {
-        const bool shape_matches = expand ? (weights->dim() == 1 && weights->size(0) == x.size(0))
-                                          : (weights->dim() == 2 && weights->size(0) == recv_count && weights->size(1) == topk);
-        TORCH_CHECK(weights->device() == x.device() && weights->scalar_type() == torch::kFloat32 && weights->is_contiguous() && shape_matches,
-                    "combine weights must be contiguous CUDA float32 [N,K] or expanded [C] on the x device");
-    }
-    if (bias.has_value()) {
-        TORCH_CHECK(bias->device() == x.device() && bias->scalar_type() == torch::kBFloat16 && bias->is_contiguous() &&
-                        bias->sizes() == at::IntArrayRef({source_tokens, hidden}),
-                    "combine bias must be contiguous [T,H], with the output dtype on the x device");
-    }
+    if (weights.has_value())
+        require(*weights, {here, torch::kFloat32, expand ? std::vector<int64_t>{x.size(0)} : std::vector<int64_t>{recv_count, topk}},
+                "combine weights must be contiguous CUDA float32 [N,K] or expanded [C] on the x device");
+    if (bias.has_value())
+        require(*bias, {here, torch::kBFloat16, {source_tokens, hidden}},
+                "combine bias must be contiguous [T,H], with the output dtype on the x device");
     const int cu_budget = resolve_cu_budget(num_sms, device);
 
     const auto compute = c10::hip::getCurrentHIPStreamMasqueradingAsCUDA(device);
@@ -720,7 +838,7 @@ CombineResult combine(PeerRuntime& runtime,
         for (const auto& tensor : metadata)
             if (tensor.numel() > 0)
                 tensor.record_stream(comm.unwrap());
-        event = std::make_shared<CompletionEvent>(comm, outputs);
+        event = CompletionEvent::record_behind(comm, outputs);
     } else if (!same_queue(comm, compute)) {
         wait_on(compute, comm);
     }
@@ -764,6 +882,9 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, module) {
         .def("barrier", &nanoep::PeerRuntime::barrier_at)
         .def("close_peer_mappings", &nanoep::PeerRuntime::close_peer_mappings)
         .def("private_recalls", &nanoep::PeerRuntime::private_recalls)
+        .def("counts_failed", &nanoep::PeerRuntime::counts_failed)
+        .def("prefers_exact_outputs", &nanoep::PeerRuntime::prefers_exact_outputs)
+        .def("lose_counts_for_test", &nanoep::PeerRuntime::lose_counts_for_test)
         .def("close", &nanoep::PeerRuntime::close);
     py::class_<nanoep::CompletionEvent, std::shared_ptr<nanoep::CompletionEvent>>(module, "CompletionEvent")
         .def("current_stream_wait", &nanoep::CompletionEvent::current_stream_wait);

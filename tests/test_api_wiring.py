@@ -285,6 +285,33 @@ def test_construction_checks_without_a_gpu():
         api.CudaBuffer(None, EPConfig(2, 2, 256, 4))
 
 
+def test_control_group_inspection_with_a_real_gloo_group():
+    """The group argument of the reference's Buffer is a Gloo control group; with one rank its
+    single-member form is accepted and anything else refused (no GPU needed for this part)."""
+    import torch.distributed as dist
+
+    assert api.CudaBuffer._inspect_group(None) == (0, 1)
+    assert not dist.is_initialized()
+    dist.init_process_group("gloo", store=dist.HashStore(), rank=0, world_size=1)
+    try:
+        assert api.CudaBuffer._inspect_group(dist.group.WORLD) == (0, 1)
+        assert api.CudaBuffer._inspect_group(dist.new_group(ranks=[0], backend="gloo")) == (0, 1)
+    finally:
+        dist.destroy_process_group()
+
+    class FakeDist:
+        def __init__(self, backend, size):
+            self.backend, self.size = backend, size
+
+    import unittest.mock as mock
+
+    for backend, size, message in (("nccl", 1, "Gloo"), ("gloo", 2, "world_size == 1")):
+        with mock.patch.object(dist, "get_backend", lambda group, b=backend: b), \
+                mock.patch.object(dist, "get_world_size", lambda group=None, n=size: n):
+            with pytest.raises(ValueError, match=message):
+                api.CudaBuffer._inspect_group(object())
+
+
 def test_reference_import_paths():
     """`nano_ep`, `nano_ep.backends` and `nano_ep.backends.cuda` export these names (nano_ep/__init__.py,
     nano_ep/backends/__init__.py); the same import paths exist here and name the same objects."""

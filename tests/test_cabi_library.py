@@ -91,6 +91,32 @@ def test_argument_checks_come_before_any_device_work():
     assert library.nanoep_wait_counts(null, null, 0.0, out) == 1
 
 
+def test_wait_counts_reads_a_mailbox_the_host_wrote():
+    """nanoep_wait_counts against a mailbox in plain host memory, no GPU involved: published counts
+    come back whole, a routing status word turns into NANOEP_ERR_ROUTING with the words still
+    delivered, and a word that never arrives ends in NANOEP_ERR_TIMEOUT once the caller's patience
+    (none here) is used up, before the stream is ever looked at."""
+    library = cabi.lib()
+    mailbox = (ctypes.c_int64 * 4)(17, 40, 33, 0)
+    out = (ctypes.c_int64 * 4)()
+    assert library.nanoep_wait_counts(mailbox, None, 0.0, out) == 0 and list(out) == [17, 40, 33, 0]
+    # N == 0 is a count like any other
+    mailbox[:] = [0, 0, 0, 0]
+    assert library.nanoep_wait_counts(mailbox, None, 0.0, out) == 0 and list(out) == [0, 0, 0, 0]
+    for status_word in (1, 2, 3):
+        mailbox[:] = [5, 9, 8, status_word]
+        assert library.nanoep_wait_counts(mailbox, None, 0.0, out) == 5 and list(out) == [5, 9, 8, status_word]
+    # word 0 still -1 (what nanoep_layout leaves there until the device has stored the rest)
+    mailbox[:] = [-1, 40, 33, 0]
+    out[:] = [7, 7, 7, 7]
+    assert library.nanoep_wait_counts(mailbox, None, 0.0, out) == 4
+    assert list(out) == [7, 7, 7, 7]  # nothing is delivered from an unpublished mailbox
+    assert b"timed out" in library.nanoep_status_string(4)
+    # ... and a late store is only seen by a later wait
+    mailbox[0] = 3
+    assert library.nanoep_wait_counts(mailbox, None, 0.0, out) == 0 and list(out) == [3, 40, 33, 0]
+
+
 def test_static_layout_checks_arguments_and_its_size_limit_before_any_device_work():
     library = cabi.lib()
     null = None

@@ -84,6 +84,34 @@ def test_readme_round_trip(device):
         assert result.topk_weights is None and result.event is None
 
 
+def test_readme_round_trip_with_a_gloo_control_group(device):
+    """The reference's toy run as its README writes it: a single-member Gloo group handed to Buffer
+    (README.md:44-70), identity experts, combine reproduces x.  Groups the build cannot serve (a
+    second member is not available on one GPU; another backend is) are refused."""
+    import torch.distributed as dist
+
+    assert not dist.is_initialized()
+    dist.init_process_group("gloo", store=dist.HashStore(), rank=0, world_size=1)
+    try:
+        group = dist.new_group(ranks=[0], backend="gloo")
+        config = EPConfig(num_experts=2, num_topk=2, hidden=256, num_max_tokens_per_rank=16)
+        x = cases.payload(16, 256, seed=0).to(device)
+        indices = torch.tensor([[0, 1]], dtype=torch.int64).repeat(16, 1).to(device)
+        weights = torch.full((16, 2), 0.5, dtype=torch.float32, device=device)
+        for control in (group, dist.group.WORLD):
+            with Buffer(control, config) as buffer:
+                assert (buffer._rank, buffer._world_size) == (0, 1)
+                received = buffer.dispatch(x, topk_idx=indices, weights=weights, do_expand=True, zero_padding=True)
+                assert (received.handle.rank, received.handle.world_size) == (0, 1)
+                expert_x = (received.x.float() * received.topk_weights[:, None]).to(received.x.dtype)
+                result = buffer.combine(expert_x, received.handle)
+                torch.testing.assert_close(result.x, x, rtol=0, atol=0)
+        with pytest.raises(ValueError, match="divisible|hidden"):
+            Buffer(group, EPConfig(num_experts=2, num_topk=2, hidden=128, num_max_tokens_per_rank=16))
+    finally:
+        dist.destroy_process_group()
+
+
 @pytest.mark.parametrize(
     "expand,zero_padding,weighted,kind,hidden,alignment",
     [
@@ -153,14 +181,20 @@ def test_fresh_and_cached_replay(device, monkeypatch, walk, expand, zero_padding
         buffer.close()
 
 
-@pytest.mark.parametrize("alignment,at_bound", [(16, True), (19, True), (20, False), (64, False)])
+def held_rows(tensor, hidden):
+    return tensor.untyped_storage().nbytes() // (2 * hidden)
+
+
+@pytest.mark.parametrize("alignment,at_bound", [(1, True), (3, True), (4, False), (64, False)])
 def test_fresh_dispatch_allocation_orders(device, alignment, at_bound):
     """A fresh dispatch allocates its outputs at their upper bound and narrows them while the
-    alignment gaps cannot exceed the assignments by more than 1024 rows (the permute then runs
-    right behind the layout), and exactly, after the host has the counts, beyond: same results."""
-    tokens, experts, topk, hidden = 40, 64, 4, 512
-    assert (experts * (alignment - 1) <= tokens * topk + 1024) == at_bound
-    idx = cases.routing("dropout", tokens, experts, topk, seed=alignment)
+    alignment gaps add at most an eighth to that bound (the permute then runs right behind the
+    layout), and exactly, after the host has the counts, beyond: same results, and never more than
+    1.25 times the rows in use are held."""
+    tokens, experts, topk, hidden = 40, 8, 4, 512
+    assert (experts * (alignment - 1) * 8 <= tokens * topk) == at_bound
+    idx = cases.routing("random", tokens, experts, topk, seed=alignment)
+    idx[0, 0] = -1
     x = cases.payload(tokens, hidden)
     w = cases.gate_weights(tokens, topk)
     with Buffer(None, EPConfig(experts, topk, hidden, tokens)) as buffer:
@@ -168,33 +202,68 @@ def test_fresh_dispatch_allocation_orders(device, alignment, at_bound):
                                 alignment=alignment, zero_padding=True)
         lay = assert_dispatch_result(fresh, x, idx, w, experts, True, alignment, True)
         assert_handle(fresh.handle, lay, True, alignment, buffer)
-        held_rows = fresh.x.untyped_storage().nbytes() // (2 * hidden)
+        bound = tokens * topk + experts * (alignment - 1)
         if at_bound:
-            assert held_rows >= tokens * topk + experts * (alignment - 1) > fresh.x.shape[0]
+            assert held_rows(fresh.x, hidden) >= bound > fresh.x.shape[0]
         else:
-            assert held_rows < tokens * topk + experts * (alignment - 1)
+            assert held_rows(fresh.x, hidden) < bound
+        assert fresh.x.untyped_storage().nbytes() <= 1.25 * fresh.x.nbytes + 512
+        assert not buffer._runtime.prefers_exact_outputs()
         replay = buffer.dispatch(x.to(device), weights=w.to(device), handle=fresh.handle, zero_padding=True)
         assert torch.equal(replay.x.view(torch.int16), fresh.x.view(torch.int16))
         assert torch.equal(replay.topk_weights, fresh.topk_weights)
 
 
-@pytest.mark.parametrize(
-    "tokens,hidden,switch",
-    [
-        pytest.param(2048, 4096, None, id="16MiB-rebuilds-by-itself"),
-        pytest.param(37, 512, "1", id="small-forced-rebuild"),
-        pytest.param(2048, 4096, "0", id="16MiB-token-order-forced"),
-    ],
-)
+@pytest.mark.parametrize("expand", [False, True], ids=["compact", "expanded"])
+def test_fresh_dispatch_never_holds_much_more_than_it_uses(device, expand):
+    """With many masked choices the upper bound is far above what routing fills.  The call that finds
+    that out permutes again into exact outputs, later calls allocate after the counts are known, and
+    a batch that fills the bound again turns the runtime back: every result is the oracle's and
+    holds at most 1.25 times its rows."""
+    tokens, experts, topk, hidden = 96, 8, 4, 512
+    sparse = cases.routing("random", tokens, experts, topk, seed=1)
+    sparse[torch.rand(tokens, topk, generator=torch.Generator().manual_seed(5)) < 0.6] = -1
+    sparse[::2] = -1  # half the tokens are not sent at all
+    dense = cases.routing("random", tokens, experts, topk, seed=2)
+    x, w = cases.payload(tokens, hidden, seed=3), cases.gate_weights(tokens, topk)
+    with Buffer(None, EPConfig(experts, topk, hidden, tokens)) as buffer:
+        runtime = buffer._runtime
+        for idx, exact_before, exact_after in ((sparse, False, True), (sparse, True, True), (dense, True, False), (dense, False, False)):
+            assert runtime.prefers_exact_outputs() is exact_before
+            result = buffer.dispatch(x.to(device), topk_idx=idx.to(device), weights=w.to(device), do_expand=expand, zero_padding=True)
+            assert_dispatch_result(result, x, idx, w, experts, expand, 1, True)
+            assert result.x.untyped_storage().nbytes() <= 1.25 * result.x.nbytes + 512
+            assert result.topk_weights.untyped_storage().nbytes() <= 1.25 * result.topk_weights.nbytes + 512
+            assert runtime.prefers_exact_outputs() is exact_after
+            combined = buffer.combine(result.x, result.handle)
+            lay = oracle.layout(idx, experts, 1)
+            want, _ = oracle.combine(result.x.cpu(), lay.recv_metadata(expand), lay.dst_slots, do_expand=expand)
+            assert_same_bits(combined.x, want, "combine after the allocation order changed")
+
+
+def test_headline_shapes_hold_at_most_a_quarter_more_than_they_use(device):
+    """The DeepSeek-V3 batch with alignment 1 (at the bound) and 128 (exact order)."""
+    from nanoep_amd import workloads
+
+    for name in ("deepseek-v3", "deepseek-v3-a128"):
+        work = workloads.WORKLOADS[name]
+        x, idx, w = workloads.make_inputs(work)
+        with Buffer(None, EPConfig(work.experts, work.topk, work.hidden, work.tokens)) as buffer:
+            result = buffer.dispatch(x.to(device), topk_idx=idx.to(device), weights=w.to(device), do_expand=True,
+                                     alignment=work.alignment, zero_padding=True)
+            lay = oracle.layout(idx, work.experts, work.alignment)
+            assert result.x.shape[0] == lay.expanded_capacity
+            assert result.x.untyped_storage().nbytes() <= 1.25 * result.x.nbytes
+            del result
+
+
 @pytest.mark.parametrize("recall", [False, True], ids=["no-recall", "recall"])
-def test_replay_with_only_the_reference_handle_tensors(device, monkeypatch, tokens, hidden, switch, recall):
+@pytest.mark.parametrize("tokens,hidden", [(2048, 4096), (37, 512)], ids=["16MiB", "small"])
+def test_replay_with_only_the_reference_handle_tensors(device, monkeypatch, tokens, hidden, recall):
     """A handle that carries just the reference's seven tensors (as one that went through the
-    reference's own Python class would) replays to the same bytes.  While it is the handle of the
-    buffer's latest fresh dispatch the runtime hands its private tensors back (recall); otherwise
-    the extension makes the slot-order list again on the device for large payloads, or walks in
-    token order."""
-    if switch is not None:
-        monkeypatch.setenv("NANOEP_REBUILD_ORDER", switch)
+    reference's own Python class would) replays to the same bytes.  While it is one of the buffer's
+    latest fresh dispatches the runtime hands its private tensors back (recall); otherwise the
+    payload follows the handle's own dst_slots and recv_metadata in token order."""
     if not recall:
         monkeypatch.setenv("NANOEP_RECALL_ORDER", "0")
     experts, topk, alignment = 16, 4, 8
@@ -218,7 +287,7 @@ def test_replay_with_only_the_reference_handle_tensors(device, monkeypatch, toke
         again = buffer.dispatch(x.to(device), topk_idx=idx.flip(0).contiguous().to(device), do_expand=True, alignment=alignment)
         lay = oracle.layout(idx.flip(0).contiguous(), experts, alignment)
         assert again.handle.layout.recv_count == lay.recv_count and again.handle.layout.expanded_capacity == lay.expanded_capacity
-        # ... and the runtime now remembers that dispatch: the older handle is no longer recalled
+        # ... the runtime remembers its latest few dispatches: the older handle is still recalled
         recalls = buffer._runtime.private_recalls()
         combined = buffer.combine(full.x, bare)
         want, _ = oracle.combine(full.x.cpu(), oracle.layout(idx, experts, alignment).recv_metadata(True),
@@ -226,8 +295,9 @@ def test_replay_with_only_the_reference_handle_tensors(device, monkeypatch, toke
         assert_same_bits(combined.x, want, "combine through the bare handle")
         late = buffer.dispatch(x.to(device), weights=w.to(device), handle=bare, zero_padding=True)
         assert_dispatch_result(late, x, idx, w, experts, True, alignment, True)
-        assert buffer._runtime.private_recalls() == recalls
-        # the latest one is, by dispatch and by combine
+        assert buffer._runtime.private_recalls() == recalls + (2 if recall else 0)
+        # and so is the latest one, by dispatch and by combine
+        recalls = buffer._runtime.private_recalls()
         newest = dataclasses.replace(again.handle, token_slots=None, slot_order=None)
         newest_replay = buffer.dispatch(x.to(device), handle=newest)
         assert_dispatch_result(newest_replay, x, idx.flip(0).contiguous(), None, experts, True, alignment, False)
@@ -237,8 +307,64 @@ def test_replay_with_only_the_reference_handle_tensors(device, monkeypatch, toke
         want_newest, _ = oracle.combine(y, flipped.recv_metadata(True), flipped.dst_slots, do_expand=True)
         assert_same_bits(buffer.combine(y.to(device), newest).x, want_newest, "combine through the newest bare handle")
         assert buffer._runtime.private_recalls() == recalls + (2 if recall else 0)
+        # after four more fresh dispatches whose handles are still alive the first handle has dropped
+        # out of the runtime's memory (handles that died are forgotten first)
+        alive = []
+        for seed in range(4):
+            other = cases.routing("dropout", tokens, experts, topk, seed=20 + seed)
+            alive.append(buffer.dispatch(x.to(device), topk_idx=other.to(device), do_expand=True, alignment=alignment).handle)
+        recalls = buffer._runtime.private_recalls()
+        forgotten = buffer.dispatch(x.to(device), weights=w.to(device), handle=bare, zero_padding=True)
+        assert_dispatch_result(forgotten, x, idx, w, experts, True, alignment, True)
+        assert buffer._runtime.private_recalls() == recalls
     finally:
         buffer.close()
+
+
+def test_a_foreign_seven_tensor_handle_is_followed_as_written(device):
+    """A valid handle in another row and slot order than this library's own (here: receive rows and
+    slots in reverse token order, as a caller may build them) is honoured by the host extension
+    whatever the payload size: every row lands where the handle's recv_metadata says, and combine
+    brings it back.  (16 MiB payload: the size from which an earlier version rebuilt its own order.)"""
+    tokens, experts, topk, hidden, alignment = 2048, 16, 4, 4096, 4
+    idx = cases.routing("dropout", tokens, experts, topk, seed=3)
+    x, w = cases.payload(tokens, hidden, seed=6), cases.gate_weights(tokens, topk)
+    lay = oracle.layout(idx, experts, alignment)
+    # reversed rows: receive row r holds the (N-1-r)-th sending token; reversed slots inside every expert segment
+    meta = lay.recv_metadata(True).flip(0).contiguous()
+    counts, offsets = lay.expert_counts, lay.expert_offsets
+    slots = meta[:, 2:].clone().to(torch.int64)
+    expert_of = torch.bucketize(slots.clamp(min=0), offsets[1:], right=True)
+    mirrored = offsets[expert_of] + counts[expert_of] - 1 - (slots - offsets[expert_of])
+    meta[:, 2:] = torch.where(slots >= 0, mirrored, slots).to(torch.int32)
+    dst = torch.where(lay.dst_slots >= 0, lay.recv_count - 1 - lay.dst_slots, lay.dst_slots)
+    public = [meta, counts, offsets, dst, lay.send_counts, idx.clone(), lay.recv_rank_prefix]
+    native = load_extension()
+    with Buffer(None, EPConfig(experts, topk, hidden, tokens)) as buffer:
+        handle = [t.to(device) for t in public]
+        stream = buffer.comm_stream.cuda_stream
+        cus = torch.cuda.get_device_properties(device).multi_processor_count
+        outputs, returned, (received, capacity), event = native.dispatch(
+            buffer._runtime, x.to(device), handle[5], w.to(device), experts, tokens, alignment, handle, lay.expanded_capacity,
+            False, True, True, cus, stream, -1, False)
+        assert event is None and (received, capacity) == (lay.recv_count, lay.expanded_capacity)
+        got_x, got_w = outputs[0].cpu(), outputs[2].cpu()
+        want_x = torch.zeros_like(got_x)
+        want_w = torch.zeros_like(got_w)
+        for row in range(meta.shape[0]):
+            token = int(meta[row, 1])
+            for k in range(topk):
+                slot = int(meta[row, 2 + k])
+                if slot >= 0:
+                    want_x[slot] = x[token]
+                    want_w[slot] = w[token, k]
+        assert_same_bits(got_x, want_x, "rows follow the handle's recv_metadata")
+        assert_same_bits(got_w, want_w, "weights follow the handle's recv_metadata")
+        (combined, restored), _ = native.combine(buffer._runtime, outputs[0], handle, outputs[2], None, tokens, True, False, cus,
+                                                 stream, -1, False)
+        want, want_cw = oracle.combine(want_x, meta, dst, do_expand=True, weights=want_w)
+        assert_same_bits(combined, want, "combine through the foreign handle")
+        assert_same_bits(restored, want_cw, "weights restored through the foreign handle")
 
 
 @pytest.mark.parametrize("expand", [False, True], ids=["compact", "expanded"])
@@ -399,6 +525,116 @@ def test_argument_errors(device):
         Buffer(None, config, allow_multiple_reduction=1)
     with pytest.raises(ValueError, match="256"):
         Buffer(None, EPConfig(4, 2, 128, 8))
+
+
+def test_fresh_dispatches_of_two_threads_on_one_buffer(device):
+    """dispatch runs without the interpreter lock, and a buffer has one mailbox for N and C: fresh
+    dispatches of two Python threads take turns at it, and each gets the counts and the layout of
+    its own routing."""
+    import threading
+
+    tokens, experts, topk, hidden = 700, 32, 4, 512
+    routings = [cases.routing("dropout", tokens - 100 * i, experts, topk, seed=40 + i) for i in range(2)]
+    for i, idx in enumerate(routings):
+        idx[: 50 * (i + 1)] = -1  # different N and C per thread
+    xs = [cases.payload(idx.shape[0], hidden, seed=i) for i, idx in enumerate(routings)]
+    expected = [oracle.layout(idx, experts, 4) for idx in routings]
+    assert expected[0].recv_count != expected[1].recv_count
+    failures = []
+    with Buffer(None, EPConfig(experts, topk, hidden, tokens)) as buffer:
+        start = threading.Barrier(2)
+
+        def worker(which):
+            try:
+                torch.cuda.set_device(device)
+                stream = torch.cuda.Stream(device=device)
+                idx_gpu, x_gpu = routings[which].to(device), xs[which].to(device)
+                torch.cuda.synchronize()
+                start.wait()
+                with torch.cuda.stream(stream):
+                    for _ in range(60):
+                        result = buffer.dispatch(x_gpu, topk_idx=idx_gpu, do_expand=True, alignment=4, zero_padding=True)
+                        layout = result.handle.layout
+                        if (layout.recv_count, layout.expanded_capacity) != (expected[which].recv_count, expected[which].expanded_capacity):
+                            failures.append((which, layout.recv_count, layout.expanded_capacity))
+                            return
+                    stream.synchronize()
+                    assert_dispatch_result(result, xs[which], routings[which], None, experts, True, 4, True)
+                    assert_handle(result.handle, expected[which], True, 4, buffer)
+            except Exception as error:  # noqa: BLE001 - reported by the main thread
+                failures.append((which, repr(error)))
+
+        threads = [threading.Thread(target=worker, args=(i,)) for i in range(2)]
+        for thread in threads:
+            thread.start()
+        for thread in threads:
+            thread.join(timeout=100)
+        assert not any(thread.is_alive() for thread in threads)
+        assert failures == []
+        assert not buffer._runtime.counts_failed()
+
+
+def test_a_fresh_dispatch_that_lost_its_counts_leaves_the_runtime_failed(device):
+    """The reference latches a failure when the host wait for N and C does not end well
+    (csrc/peer.cu:229-232) and serves nothing afterwards: a count stored late must not answer a
+    later call.  Here the loss is staged on the host (a turn at the mailbox that ends without a
+    verdict); no kernel misbehaves."""
+    tokens, experts, topk, hidden = 8, 4, 2, 256
+    idx = cases.routing("random", tokens, experts, topk).to(device)
+    x = cases.payload(tokens, hidden).to(device)
+    buffer = Buffer(None, EPConfig(experts, topk, hidden, tokens))
+    received = buffer.dispatch(x, topk_idx=idx, do_expand=True)
+    assert not buffer._runtime.counts_failed()
+    buffer._runtime.lose_counts_for_test()
+    assert buffer._runtime.counts_failed()
+    for call in (
+        lambda: buffer.dispatch(x, topk_idx=idx, do_expand=True),
+        lambda: buffer.dispatch(x, handle=received.handle),
+        lambda: buffer.combine(received.x, received.handle),
+        lambda: buffer._runtime.lose_counts_for_test(),
+    ):
+        with pytest.raises(RuntimeError, match="failed while waiting for its counts"):
+            call()
+    buffer.close()  # closing still works
+    with pytest.raises(RuntimeError, match="closed"):
+        buffer.dispatch(x, topk_idx=idx)
+
+
+@pytest.mark.parametrize("alignment", [1, 16], ids=["outputs-at-the-bound", "outputs-exact"])
+def test_rejected_routing_with_padding_and_weights_then_a_good_dispatch(device, alignment):
+    """A routing error is only known once the host has the status word; where the outputs are
+    allocated at their bound the permute has by then run on the rejected layout.  It must not harm
+    anything: earlier results and their neighbours in memory keep their bytes, the error is the
+    routing error, and the next dispatch is the oracle's."""
+    tokens, experts, topk, hidden = 300, 16, 4, 512
+    idx = cases.routing("dropout", tokens, experts, topk, seed=8)
+    x, w = cases.payload(tokens, hidden, seed=2), cases.gate_weights(tokens, topk)
+    with Buffer(None, EPConfig(experts, topk, hidden, tokens)) as buffer:
+        before = buffer.dispatch(x.to(device), topk_idx=idx.to(device), weights=w.to(device), do_expand=True,
+                                 alignment=alignment, zero_padding=True)
+        kept_x, kept_w = before.x.clone(), before.topk_weights.clone()
+        # freed blocks around the next allocations carry a known pattern
+        guards = [torch.full((rows, hidden), -3.0, dtype=torch.bfloat16, device=device) for rows in (64, 2048, 64)]
+        pattern = [guard.clone() for guard in guards]
+        for bad_value, message in ((experts, "out of range"), (-2, "out of range"), (None, "duplicate")):
+            bad = idx.clone()
+            if bad_value is None:
+                bad[7] = 3
+            else:
+                bad[5, 1] = bad_value
+            with pytest.raises(RuntimeError, match=message):
+                buffer.dispatch(x.to(device), topk_idx=bad.to(device), weights=w.to(device), do_expand=True,
+                                alignment=alignment, zero_padding=True)
+            assert not buffer._runtime.counts_failed()
+        torch.cuda.synchronize()
+        for guard, want in zip(guards, pattern):
+            assert torch.equal(guard.view(torch.int16), want.view(torch.int16))
+        assert torch.equal(before.x.view(torch.int16), kept_x.view(torch.int16))
+        assert torch.equal(before.topk_weights.view(torch.int32), kept_w.view(torch.int32))
+        good = buffer.dispatch(x.to(device), topk_idx=idx.to(device), weights=w.to(device), do_expand=True,
+                               alignment=alignment, zero_padding=True)
+        lay = assert_dispatch_result(good, x, idx, w, experts, True, alignment, True)
+        assert_handle(good.handle, lay, True, alignment, buffer)
 
 
 def test_deterministic_fill_is_rejected_by_the_api_but_not_the_backend(device):

@@ -217,8 +217,6 @@ def test_more_tokens_than_resident_waves(device, expand, zero_padding, weighted,
     idx[:3] = -1
     idx[::2, 1:] = -1
     run_dispatch_combine(device, idx, hidden, 3, 128, expand, zero_padding, weighted, seed=3)
-    # the same work under a small CU budget exercises the grid-stride loop
-    run_dispatch_combine(device, idx, hidden, 3, 128, expand, zero_padding, weighted, seed=4, num_cus=2)
 
 
 @pytest.mark.parametrize(
@@ -371,6 +369,54 @@ def test_windows_of_1024_tokens(device, tokens, experts, topk, hidden):
     assert cabi.lib().nanoep_layout_block_tokens(tokens, experts, hidden) == 1024
     idx = cases.routing("dropout", tokens, experts, topk, seed=tokens)
     run_dispatch_combine(device, idx, hidden, experts, 8, True, True, True, seed=3)
+
+
+@pytest.mark.parametrize("window,tokens", [(96, 1000), (160, 4096), (192, 4096), (224, 2000), (512, 1500)])
+def test_forced_window_sizes(device, monkeypatch, window, tokens):
+    """NANOEP_WINDOW_TOKENS orders the slot-order list by windows of any multiple of 32 tokens up to
+    256 (one layout workgroup each; the last one ragged, and more workgroups' worth of tokens than
+    the list buffer, which is sized by blocks of 256, has room for beyond the batch)."""
+    monkeypatch.setenv("NANOEP_WINDOW_TOKENS", str(window))
+    assert cabi.lib().nanoep_layout_block_tokens(tokens, 24, 512) == window
+    idx = cases.routing("dropout", tokens, 24, 4, seed=window)
+    run_dispatch_combine(device, idx, 512, 24, 8, True, True, True, seed=5)
+
+
+@pytest.mark.parametrize("use_order", [True, False], ids=["slot-order", "token-order"])
+@pytest.mark.parametrize("bad", ["out-of-range", "duplicate"])
+def test_dispatch_behind_a_rejected_layout_stays_inside_its_bound(device, bad, use_order):
+    """A caller that enqueues the permute before it has read the counts (outputs at their upper
+    bound, entry count read on the device) finds out about a routing error afterwards.  Whatever
+    the rejected layout holds, the permute, its zero fill and its weights write nothing outside
+    the rows they were given: guard rows on both sides keep their pattern."""
+    tokens, experts, topk, hidden, alignment, guard = 700, 12, 4, 512, 16, 8
+    idx = cases.routing("dropout", tokens, experts, topk, seed=31)
+    if bad == "duplicate":
+        idx[5] = 3
+        idx[600, 1] = idx[600, 0] = 7
+    else:
+        idx[5, 2], idx[300, 0], idx[699, 3] = experts, -5, 1 << 40
+    x = cases.payload(tokens, hidden, seed=1).to(device)
+    w = cases.gate_weights(tokens, topk).to(device)
+    metadata, counts = cabi.layout(idx.to(device), experts, alignment, True, raise_on_routing=False, hidden=hidden)
+    assert counts[3] & (2 if bad == "duplicate" else 1)
+    bound = tokens * topk + experts * (alignment - 1)
+    rows = torch.full((guard + bound + guard, hidden), -3.0, dtype=torch.bfloat16, device=device)
+    row_weights = torch.full((guard + bound + guard,), -3.0, dtype=torch.float32, device=device)
+    order = metadata[8] if use_order else None
+    library = cabi.lib()
+    cabi.check(library.nanoep_dispatch(
+        cabi.ptr(x), cabi.ptr(w), cabi.ptr(metadata[0]), cabi.ptr(metadata[3]), cabi.ptr(metadata[7]), cabi.ptr(order),
+        -1 if use_order else 0, cabi.ptr(metadata[1]), cabi.ptr(metadata[2]), tokens, bound, tokens, hidden, topk, experts, alignment, 1, 1,
+        rows[guard:].data_ptr(), None, row_weights[guard:].data_ptr(), 0, cabi.stream_handle()))
+    torch.cuda.synchronize()
+    for name, tensor in (("rows", rows), ("weights", row_weights)):
+        edges = torch.cat((tensor[:guard], tensor[guard + bound:])).cpu()
+        assert torch.equal(edges, torch.full_like(edges, -3.0)), f"{name} outside the bound were written"
+    # every row that was written holds a source row or zeros
+    written = rows[guard:guard + bound].cpu()
+    touched = (written.view(torch.int16) != torch.tensor(-3.0, dtype=torch.bfloat16).view(torch.int16)).any(dim=1)
+    assert touched.any()
 
 
 @pytest.mark.parametrize("tokens", [300, 5000])
