@@ -13,7 +13,8 @@ then REGIONS timed regions of REGION_LAUNCHES back-to-back launches each, every 
 a device synchronisation and two HIP events on the kernels' stream; the figure reported for a kernel
 is the MEDIAN of the regions' per-launch times, with the fastest region beside it (`*_min`).  The
 region of exactly --steps steps after --warmup warm-up steps is timed as well and reported as
-`cli_region`.  `--workload all` adds the other benchmark shapes under `roofline_by_workload`.
+`cli_region`.  The other benchmark shapes follow under `roofline_by_workload` (same protocol, shorter
+CPU samples; `--workload deepseek-v3` leaves them out).
 """
 
 from __future__ import annotations
@@ -47,11 +48,13 @@ def parse_args():
     parser.add_argument("--gpus", type=int, default=1)
     parser.add_argument("--steps", type=int, default=200)
     parser.add_argument("--warmup", type=int, default=50)
-    parser.add_argument("--workload", default=HEADLINE,
-                        help="one benchmark shape, or `all`: the headline shape plus the others under roofline_by_workload")
+    parser.add_argument("--workload", default="all",
+                        help="`all` (default): the headline shape, then the other benchmark shapes under roofline_by_workload; "
+                             "or the name of one shape")
     parser.add_argument("--cpu-seconds", type=float, default=15.0, help="CPU baseline budget per workload; 0 skips it")
-    parser.add_argument("--scalar-oracle", action="store_true",
-                        help="also time the scalar-loop oracle once (readme-toy and mixtral shapes only: it is a specification, not a performance path)")
+    parser.add_argument("--no-scalar-oracle", dest="scalar_oracle", action="store_false",
+                        help="skip timing the scalar-loop oracle (it runs once on the readme-toy and mixtral shapes only: "
+                             "it is a specification, not a performance path)")
     parser.add_argument("--regions", type=int, default=REGIONS)
     parser.add_argument("--region-launches", type=int, default=REGION_LAUNCHES)
     parser.add_argument("--calibration-copy-mib", type=int, default=0,
@@ -158,13 +161,15 @@ def cpu_baseline(workload, x, idx, weights, budget_seconds, gpu_dispatched=None,
     layout = oracle.layout(idx, workload.experts, workload.alignment)
     received, capacity = layout.recv_count, layout.expanded_capacity
     assignments = int(layout.expert_counts.sum())
-    nbytes = workloads.dispatch_bytes(workload, received, assignments, capacity) + workloads.combine_bytes(workload, received, assignments)
+    nbytes = (workloads.dispatch_bytes(workload, received, assignments, capacity)
+              + workloads.combine_bytes(workload, received, assignments, weighted=workload.combine_weights))
     metadata = layout.recv_metadata(workload.expand)
 
     def step():
-        out_x, _, _, _ = oracle.dispatch(x, idx, workload.experts, weights, do_expand=workload.expand,
-                                         alignment=workload.alignment, lay=layout)
-        oracle.combine(out_x, metadata, layout.dst_slots, do_expand=workload.expand)
+        out_x, _, out_w, _ = oracle.dispatch(x, idx, workload.experts, weights, do_expand=workload.expand,
+                                             alignment=workload.alignment, lay=layout)
+        oracle.combine(out_x, metadata, layout.dst_slots, do_expand=workload.expand,
+                       weights=out_w if workload.combine_weights else None)
 
     parity = None
     if gpu_dispatched is not None:
@@ -267,7 +272,7 @@ def measure(workload, args, device, detailed):
     with torch.cuda.stream(stream):
         # fresh dispatch: layout kernels + host wait for N/C + permute, as seen by the caller
         fresh_times, fresh_gpu_times = [], []
-        fresh_calls = (WARMUP_MIN + 4 * rotation) if detailed else 2
+        fresh_calls = WARMUP_MIN + (4 * rotation if detailed else 20)
         for call in range(fresh_calls, -1, -1):  # rotating sources like the timed steps; the last call takes xs[0]
             begin, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
             torch.cuda.synchronize()
@@ -277,7 +282,7 @@ def measure(workload, args, device, detailed):
                                        alignment=workload.alignment, zero_padding=workload.zero_padding)
             end.record(stream)
             torch.cuda.synchronize()
-            if call < fresh_calls - WARMUP_MIN or not detailed:
+            if call < fresh_calls - WARMUP_MIN:
                 fresh_times.append(time.perf_counter() - t0)
                 fresh_gpu_times.append(begin.elapsed_time(end) * 1e-3)
         handle = received.handle
@@ -289,16 +294,25 @@ def measure(workload, args, device, detailed):
         n_recv, capacity = handle.layout.recv_count, handle.layout.expanded_capacity
         assignments = int(handle.layout.expert_counts.sum().item())
         d_bytes = workloads.dispatch_bytes(workload, n_recv, assignments, capacity)
-        c_bytes = workloads.combine_bytes(workload, n_recv, assignments)
+        c_bytes = workloads.combine_bytes(workload, n_recv, assignments, weighted=workload.combine_weights)
 
         ring = [received.x, received.x.clone(), received.x.clone()]  # combine reads a two-steps-old dispatch output
 
+        asynchronous = workload.async_op
+        ring_weights = received.topk_weights if workload.combine_weights else None
+
         def do_dispatch(i):
-            out = buffer.dispatch(xs[i % rotation], weights=weights, handle=handle, zero_padding=workload.zero_padding)
+            out = buffer.dispatch(xs[i % rotation], weights=weights, handle=handle, zero_padding=workload.zero_padding,
+                                  async_op=asynchronous)
+            if asynchronous:
+                out.event.current_stream_wait()
             ring[i % 3] = out.x
 
         def do_combine(i):
-            return buffer.combine(ring[(i + 1) % 3], handle)
+            out = buffer.combine(ring[(i + 1) % 3], handle, weights=ring_weights, async_op=asynchronous)
+            if asynchronous:
+                out.event.current_stream_wait()
+            return out
 
         def step(i):
             do_dispatch(i)
@@ -372,7 +386,9 @@ def measure(workload, args, device, detailed):
                 "received_rows": n_recv,
                 "assignments": assignments,
                 "expanded_capacity": capacity,
-                "step": "cached-handle dispatch + combine through Buffer.dispatch / Buffer.combine",
+                "step": "cached-handle dispatch + combine through Buffer.dispatch / Buffer.combine"
+                        + (", async_op=True with the consumer stream waiting on each completion event" if workload.async_op else "")
+                        + (", combine returning the weights" if workload.combine_weights else ""),
                 "rotating_source_copies": rotation,
             },
             "timing": {"warmup_launches": WARMUP_MIN, "regions": regions, "launches_per_region": launches,
@@ -422,7 +438,7 @@ def main():
 
     from nanoep_amd import workloads
 
-    names = [HEADLINE, "mixtral", "qwen3-moe", "ep8-share", "deepseek-v3-a128"] if args.workload == "all" else [args.workload]
+    names = [HEADLINE, "mixtral", "qwen3-moe", "ep8-share", "deepseek-v3-a128", "readme-toy"] if args.workload == "all" else [args.workload]
     if any(name not in workloads.WORKLOADS for name in names):
         log("unknown workload", args.workload, "choose from", sorted(workloads.WORKLOADS), "or all")
         return 2

@@ -23,6 +23,8 @@ class Workload:
     alignment: int
     zero_padding: bool
     description: str
+    async_op: bool = False          # calls return a completion event that the consumer stream waits on
+    combine_weights: bool = False   # combine is given the dispatched weights and returns them as [T, K]
 
 
 WORKLOADS = {
@@ -37,7 +39,9 @@ WORKLOADS = {
     "ep8-share": Workload("ep8-share", 32768, 7168, 32, 8, "zipf", False, 1, False,
                           "32768 x 7168 (8 source segments x 4096), 32 local experts top-8 Zipf(1.2), compact, cached handle"),
     "qwen3-moe": Workload("qwen3-moe", 8192, 2048, 128, 8, "biased-topk", True, 128, True,
-                          "8192 x 2048, 128 experts top-8 with per-expert bias, expanded, alignment 128, zero_padding"),
+                          "8192 x 2048, 128 experts top-8 with per-expert bias, expanded, alignment 128, zero_padding, "
+                          "async_op with the consumer waiting on the completion event, combine returning the weights",
+                          async_op=True, combine_weights=True),
 }
 
 
