@@ -142,8 +142,10 @@ int nanoep_wait_counts(int64_t* host_counts, void* stream, double timeout_second
  * When slot_order is given for an expanded dispatch, the work is walked in that order instead and
  * neither of the other lookups is read for the payload.  slot_order_entries is A when the caller
  * knows it (the list may then be just its first A entries); a caller that enqueues the dispatch
- * before it has read the counts passes -1 with the full buffer, and the kernel takes A from the
- * buffer's last word.
+ * before it has read the counts passes a negative number with the full buffer, and the kernel takes
+ * A from the buffer's last word: -1 sizes the launch for the most entries the list can hold (T * K),
+ * -g (g > 1) for about g entries, which is cheaper when many choices are masked and correct whatever
+ * A turns out to be (workgroups then take several turns).
  * x / recv_x are bf16, 16-byte aligned, H % 8 == 0.  weights / recv_weights / recv_topk_idx may be
  * NULL (recv_topk_idx must be NULL when expanded).  num_cus is the reference's SM budget
  * (0 = whole device): it is range-checked against the device's compute-unit count and otherwise

@@ -192,13 +192,17 @@ __global__ void __launch_bounds__(1024) dispatch_ordered_kernel(const u32x4* __r
     NANOEP_FETCH_ARGS_4(copy_blocks, copy_per_xcd, parts, parts_magic);
     NANOEP_FETCH_ARGS_4(parts_shift, chunks_per_block, rows_per_block, vectors);
     NANOEP_FETCH_ARGS_4(chunks, topk_magic, topk_shift, live_count);
+    // workgroups per XCD the grid holds for the copy work: with the entry count on the device the live
+    // list may be shorter (the rest of the grid leaves at once) or longer (workgroups then take more
+    // than one turn, `grid_copy_per_xcd` list positions apart) than what the grid was sized for
+    const uint32_t grid_copy_per_xcd = copy_per_xcd;
     if (kDeviceCount) {
-        // The list length was not known when the grid was sized: shrink the walk to the entries in
-        // use, so that the per-XCD ranges split the real work and not its unused tail.
+        // The list length was not known when the grid was sized: the walk covers the entries in use,
+        // so that the per-XCD ranges split the real work and not an unused tail.
         // A word that cannot be a count (the layout did not run) walks nothing.
         const int64_t live = uniform_load(live_count);
         if (live != static_cast<int64_t>(entries)) {
-            entries = live >= 0 && live < static_cast<int64_t>(entries) ? static_cast<uint32_t>(live) : 0u;
+            entries = live >= 0 && live <= static_cast<int64_t>(source_limit) ? static_cast<uint32_t>(live) : 0u;
             copy_blocks = (rows_per_block == 1 ? entries : (entries + rows_per_block - 1) / rows_per_block) * parts;
             copy_per_xcd = (copy_blocks + kNumXcds - 1) / kNumXcds;
         }
@@ -211,70 +215,80 @@ __global__ void __launch_bounds__(1024) dispatch_ordered_kernel(const u32x4* __r
         // carry it at no measurable cost, while these extra workgroups cost 0.1 ns per assignment
         // (4096 x 7168: +1 us, 32768 x 7168: +25 us of 700).
         const uint32_t wave = threadIdx.z * chunks_per_block + threadIdx.y;
-        const uint32_t flat = ((blockIdx.x - payload_blocks) * (chunks_per_block * rows_per_block) + wave) * kWave + threadIdx.x;
-        if (flat >= entries)
-            return;
-        const int64_t entry = slot_order[flat];
-        const uint32_t source = static_cast<uint32_t>(entry);
-        const uint32_t out_row = static_cast<uint32_t>(static_cast<uint64_t>(entry) >> 32);
-        if (entry >= 0 && source < source_limit && out_row < out_rows)
-            recv_weights[out_row] = weights[source];
+        const uint32_t lanes = (gridDim.x - payload_blocks) * (chunks_per_block * rows_per_block) * kWave;
+        for (uint32_t flat = ((blockIdx.x - payload_blocks) * (chunks_per_block * rows_per_block) + wave) * kWave + threadIdx.x;
+             flat < entries; flat += lanes) {
+            const int64_t entry = slot_order[flat];
+            const uint32_t source = static_cast<uint32_t>(entry);
+            const uint32_t out_row = static_cast<uint32_t>(static_cast<uint64_t>(entry) >> 32);
+            if (entry >= 0 && source < source_limit && out_row < out_rows)
+                recv_weights[out_row] = weights[source];
+        }
         return;
     }
     const uint32_t index_in_xcd = blockIdx.x / kNumXcds;
-    if (kZeroFill && index_in_xcd >= copy_per_xcd) {
-        const uint32_t pad_index = index_in_xcd - copy_per_xcd;
+    // the XCD's workgroups up to `copy_turns` copy, the ones behind them clear gap rows
+    const uint32_t copy_turns = kDeviceCount && copy_per_xcd > grid_copy_per_xcd ? grid_copy_per_xcd : copy_per_xcd;
+    if (kZeroFill && index_in_xcd >= copy_turns) {
+        const uint32_t pad_index = index_in_xcd - copy_turns;
         const uint32_t pad_block = (blockIdx.x % kNumXcds) * pad_per_xcd + pad_index;
         if (pad_index < pad_per_xcd && pad_block < pad_blocks)
             zero_fill_gap_rows(pad_block, pad_per_expert, pad_groups_per_expert, chunks_per_block, rows_per_block,
                                expert_counts, expert_offsets, recv_x, recv_weights, out_rows, static_cast<int>(vectors));
         return;
     }
-    const uint32_t block = (blockIdx.x % kNumXcds) * copy_per_xcd + index_in_xcd;
-    uint32_t candidate, chunk;
-    if (kWholeRows) {
-        // one workgroup a row, as many wavefronts as the row has pieces: the block is the list entry
-        if (index_in_xcd >= copy_per_xcd || block >= entries)
-            return;
-        candidate = block;
-        chunk = __builtin_amdgcn_readfirstlane(threadIdx.y);
-    } else {
-        if (index_in_xcd >= copy_per_xcd || block >= copy_blocks)
-            return;
-        const uint32_t group = fast_divide(block, parts_magic, parts_shift);
-        const uint32_t part = block - group * parts;
-        candidate = group * rows_per_block + __builtin_amdgcn_readfirstlane(threadIdx.z);
-        chunk = part * chunks_per_block + __builtin_amdgcn_readfirstlane(threadIdx.y);
-        if (candidate >= entries || chunk >= chunks)
-            return;
-    }
-    const int64_t entry = uniform_load(slot_order + candidate);
-    const uint32_t source = static_cast<uint32_t>(entry);
-    const uint32_t out_row = static_cast<uint32_t>(static_cast<uint64_t>(entry) >> 32);
-    if (!(entry >= 0 && source < source_limit && out_row < out_rows))
+    if (index_in_xcd >= copy_turns)
         return;
-    const uint32_t token = fast_divide(source, topk_magic, topk_shift);
-    const uint32_t vector = chunk * (kSpan * kWave) + threadIdx.x;
-    // no workgroups behind the payload: the row's first wavefront moves its weight, fetched through
-    // the scalar path while the payload load is in flight
-    const bool carries_weight = chunk == 0 && recv_weights != nullptr && (kWholeRows || payload_blocks == gridDim.x);
-    float weight = 0.0f;
-    if (carries_weight)
-        weight = uniform_load(weights + source);
-    u32x4 data[kSpan];
+    // one turn, except where a device-side count found more entries than the grid was sized for
+    for (uint32_t at = index_in_xcd; at < copy_per_xcd; at += grid_copy_per_xcd) {
+        const uint32_t block = (blockIdx.x % kNumXcds) * copy_per_xcd + at;
+        uint32_t candidate, chunk;
+        if (kWholeRows) {
+            // one workgroup a row, as many wavefronts as the row has pieces: the block is the list entry
+            if (block >= entries)
+                break;
+            candidate = block;
+            chunk = __builtin_amdgcn_readfirstlane(threadIdx.y);
+        } else {
+            if (block >= copy_blocks)
+                break;
+            const uint32_t group = fast_divide(block, parts_magic, parts_shift);
+            const uint32_t part = block - group * parts;
+            candidate = group * rows_per_block + __builtin_amdgcn_readfirstlane(threadIdx.z);
+            chunk = part * chunks_per_block + __builtin_amdgcn_readfirstlane(threadIdx.y);
+        }
+        if (kWholeRows || (candidate < entries && chunk < chunks)) {
+            const int64_t entry = uniform_load(slot_order + candidate);
+            const uint32_t source = static_cast<uint32_t>(entry);
+            const uint32_t out_row = static_cast<uint32_t>(static_cast<uint64_t>(entry) >> 32);
+            if (entry >= 0 && source < source_limit && out_row < out_rows) {
+                const uint32_t token = fast_divide(source, topk_magic, topk_shift);
+                const uint32_t vector = chunk * (kSpan * kWave) + threadIdx.x;
+                // no workgroups behind the payload: the row's first wavefront moves its weight, fetched through
+                // the scalar path while the payload load is in flight
+                const bool carries_weight = chunk == 0 && recv_weights != nullptr && (kWholeRows || payload_blocks == gridDim.x);
+                float weight = 0.0f;
+                if (carries_weight)
+                    weight = uniform_load(weights + source);
+                u32x4 data[kSpan];
 #pragma unroll
-    for (int s = 0; s < kSpan; ++s) {
-        const uint32_t at = vector + s * kWave;
-        data[s] = x[static_cast<uint64_t>(token) * vectors + (at < vectors ? at : 0u)];
-    }
+                for (int s = 0; s < kSpan; ++s) {
+                    const uint32_t from = vector + s * kWave;
+                    data[s] = x[static_cast<uint64_t>(token) * vectors + (from < vectors ? from : 0u)];
+                }
 #pragma unroll
-    for (int s = 0; s < kSpan; ++s) {
-        const uint32_t at = vector + s * kWave;
-        if (at < vectors)
-            store_vec<true>(recv_x + static_cast<uint64_t>(out_row) * vectors + at, data[s]);
+                for (int s = 0; s < kSpan; ++s) {
+                    const uint32_t to = vector + s * kWave;
+                    if (to < vectors)
+                        store_vec<true>(recv_x + static_cast<uint64_t>(out_row) * vectors + to, data[s]);
+                }
+                if (carries_weight && threadIdx.x == 0)
+                    recv_weights[out_row] = weight;
+            }
+        }
+        if (!kDeviceCount)
+            break;
     }
-    if (carries_weight && threadIdx.x == 0)
-        recv_weights[out_row] = weight;
 }
 
 // Compact layout: receive row r holds source token src_token(r), in token order, so the dispatch is
@@ -387,10 +401,15 @@ int nanoep_dispatch(const void* x, const float* weights, const int32_t* recv_met
     const bool ordered = expand && slot_order != nullptr && order_bound > 0 && order_switch != 0;
     if (ordered && (slot_order_entries > order_bound || num_tokens * num_topk >= (int64_t{1} << 31)))
         return NANOEP_ERR_INVALID_ARGUMENT;
-    // a negative entry count defers to the count word the layout stored behind the list
+    // A negative entry count defers to the count word the layout stored behind the list.  -1 sizes the
+    // grid for the most entries the list can hold (T * K), -g for about g of them: workgroups beyond
+    // the live count leave at once, and where the live count is above g workgroups take several turns.
     const int64_t* live_count = ordered && slot_order_entries < 0 ? slot_order + order_bound : nullptr;
-    if (live_count != nullptr)
-        slot_order_entries = order_bound;
+    if (live_count != nullptr) {
+        const int64_t most = num_tokens * num_topk;
+        const int64_t expected = slot_order_entries == -1 ? most : -slot_order_entries;
+        slot_order_entries = expected < most ? expected : most;
+    }
 
     const int vectors = hidden / 8;
     int chunks = (vectors + kWave - 1) / kWave;

@@ -181,6 +181,16 @@ class PeerRuntime {
     bool prefers_exact_outputs() const { return prefers_exact_outputs_.load(); }
     void note_output_fill(bool bound_was_close) { prefers_exact_outputs_.store(!bound_was_close); }
 
+    // Share of the routing choices that were valid in the latest fresh expanded dispatch, in 1/1024
+    // (1024 before the first one).  A permute that is enqueued before the host knows the count sizes
+    // its launch for this share of T * K plus a margin instead of for all of it; any count is still
+    // handled, the workgroups of a launch that turns out too small take several turns.
+    int64_t valid_share_1024() const { return valid_share_1024_.load(); }
+    void note_valid_share(int64_t assignments, int64_t choices) {
+        if (choices > 0)
+            valid_share_1024_.store((assignments * 1024 + choices - 1) / choices);
+    }
+
     // The private handle tensors (slot table, slot-order list) of the latest few fresh expanded
     // dispatches.  A caller that keeps only the reference's seven handle tensors gets them back on
     // a replay of one of those handles: an entry is recognised by the identity of the handle's
@@ -336,6 +346,7 @@ class PeerRuntime {
     std::atomic<bool> counts_pending_{false};
     std::atomic<bool> counts_failed_{false};
     std::atomic<bool> prefers_exact_outputs_{false};
+    std::atomic<int64_t> valid_share_1024_{1024};
     std::deque<RememberedHandle> remembered_;  // newest first
     mutable int64_t private_recalls_ = 0;
     mutable std::mutex private_mutex_;
@@ -577,6 +588,12 @@ DispatchResult dispatch(PeerRuntime& runtime,
         int64_t order_entries = 0;
         const int64_t* order = slot_order_list(handle, tokens, topk, local_experts, expand, &order_entries);
         TORCH_CHECK(!count_on_device || order == nullptr || order_entries == -1, "slot-order buffer is incomplete");
+        if (count_on_device && order != nullptr) {
+            // the launch is sized for the share of valid choices the runtime saw last, plus 3 %
+            const int64_t share = runtime.valid_share_1024() + 31;
+            const int64_t expected = share >= 1024 ? tokens * topk : tokens * topk * share / 1024;
+            order_entries = expected >= tokens * topk || expected < 2 ? -1 : -expected;
+        }
         check_status(
             nanoep_dispatch(x.data_ptr(), weights.has_value() ? weights->data_ptr<float>() : nullptr, handle[0].data_ptr<int32_t>(),
                             handle[3].data_ptr<int64_t>(), slot_table(handle, tokens, topk, expand), order, order_entries,
@@ -707,6 +724,7 @@ DispatchResult dispatch(PeerRuntime& runtime,
         if (ordered) {
             TORCH_CHECK(counts[2] >= 0 && counts[2] <= slot_order.size(0), "assignment count exceeds the slot-order list");
             metadata[8] = slot_order.narrow(0, 0, counts[2]);  // replays walk the A assignments only
+            runtime.note_valid_share(counts[2], tokens * topk);
         }
         const int64_t used_rows = expand ? expanded_capacity : recv_count;
         const bool bound_is_close = used_rows * 5 >= row_bound * 4;  // the bound holds at most 1.25 x the rows in use
@@ -884,6 +902,7 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, module) {
         .def("private_recalls", &nanoep::PeerRuntime::private_recalls)
         .def("counts_failed", &nanoep::PeerRuntime::counts_failed)
         .def("prefers_exact_outputs", &nanoep::PeerRuntime::prefers_exact_outputs)
+        .def("valid_share_1024", &nanoep::PeerRuntime::valid_share_1024)
         .def("lose_counts_for_test", &nanoep::PeerRuntime::lose_counts_for_test)
         .def("close", &nanoep::PeerRuntime::close);
     py::class_<nanoep::CompletionEvent, std::shared_ptr<nanoep::CompletionEvent>>(module, "CompletionEvent")

@@ -169,7 +169,13 @@ def dispatch(x, weights, metadata, counts, num_local_experts, alignment, expand,
     recv_w = None if weights is None else new((rows,) if expand else (rows, topk), torch.float32)
     order = slot_order_of(metadata, use_order)
     # exact count A, or -1: the kernel reads A from the word behind the list
-    order_entries = 0 if order is None else (counts[2] if order_count == "exact" else -1)
+    # ... or -g: the same, with the launch sized for about g entries (order_count=("device", g))
+    if order is None:
+        order_entries = 0
+    elif order_count == "exact":
+        order_entries = counts[2]
+    else:
+        order_entries = -1 if order_count == "device" else -int(order_count[1])
     previous = os.environ.pop("NANOEP_DISPATCH_ORDER", None)
     previous_span = os.environ.pop("NANOEP_DISPATCH_SPAN", None)
     previous_rows = os.environ.pop("NANOEP_DISPATCH_WHOLE_ROWS", None)

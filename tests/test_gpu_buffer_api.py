@@ -241,6 +241,25 @@ def test_fresh_dispatch_never_holds_much_more_than_it_uses(device, expand):
             assert_same_bits(combined.x, want, "combine after the allocation order changed")
 
 
+def test_fresh_dispatch_launch_follows_the_share_of_valid_choices(device):
+    """The permute of a fresh dispatch is enqueued before the host knows how many choices are valid;
+    its launch is sized by the share the runtime saw last.  Batches whose share falls and rises
+    again (so that the launch is too large, then too small) all give the oracle's result."""
+    tokens, experts, topk, hidden = 600, 32, 8, 1024
+    full = cases.routing("random", tokens, experts, topk, seed=3)
+    x, w = cases.payload(tokens, hidden, seed=3), cases.gate_weights(tokens, topk)
+    generator = torch.Generator().manual_seed(11)
+    with Buffer(None, EPConfig(experts, topk, hidden, tokens)) as buffer:
+        assert buffer._runtime.valid_share_1024() == 1024
+        for masked in (0.0, 0.15, 0.15, 0.05, 0.0, 0.1):
+            idx = torch.where(torch.rand(tokens, topk, generator=generator) < masked, torch.full_like(full, -1), full)
+            result = buffer.dispatch(x.to(device), topk_idx=idx.to(device), weights=w.to(device), do_expand=True, zero_padding=True)
+            lay = assert_dispatch_result(result, x, idx, w, experts, True, 1, True)
+            assert not buffer._runtime.prefers_exact_outputs()
+            valid = int(lay.expert_counts.sum())
+            assert buffer._runtime.valid_share_1024() == -(-valid * 1024 // (tokens * topk))
+
+
 def test_headline_shapes_hold_at_most_a_quarter_more_than_they_use(device):
     """The DeepSeek-V3 batch with alignment 1 (at the bound) and 128 (exact order)."""
     from nanoep_amd import workloads

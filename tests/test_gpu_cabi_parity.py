@@ -382,6 +382,31 @@ def test_forced_window_sizes(device, monkeypatch, window, tokens):
     run_dispatch_combine(device, idx, 512, 24, 8, True, True, True, seed=5)
 
 
+@pytest.mark.parametrize(
+    "tokens,experts,topk,hidden,alignment",
+    [
+        pytest.param(700, 12, 4, 512, 16, id="general-kernel-with-zero-fill"),
+        pytest.param(900, 40, 8, 5120, 1, id="one-workgroup-a-row"),
+        pytest.param(3000, 16, 2, 256, 4, id="weights-in-workgroups-of-their-own"),
+    ],
+)
+def test_device_side_count_with_a_launch_sized_for_another_count(device, tokens, experts, topk, hidden, alignment):
+    """A dispatch enqueued before the host knows A may size its launch for an expected count: far
+    too small (workgroups take many turns), a little too small, exact, too large.  Same bytes."""
+    idx = cases.routing("dropout", tokens, experts, topk, seed=77)
+    x = cases.payload(tokens, hidden, seed=8).to(device)
+    w = cases.gate_weights(tokens, topk).to(device)
+    metadata, counts = cabi.layout(idx.to(device), experts, alignment, True, hidden=hidden)
+    assignments = counts[2]
+    want_x, _, want_w = cabi.dispatch(x, w, metadata, counts, experts, alignment, True, True, poison=POISON)
+    for expected in (2, 9, assignments // 3, assignments - 1, assignments, assignments + 1, tokens * topk, tokens * topk + 1000):
+        for span in (1, 2):
+            got_x, _, got_w = cabi.dispatch(x, w, metadata, counts, experts, alignment, True, True, poison=POISON,
+                                            order_count=("device", expected), span=span)
+            assert torch.equal(got_x.view(torch.int16), want_x.view(torch.int16)), (expected, span)
+            assert torch.equal(got_w.view(torch.int32), want_w.view(torch.int32)), (expected, span)
+
+
 @pytest.mark.parametrize("use_order", [True, False], ids=["slot-order", "token-order"])
 @pytest.mark.parametrize("bad", ["out-of-range", "duplicate"])
 def test_dispatch_behind_a_rejected_layout_stays_inside_its_bound(device, bad, use_order):
