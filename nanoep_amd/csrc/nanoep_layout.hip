@@ -377,36 +377,67 @@ __device__ __forceinline__ void assign_token_slots(int64_t token,
                                                    int64_t* __restrict__ dst_slots,
                                                    int32_t* __restrict__ token_slots,
                                                    int64_t* __restrict__ order) {
+    typedef int32_t i32x2 __attribute__((ext_vector_type(2)));
+    typedef int32_t i32x4 __attribute__((ext_vector_type(4)));
+    // a token's row of the slot table: wide stores where the row width keeps them aligned
+    const auto store_table_row = [&](const int32_t (&values)[kCap]) {
+        if (token_slots == nullptr)
+            return;
+        int32_t* row = token_slots + token * num_topk;
+        if ((num_topk & 3) == 0 && (reinterpret_cast<uintptr_t>(token_slots) & 15) == 0) {
+#pragma unroll
+            for (int k = 0; k < kCap; k += 4)
+                if (k < num_topk)
+                    *reinterpret_cast<i32x4*>(row + k) = i32x4{values[k], values[k + 1], values[k + 2], values[k + 3]};
+        } else {
+#pragma unroll
+            for (int k = 0; k < kCap; ++k)
+                if (k < num_topk)
+                    row[k] = values[k];
+        }
+    };
+    int32_t values[kCap];
+#pragma unroll
+    for (int k = 0; k < kCap; ++k)
+        values[k] = -1;
     if (row_in_block < 0) {
         dst_slots[token] = -1;
-        if (token_slots != nullptr)
-            for (int k = 0; k < num_topk; ++k)
-                token_slots[token * num_topk + k] = -1;
+        store_table_row(values);
         return;
     }
     const int64_t row = row_base + row_in_block;
     dst_slots[token] = row;
-    int32_t* out = recv_metadata + row * (num_topk + 2);
-    out[0] = 0;
-    out[1] = static_cast<int32_t>(token);
 #pragma unroll
     for (int k = 0; k < kCap; ++k) {
         if (k >= num_topk)
             break;
-        int32_t value = -1;
         if (packed[k] >= 0) {
             const int expert = packed[k] >> kRankBits;
             const int rank = packed[k] & kRankMask;
-            value = expand ? slot_base[expert] + rank : expert;
+            values[k] = expand ? slot_base[expert] + rank : expert;
             if (order != nullptr) {
                 const uint32_t source = static_cast<uint32_t>(token * num_topk + k);
-                order[order_base[expert] + rank] = (static_cast<int64_t>(value) << 32) | source;
+                order[order_base[expert] + rank] = (static_cast<int64_t>(values[k]) << 32) | source;
             }
         }
-        out[2 + k] = value;
-        if (token_slots != nullptr)
-            token_slots[token * num_topk + k] = value;
     }
+    // the receive row [0, token, K values]: pairs of words when K is even and the table 8-byte aligned (every row then is)
+    int32_t* out = recv_metadata + row * (num_topk + 2);
+    if ((num_topk & 1) == 0 && (reinterpret_cast<uintptr_t>(recv_metadata) & 7) == 0) {
+        *reinterpret_cast<i32x2*>(out) = i32x2{0, static_cast<int32_t>(token)};
+#pragma unroll
+        for (int k = 0; k < kCap; k += 2)
+            if (k < num_topk)
+                *reinterpret_cast<i32x2*>(out + 2 + k) = i32x2{values[k], values[k + 1]};
+    } else {
+        out[0] = 0;
+        out[1] = static_cast<int32_t>(token);
+#pragma unroll
+        for (int k = 0; k < kCap; ++k)
+            if (k < num_topk)
+                out[2 + k] = values[k];
+    }
+    store_table_row(values);
 }
 
 __device__ __forceinline__ int64_t wave_inclusive_scan(int64_t value) {
@@ -482,6 +513,11 @@ __device__ __forceinline__ void layout_assign_block(const int32_t* block_counts,
     for (int k = 0; k < kCap; ++k)
         packed[k] = live ? packed_rank[token * num_topk + (k < num_topk ? k : 0)] : -1;
 
+    // workgroup 0 gathers the blocks' routing status; the first word a thread is fetched here, used
+    // behind the histogram loads, so that its round trip is not a second one behind theirs
+    int first_status = 0;
+    if (kFusedScan && block == 0 && tid < num_blocks)
+        first_status = block_status[tid];
     if (kFusedScan) {
         for (int i = tid; i < 4 * rows; i += threads)
             assign_lds[i] = 0;
@@ -508,22 +544,43 @@ __device__ __forceinline__ void layout_assign_block(const int32_t* block_counts,
             const bool active = segment < segments && column < rows;
             const bool active_second = segment < segments && second < rows;
             int total[2] = {0, 0}, before[2] = {0, 0}, own[2] = {0, 0}, window[2] = {0, 0}, earlier[2] = {0, 0};
+            // Histogram words are fetched sixteen blocks at a time, all loads of a batch in flight
+            // together whatever the number of blocks (positions past the last block re-read it and
+            // count nothing), and only a wavefront that holds a second column fetches it.
+            const bool wave_has_second = column - (tid & (kWave - 1)) + columns_per_pass < rows;
+            const int64_t second_or_first = active_second ? second : column;
             if (active) {
-#pragma unroll 16
-                for (int b = begin; b < end; ++b) {
-                    const int count = block_counts[static_cast<int64_t>(b) * rows + column];
-                    const int count_second = active_second ? block_counts[static_cast<int64_t>(b) * rows + second] : 0;
-                    const bool in_window = b >= window_first && b < window_end;
-                    total[0] += count;
-                    total[1] += count_second;
-                    before[0] += b < block ? count : 0;
-                    before[1] += b < block ? count_second : 0;
-                    own[0] = b == block ? count : own[0];
-                    own[1] = b == block ? count_second : own[1];
-                    window[0] += in_window ? count : 0;
-                    window[1] += in_window ? count_second : 0;
-                    earlier[0] += in_window && b < block ? count : 0;
-                    earlier[1] += in_window && b < block ? count_second : 0;
+                for (int b0 = begin; b0 < end; b0 += 16) {
+                    int fetched[16], fetched_second[16];
+#pragma unroll
+                    for (int j = 0; j < 16; ++j) {
+                        const int64_t b = b0 + j < end ? b0 + j : end - 1;
+                        fetched[j] = block_counts[b * rows + column];
+                    }
+                    if (wave_has_second) {
+#pragma unroll
+                        for (int j = 0; j < 16; ++j) {
+                            const int64_t b = b0 + j < end ? b0 + j : end - 1;
+                            fetched_second[j] = block_counts[b * rows + second_or_first];
+                        }
+                    }
+#pragma unroll
+                    for (int j = 0; j < 16; ++j) {
+                        const int b = b0 + j;
+                        const int count = b < end ? fetched[j] : 0;
+                        const int count_second = wave_has_second && active_second && b < end ? fetched_second[j] : 0;
+                        const bool in_window = b >= window_first && b < window_end;
+                        total[0] += count;
+                        total[1] += count_second;
+                        before[0] += b < block ? count : 0;
+                        before[1] += b < block ? count_second : 0;
+                        own[0] = b == block ? count : own[0];
+                        own[1] = b == block ? count_second : own[1];
+                        window[0] += in_window ? count : 0;
+                        window[1] += in_window ? count_second : 0;
+                        earlier[0] += in_window && b < block ? count : 0;
+                        earlier[1] += in_window && b < block ? count_second : 0;
+                    }
                 }
             }
             for (int i = 0; i < 2; ++i) {
@@ -543,13 +600,19 @@ __device__ __forceinline__ void layout_assign_block(const int32_t* block_counts,
                     if (earlier[i] != 0)
                         atomicAdd(&window_before[at], earlier[i]);
                 }
-                if (at < local_experts && own[i] != 0)
-                    atomicAdd(&own_assignments, own[i]);
             }
+            // this block's own assignments: one LDS atomic a wavefront (256 lanes adding to one word
+            // one after the other were most of a microsecond in front of the barrier)
+            int own_sum = (active && column < local_experts ? own[0] : 0) + (active_second && second < local_experts ? own[1] : 0);
+#pragma unroll
+            for (int distance = kWave / 2; distance > 0; distance /= 2)
+                own_sum += __shfl_xor(own_sum, distance, kWave);
+            if ((tid & (kWave - 1)) == 0 && own_sum != 0)
+                atomicAdd(&own_assignments, own_sum);
         }
         if (block == 0) {
-            int bad = 0;
-            for (int b = tid; b < num_blocks; b += threads)
+            int bad = first_status;
+            for (int b = tid + threads; b < num_blocks; b += threads)
                 bad |= block_status[b];
             if (bad)
                 atomicOr(&status_bits, bad);
@@ -635,8 +698,12 @@ __device__ __forceinline__ void layout_assign_block(const int32_t* block_counts,
         order_base[e] = running_own + window_before[e];  // behind the expert's entries of the window's earlier blocks
         running_own += in_window;
     }
+    const int64_t received = kFusedScan ? column_total[local_experts] : 0;
+    __syncthreads();
     if (kFusedScan && block == 0 && tid == 0) {
-        const int64_t received = column_total[local_experts];
+        // Behind the workgroup's last barrier: the store to host memory and the wait that orders it
+        // hold up this one wavefront's share of the token writes below, not the whole workgroup
+        // (in front of the barrier they were a microsecond of the kernel).
         expert_offsets[local_experts] = capacity;
         send_counts[0] = received;
         recv_rank_prefix[0] = received;
@@ -646,7 +713,6 @@ __device__ __forceinline__ void layout_assign_block(const int32_t* block_counts,
         __threadfence_system();
         __hip_atomic_store(&host_counts[0], received, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_SYSTEM);
     }
-    __syncthreads();
     // The list is dense: a window's part starts where the assignments of the blocks before the window
     // end.  Every block also clears as many entries of the unused tail as it has masked choices.
     int64_t* order = nullptr;
