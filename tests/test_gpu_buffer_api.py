@@ -250,14 +250,14 @@ def test_fresh_dispatch_launch_follows_the_share_of_valid_choices(device):
     x, w = cases.payload(tokens, hidden, seed=3), cases.gate_weights(tokens, topk)
     generator = torch.Generator().manual_seed(11)
     with Buffer(None, EPConfig(experts, topk, hidden, tokens)) as buffer:
-        assert buffer._runtime.valid_share_1024() == 1024
+        assert buffer._runtime.valid_share_65536() == 65536
         for masked in (0.0, 0.15, 0.15, 0.05, 0.0, 0.1):
             idx = torch.where(torch.rand(tokens, topk, generator=generator) < masked, torch.full_like(full, -1), full)
             result = buffer.dispatch(x.to(device), topk_idx=idx.to(device), weights=w.to(device), do_expand=True, zero_padding=True)
             lay = assert_dispatch_result(result, x, idx, w, experts, True, 1, True)
             assert not buffer._runtime.prefers_exact_outputs()
             valid = int(lay.expert_counts.sum())
-            assert buffer._runtime.valid_share_1024() == -(-valid * 1024 // (tokens * topk))
+            assert buffer._runtime.valid_share_65536() == -(-valid * 65536 // (tokens * topk))
 
 
 def test_headline_shapes_hold_at_most_a_quarter_more_than_they_use(device):
