@@ -344,7 +344,7 @@ def test_a_foreign_seven_tensor_handle_is_followed_as_written(device):
     """A valid handle in another row and slot order than this library's own (here: receive rows and
     slots in reverse token order, as a caller may build them) is honoured by the host extension
     whatever the payload size: every row lands where the handle's recv_metadata says, and combine
-    brings it back.  (16 MiB payload: the size from which an earlier version rebuilt its own order.)"""
+    brings it back.  (A 16 MiB payload: nothing about the size of the batch changes that.)"""
     tokens, experts, topk, hidden, alignment = 2048, 16, 4, 4096, 4
     idx = cases.routing("dropout", tokens, experts, topk, seed=3)
     x, w = cases.payload(tokens, hidden, seed=6), cases.gate_weights(tokens, topk)
