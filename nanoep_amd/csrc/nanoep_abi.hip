@@ -1,10 +1,43 @@
 // Version, status strings, window layout, profiler calibration copy.
 
+#include <unistd.h>
+
 #include "nanoep_device.h"
+
+extern char** environ;
 
 namespace nanoep {
 
 thread_local hipError_t g_last_hip_error = hipSuccess;
+thread_local Tuning g_tuning;
+
+void refresh_tuning() {
+    Tuning fresh;
+    struct Switch {
+        const char* name;  // behind the NANOEP_ prefix
+        int* value;
+    };
+    const Switch switches[] = {
+        {"CHUNKS_PER_BLOCK", &fresh.chunks_per_block}, {"ROWS_PER_BLOCK", &fresh.rows_per_block},
+        {"DISPATCH_ORDER", &fresh.dispatch_order},     {"DISPATCH_SPAN", &fresh.dispatch_span},
+        {"DISPATCH_SIDE", &fresh.dispatch_side},       {"DISPATCH_WHOLE_ROWS", &fresh.dispatch_whole_rows},
+        {"LAYOUT_LAUNCHES", &fresh.layout_launches},   {"WINDOW_TOKENS", &fresh.window_tokens},
+    };
+    if (environ != nullptr) {
+        for (char** entry = environ; *entry != nullptr; ++entry) {
+            const char* text = *entry;
+            if (text[0] != 'N' || std::strncmp(text, "NANOEP_", 7) != 0)
+                continue;
+            for (const Switch& item : switches) {
+                const size_t length = std::strlen(item.name);
+                // NANOEP_<NAME>=<number>; an empty value leaves the default
+                if (std::strncmp(text + 7, item.name, length) == 0 && text[7 + length] == '=' && text[8 + length] != '\0')
+                    *item.value = std::atoi(text + 8 + length);
+            }
+        }
+    }
+    g_tuning = fresh;
+}
 
 namespace {
 

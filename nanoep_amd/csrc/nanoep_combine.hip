@@ -306,6 +306,7 @@ int nanoep_combine(const void* y, const float* weights, const void* bias, const 
                    const int64_t* dst_slots, const int32_t* token_slots, int64_t recv_count, int64_t y_rows,
                    int64_t num_tokens, int hidden, int num_topk, int expand, int multiple_reduction, void* out_x,
                    float* out_weights, int num_cus, void* stream_handle) {
+    refresh_tuning();
     if (hidden <= 0 || hidden % 8 != 0 || num_topk <= 0 || num_topk > kMaxTopk)
         return NANOEP_ERR_INVALID_ARGUMENT;
     if (recv_count < 0 || num_tokens < 0 || recv_count > num_tokens || num_tokens > INT32_MAX || y_rows < 0 ||

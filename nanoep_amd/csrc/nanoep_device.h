@@ -70,12 +70,24 @@ extern thread_local hipError_t g_last_hip_error;
 
 inline size_t align_up(size_t value, size_t alignment) { return (value + alignment - 1) / alignment * alignment; }
 
-inline int env_int(const char* name, int fallback) {
-    const char* text = std::getenv(name);
-    if (text == nullptr || *text == '\0')
-        return fallback;
-    return std::atoi(text);
-}
+// Tuning switches of the library, read from the environment (NANOEP_<NAME>; tests and sweeps flip
+// them between calls).  Every entry point of the C ABI reads them afresh with one walk over the
+// environment (refresh_tuning) into this per-thread record; the code below the entry points only
+// looks at the record.  (A getenv per switch and use walked the whole environment a dozen to two
+// dozen times a call, microseconds on the host path of a fresh dispatch.)
+struct Tuning {
+    int chunks_per_block = 0;       // NANOEP_CHUNKS_PER_BLOCK: wavefronts along a row in a workgroup, 0 = by shape
+    int rows_per_block = 0;         // NANOEP_ROWS_PER_BLOCK: rows a workgroup, 0 = by shape
+    int dispatch_order = -1;        // NANOEP_DISPATCH_ORDER: 0 forces the token-order walk
+    int dispatch_span = 0;          // NANOEP_DISPATCH_SPAN: 1 | 2 chunks a wavefront of the slot-order walk, 0 = by size
+    int dispatch_side = -1;         // NANOEP_DISPATCH_SIDE: 0 | 1 weights of that walk in workgroups of their own
+    int dispatch_whole_rows = -1;   // NANOEP_DISPATCH_WHOLE_ROWS: 0 | 1 the kernel variant for one workgroup a list entry
+    int layout_launches = 0;        // NANOEP_LAYOUT_LAUNCHES: 2 | 3 forces the layout plan
+    int window_tokens = 0;          // NANOEP_WINDOW_TOKENS: forces the window of the slot-order list
+};
+
+extern thread_local Tuning g_tuning;  // defined in nanoep_abi.hip
+void refresh_tuning();                // defined in nanoep_abi.hip
 
 // Calls f with the smallest compile-time bound in {4, 8, 16, 32} that covers num_topk.
 template <typename F>
@@ -165,7 +177,7 @@ enum WalkShape {
 
 inline RowBlocking pick_row_blocking(int chunks, WalkShape shape) {
     RowBlocking blocking{};
-    int per_block = env_int("NANOEP_CHUNKS_PER_BLOCK", 0);
+    int per_block = g_tuning.chunks_per_block;
     if (per_block < 1 || per_block > kMaxWavesPerBlock) {
         per_block = kDefaultChunksPerBlock;
         if (shape == kSlotOrderWalk) {
@@ -187,7 +199,7 @@ inline RowBlocking pick_row_blocking(int chunks, WalkShape shape) {
     blocking.parts = static_cast<unsigned>((chunks + per_block - 1) / per_block);
     int rows = 1;
     if (blocking.parts == 1) {
-        rows = env_int("NANOEP_ROWS_PER_BLOCK", 0);
+        rows = g_tuning.rows_per_block;
         if (rows < 1 || rows * per_block > kMaxWavesPerBlock)
             rows = per_block >= 4 ? 1 : 4 / per_block;
     }

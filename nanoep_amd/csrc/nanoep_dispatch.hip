@@ -369,6 +369,7 @@ int nanoep_dispatch(const void* x, const float* weights, const int32_t* recv_met
                     int64_t recv_count, int64_t expanded_capacity, int64_t num_tokens, int hidden, int num_topk,
                     int64_t num_local_experts, int64_t alignment, int expand, int zero_padding, void* recv_x,
                     int64_t* recv_topk_idx, float* recv_weights, int num_cus, void* stream_handle) {
+    refresh_tuning();
     if (hidden <= 0 || hidden % 8 != 0 || num_topk <= 0 || num_topk > kMaxTopk || num_local_experts <= 0 || alignment <= 0)
         return NANOEP_ERR_INVALID_ARGUMENT;
     if (recv_count < 0 || num_tokens < 0 || recv_count > num_tokens || num_tokens > INT32_MAX || expanded_capacity < 0 ||
@@ -397,7 +398,7 @@ int nanoep_dispatch(const void* x, const float* weights, const int32_t* recv_met
     // The walk is used whenever the handle carries the list.  With cache-resident sources and fewer
     // than eight token blocks the token-order walk is up to 15 % faster, but with cold sources it is
     // 25-60 % slower at every size, so the list decides.
-    const int order_switch = env_int("NANOEP_DISPATCH_ORDER", -1);  // 0 forces the token-order walk
+    const int order_switch = g_tuning.dispatch_order;  // 0 forces the token-order walk
     const bool ordered = expand && slot_order != nullptr && order_bound > 0 && order_switch != 0;
     if (ordered && (slot_order_entries > order_bound || num_tokens * num_topk >= (int64_t{1} << 31)))
         return NANOEP_ERR_INVALID_ARGUMENT;
@@ -422,7 +423,7 @@ int nanoep_dispatch(const void* x, const float* weights, const int32_t* recv_met
     if (ordered) {
         const bool short_rows = chunks == 2;
         span = short_rows || static_cast<int64_t>(num_tokens) * hidden * 2 > kLastLevelCacheBytes ? 2 : 1;
-        const int forced_span = env_int("NANOEP_DISPATCH_SPAN", 0);
+        const int forced_span = g_tuning.dispatch_span;
         if (forced_span == 1 || forced_span == 2)
             span = forced_span;
         chunks = (chunks + span - 1) / span;
@@ -448,7 +449,7 @@ int nanoep_dispatch(const void* x, const float* weights, const int32_t* recv_met
     // slot-order walk over rows of one or two chunks: one lane per list entry moves the weights, in
     // workgroups at the end of the grid (+3-4 %); longer rows carry the weight on their first wavefront
     // (8192 x 2048 top-8 with alignment 128: 56.0 against 57.0 us).  NANOEP_DISPATCH_SIDE=0|1 overrides.
-    const int side_switch = env_int("NANOEP_DISPATCH_SIDE", -1);
+    const int side_switch = g_tuning.dispatch_side;
     const bool side_weights = ordered && recv_weights != nullptr && (side_switch < 0 ? row_chunks <= 2 : side_switch != 0);
     const int64_t side_lanes = side_weights ? copy_candidates : 0;
     const int64_t side_blocks = (side_lanes + kWave * waves - 1) / (kWave * waves);
@@ -490,7 +491,7 @@ int nanoep_dispatch(const void* x, const float* weights, const int32_t* recv_met
         // division to find its entry and piece (4096 x 7168: 81.5 -> 80.4 us, with alignment 128
         // 100.6 -> 96.9 us, 8192 x 5120: 123.1 -> 120.3 us).  Rows of four pieces are better off
         // with the general path (8192 x 2048 with cache-resident sources: 37.6 against 38.3 us).
-        const int whole_rows_switch = env_int("NANOEP_DISPATCH_WHOLE_ROWS", -1);
+        const int whole_rows_switch = g_tuning.dispatch_whole_rows;
         const bool whole_rows = blocking.parts == 1 && blocking.rows_per_block == 1 &&
                                 blocking.chunks_per_block == static_cast<unsigned>(chunks) && side_blocks == 0 &&
                                 (whole_rows_switch < 0 ? chunks >= 5 : whole_rows_switch != 0);

@@ -36,7 +36,7 @@ constexpr int kMaxWindowTokens = 1024;
 //    to get there.
 int layout_window_tokens(int64_t tokens_total, int hidden) {
     // NANOEP_WINDOW_TOKENS forces a window: any multiple of 32 up to 256 (one layout workgroup), or 512 / 1024
-    const int forced = env_int("NANOEP_WINDOW_TOKENS", 0);
+    const int forced = g_tuning.window_tokens;
     if (forced >= 32 && forced % 32 == 0 && (forced <= 256 || forced == 512 || forced == 1024) && tokens_total > 256)
         return forced;
     int window = 256;
@@ -81,7 +81,7 @@ bool layout_uses_fused_scan(int64_t tokens_total, int64_t local_experts, int hid
     if (per_block == 0 || tokens_total == 0)
         return false;
     const int64_t blocks = (tokens_total + per_block - 1) / per_block;
-    const int forced = env_int("NANOEP_LAYOUT_LAUNCHES", 0);
+    const int forced = g_tuning.layout_launches;
     if (forced == 3)
         return false;
     return forced == 2 || blocks <= kFusedScanMaxBlocks;
@@ -849,7 +849,7 @@ int enqueue_layout(const int64_t* topk_idx, int64_t num_tokens, int num_topk, in
     // tokens: 159 against 198 us).  Beyond, the blocks^2 loads lose (2^20 tokens, 8 experts: 124
     // against 67 us) and a third launch does the scan once.
     const bool fused_scan = layout_uses_fused_scan(num_tokens, num_local_experts, hidden);
-    const int forced_launches = env_int("NANOEP_LAYOUT_LAUNCHES", 0);
+    const int forced_launches = g_tuning.layout_launches;
     const int window_blocks = layout_window_blocks(num_tokens, num_local_experts, hidden, fused_scan);
     hipError_t launch_status = hipSuccess;
     with_topk_cap(num_topk, [&](auto cap) {
@@ -929,12 +929,14 @@ using namespace nanoep;
 extern "C" {
 
 size_t nanoep_layout_workspace_bytes(int64_t num_tokens, int num_topk, int64_t num_local_experts) {
+    refresh_tuning();
     if (num_tokens < 0 || num_topk <= 0 || num_local_experts <= 0)
         return 0;
     return carve_layout_workspace(nullptr, num_tokens, num_topk, num_local_experts).bytes;
 }
 
 int nanoep_layout_block_tokens(int64_t num_tokens, int64_t num_local_experts, int hidden) {
+    refresh_tuning();
     if (num_local_experts <= 0 || num_tokens < 0 || hidden < 0)
         return 0;
     // tokens the slot-order list is ordered by: the layout workgroup's tokens times the blocks of a window
@@ -944,6 +946,7 @@ int nanoep_layout_block_tokens(int64_t num_tokens, int64_t num_local_experts, in
 }
 
 int64_t nanoep_slot_order_entries(int64_t num_tokens, int num_topk, int64_t num_local_experts) {
+    refresh_tuning();
     if (num_tokens < 0 || num_topk <= 0 || num_local_experts <= 0)
         return 0;
     if (layout_smallest_block(num_tokens, num_local_experts) == 0 || num_tokens == 0)
@@ -957,6 +960,7 @@ int nanoep_layout(const int64_t* topk_idx, int64_t num_tokens, int num_topk, int
                   int64_t* expert_offsets, int64_t* dst_slots, int64_t* send_counts, int64_t* topk_snapshot,
                   int64_t* recv_rank_prefix, int32_t* token_slots, int64_t* slot_order, void* workspace,
                   size_t workspace_bytes, int64_t* host_counts, void* stream_handle) {
+    refresh_tuning();
     const int status = check_layout_arguments(topk_idx, num_tokens, num_topk, num_local_experts, alignment, expand, hidden,
                                               recv_metadata, expert_counts, expert_offsets, dst_slots, send_counts, topk_snapshot,
                                               recv_rank_prefix, slot_order, host_counts);
@@ -977,6 +981,7 @@ int nanoep_layout_static(const int64_t* topk_idx, int64_t num_tokens, int num_to
                          int64_t* expert_offsets, int64_t* dst_slots, int64_t* send_counts, int64_t* topk_snapshot,
                          int64_t* recv_rank_prefix, int32_t* token_slots, int64_t* slot_order, int64_t* host_counts,
                          void* stream_handle) {
+    refresh_tuning();
     const int status = check_layout_arguments(topk_idx, num_tokens, num_topk, num_local_experts, alignment, expand, hidden,
                                               recv_metadata, expert_counts, expert_offsets, dst_slots, send_counts, topk_snapshot,
                                               recv_rank_prefix, slot_order, host_counts);

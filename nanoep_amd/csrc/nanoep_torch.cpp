@@ -575,7 +575,8 @@ DispatchResult dispatch(PeerRuntime& runtime,
     const auto allocate_outputs = [&](int64_t x_rows, int64_t n_rows) {
         allocate_for_consumer([&] {
             out_x = torch::empty({x_rows, hidden}, x.options());
-            out_indices = expand ? torch::empty({0}, routing.options()) : torch::empty({n_rows, topk}, routing.options());
+            if (!expand)
+                out_indices = torch::empty({n_rows, topk}, routing.options());
             out_weights = !weights.has_value() ? torch::empty({0}, float_options)
                           : expand            ? torch::empty({x_rows}, float_options)
                                               : torch::empty({n_rows, topk}, float_options);
@@ -636,30 +637,31 @@ DispatchResult dispatch(PeerRuntime& runtime,
         torch::Tensor recv_metadata, expert_counts, expert_offsets, dst_slots, send_counts, snapshot, prefix, token_slots, slot_order;
         // the slot-order list packs token * K + k into 32 bits
         const bool ordered = expand && tokens * topk < (int64_t{1} << 31);
-        // The handle tensors of one call are views of two arenas (one per element type), and the
+        // The handle tensors of one call are views of one allocation (the int64 ones, then the int32 ones), and the
         // views are made after the layout has been enqueued: on a path whose small-batch cost is
         // host latency, the GPU starts three allocator round trips after the call instead of ten
         // and works while the rest of the bookkeeping is done.
         const int64_t order_entries = ordered ? nanoep_slot_order_entries(tokens, static_cast<int>(topk), local_experts) : 0;
         const int64_t count64 = 2 * local_experts + 3 + tokens + tokens * topk + order_entries;
-        const int64_t count32 = tokens * (topk + 2) + (expand ? tokens * topk : 0);
+        const int64_t at_table = (tokens * (topk + 2) + 3) / 4 * 4;  // the slot table starts 16-byte aligned
+        const int64_t count32 = at_table + (expand ? tokens * topk : 0);
         const size_t workspace_bytes = nanoep_layout_workspace_bytes(tokens, static_cast<int>(topk), local_experts);
         TORCH_CHECK(workspace_bytes > 0, "unsupported routing geometry for the layout kernels");
         TORCH_CHECK(nanoep_layout_block_tokens(tokens, local_experts, static_cast<int>(hidden)) > 0,
                     "the layout kernels take at most 3839 local experts, got ", local_experts);
+        // one allocation: the int64 tensors first, the int32 ones behind them as a view of the same storage
         torch::Tensor arena64, arena32;
         allocate_for_consumer([&] {
-            arena64 = torch::empty({count64}, int64_options);
-            arena32 = torch::empty({count32 > 0 ? count32 : 1}, int64_options.dtype(torch::kInt32));
+            arena64 = torch::empty({count64 + (count32 + 1) / 2}, int64_options);
             return 0;
         });
         auto workspace = torch::empty({static_cast<int64_t>(workspace_bytes)}, int64_options.dtype(torch::kUInt8));
         // arena64: expert_counts [L] | expert_offsets [L+1] | send_counts [1] | recv_rank_prefix [1] |
         //          dst_slots [T] | topk snapshot [T*K] | slot_order;   arena32: recv_metadata [T*(K+2)] | token_slots [T*K]
         const int64_t at_offsets = local_experts, at_send = 2 * local_experts + 1, at_prefix = at_send + 1, at_dst = at_prefix + 1;
-        const int64_t at_snapshot = at_dst + tokens, at_order = at_snapshot + tokens * topk, at_table = tokens * (topk + 2);
+        const int64_t at_snapshot = at_dst + tokens, at_order = at_snapshot + tokens * topk;
         int64_t* base64 = arena64.data_ptr<int64_t>();
-        int32_t* base32 = arena32.data_ptr<int32_t>();
+        int32_t* base32 = reinterpret_cast<int32_t*>(base64 + count64);
 
         // From here until the counts have been read this call owns the runtime's mailbox; a fresh
         // dispatch of another thread on the same runtime waits here for its turn.
@@ -672,6 +674,7 @@ DispatchResult dispatch(PeerRuntime& runtime,
         if (layout_status != NANOEP_OK && layout_status != NANOEP_ERR_HIP)
             turn.abandon();  // refused before anything was enqueued
         check_status(layout_status, "layout");
+        arena32 = arena64.narrow(0, count64, (count32 + 1) / 2).view(torch::kInt32);
         expert_counts = arena64.narrow(0, 0, local_experts);
         expert_offsets = arena64.narrow(0, at_offsets, local_experts + 1);
         send_counts = arena64.narrow(0, at_send, 1);
@@ -747,6 +750,8 @@ DispatchResult dispatch(PeerRuntime& runtime,
             runtime.remember_private(metadata, alignment);
     }
 
+    if (expand)
+        out_indices = torch::empty({0}, routing.options());  // absent at this boundary; made off the path to the launch
     std::vector<torch::Tensor> outputs{out_x, out_indices, out_weights};
     std::shared_ptr<CompletionEvent> event;
     if (async_op) {
