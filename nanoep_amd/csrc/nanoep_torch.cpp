@@ -583,25 +583,41 @@ DispatchResult dispatch(PeerRuntime& runtime,
             return 0;
         });
     };
-    // count_on_device: the handle carries the whole slot-order buffer and the number of entries in
-    // use is not known on the host yet, so the kernel reads it from the buffer's last word
-    const auto launch_permute = [&](const std::vector<torch::Tensor>& handle, int64_t received, int64_t capacity,
-                                    bool count_on_device = false) {
+    // What the permute reads of a handle, as plain pointers.  order_entries: A, or -1 for "the whole
+    // slot-order buffer is there and the kernel finds A in its last word".
+    struct HandleView {
+        const int32_t* recv_metadata = nullptr;
+        const int64_t* dst_slots = nullptr;
+        const int32_t* token_slots = nullptr;
+        const int64_t* slot_order = nullptr;
         int64_t order_entries = 0;
-        const int64_t* order = slot_order_list(handle, tokens, topk, local_experts, expand, &order_entries);
-        TORCH_CHECK(!count_on_device || order == nullptr || order_entries == -1, "slot-order buffer is incomplete");
-        if (count_on_device && order != nullptr) {
+        const int64_t* expert_counts = nullptr;
+        const int64_t* expert_offsets = nullptr;
+    };
+    const auto view_of = [&](const std::vector<torch::Tensor>& handle) {
+        HandleView view;
+        view.recv_metadata = handle[0].data_ptr<int32_t>();
+        view.dst_slots = handle[3].data_ptr<int64_t>();
+        view.token_slots = slot_table(handle, tokens, topk, expand);
+        view.slot_order = slot_order_list(handle, tokens, topk, local_experts, expand, &view.order_entries);
+        view.expert_counts = handle[1].data_ptr<int64_t>();
+        view.expert_offsets = handle[2].data_ptr<int64_t>();
+        return view;
+    };
+    // count_on_device: the number of list entries in use is not known on the host yet
+    const auto launch_permute = [&](HandleView handle, int64_t received, int64_t capacity, bool count_on_device = false) {
+        TORCH_CHECK(!count_on_device || handle.slot_order == nullptr || handle.order_entries == -1, "slot-order buffer is incomplete");
+        if (count_on_device && handle.slot_order != nullptr) {
             // the launch is sized for the share of valid choices the runtime saw last, plus 0.5 %
             const int64_t share = runtime.valid_share_65536() + 328;
             const int64_t expected = share >= 65536 ? tokens * topk : tokens * topk * share / 65536;
-            order_entries = expected >= tokens * topk || expected < 2 ? -1 : -expected;
+            handle.order_entries = expected >= tokens * topk || expected < 2 ? -1 : -expected;
         }
         check_status(
-            nanoep_dispatch(x.data_ptr(), weights.has_value() ? weights->data_ptr<float>() : nullptr, handle[0].data_ptr<int32_t>(),
-                            handle[3].data_ptr<int64_t>(), slot_table(handle, tokens, topk, expand), order, order_entries,
-                            handle[1].data_ptr<int64_t>(), handle[2].data_ptr<int64_t>(), received, capacity, tokens, static_cast<int>(hidden),
-                            static_cast<int>(topk), local_experts, alignment, expand ? 1 : 0, zero_padding ? 1 : 0, out_x.data_ptr(),
-                            expand ? nullptr : out_indices.data_ptr<int64_t>(),
+            nanoep_dispatch(x.data_ptr(), weights.has_value() ? weights->data_ptr<float>() : nullptr, handle.recv_metadata, handle.dst_slots,
+                            handle.token_slots, handle.slot_order, handle.order_entries, handle.expert_counts, handle.expert_offsets,
+                            received, capacity, tokens, static_cast<int>(hidden), static_cast<int>(topk), local_experts, alignment,
+                            expand ? 1 : 0, zero_padding ? 1 : 0, out_x.data_ptr(), expand ? nullptr : out_indices.data_ptr<int64_t>(),
                             weights.has_value() ? out_weights.data_ptr<float>() : nullptr, cu_budget, comm.stream()),
             "dispatch");
     };
@@ -627,7 +643,7 @@ DispatchResult dispatch(PeerRuntime& runtime,
         if (expand && recv_count > 0 && env_switch("NANOEP_RECALL_ORDER") != 0)
             runtime.recall_private(metadata, alignment);
         if (recv_count > 0)
-            launch_permute(metadata, recv_count, expanded_capacity);
+            launch_permute(view_of(metadata), recv_count, expanded_capacity);
     } else {
         hipStreamCaptureStatus capture = hipStreamCaptureStatusNone;
         check_hip(hipStreamIsCapturing(comm.stream(), &capture), "hipStreamIsCapturing");
@@ -674,23 +690,6 @@ DispatchResult dispatch(PeerRuntime& runtime,
         if (layout_status != NANOEP_OK && layout_status != NANOEP_ERR_HIP)
             turn.abandon();  // refused before anything was enqueued
         check_status(layout_status, "layout");
-        arena32 = arena64.narrow(0, count64, (count32 + 1) / 2).view(torch::kInt32);
-        expert_counts = arena64.narrow(0, 0, local_experts);
-        expert_offsets = arena64.narrow(0, at_offsets, local_experts + 1);
-        send_counts = arena64.narrow(0, at_send, 1);
-        prefix = arena64.narrow(0, at_prefix, 1);
-        dst_slots = arena64.narrow(0, at_dst, tokens).view({tokens, 1});
-        snapshot = arena64.narrow(0, at_snapshot, tokens * topk).view({tokens, topk});
-        recv_metadata = arena32.narrow(0, 0, tokens * (topk + 2)).view({tokens, topk + 2});
-        metadata = {recv_metadata, expert_counts, expert_offsets, dst_slots, send_counts, snapshot, prefix};
-        if (expand) {
-            token_slots = arena32.narrow(0, at_table, tokens * topk).view({tokens, topk});
-            metadata.push_back(token_slots);  // private eighth entry: slot[t,k] in one lookup
-        }
-        if (ordered) {
-            slot_order = arena64.narrow(0, at_order, order_entries);
-            metadata.push_back(slot_order);  // private ninth entry: assignments in block-wise slot order
-        }
 
         // The exact shapes (N, C) are only known once the layout kernels have run.  Waiting for
         // them before launching the permute leaves the GPU idle for a host round trip, so where the
@@ -708,8 +707,36 @@ DispatchResult dispatch(PeerRuntime& runtime,
         const bool speculative = tokens > 0 && gap_bound * 8 <= choice_bound && row_bound <= std::numeric_limits<int32_t>::max() &&
                                  order_switch != 0 && (order_switch == 1 || !runtime.prefers_exact_outputs());
         if (speculative) {
+            // enqueued straight from the arena's pointers: the tensors of the handle are made below,
+            // while the GPU works
+            HandleView fresh;
+            fresh.recv_metadata = base32;
+            fresh.dst_slots = base64 + at_dst;
+            fresh.token_slots = expand ? base32 + at_table : nullptr;
+            fresh.slot_order = order_entries > 0 ? base64 + at_order : nullptr;
+            fresh.order_entries = order_entries > 0 ? -1 : 0;
+            fresh.expert_counts = base64;
+            fresh.expert_offsets = base64 + at_offsets;
             allocate_outputs(row_bound, tokens);
-            launch_permute(metadata, tokens, row_bound, /*count_on_device=*/true);
+            launch_permute(fresh, tokens, row_bound, /*count_on_device=*/true);
+        }
+
+        arena32 = arena64.narrow(0, count64, (count32 + 1) / 2).view(torch::kInt32);
+        expert_counts = arena64.narrow(0, 0, local_experts);
+        expert_offsets = arena64.narrow(0, at_offsets, local_experts + 1);
+        send_counts = arena64.narrow(0, at_send, 1);
+        prefix = arena64.narrow(0, at_prefix, 1);
+        dst_slots = arena64.narrow(0, at_dst, tokens).view({tokens, 1});
+        snapshot = arena64.narrow(0, at_snapshot, tokens * topk).view({tokens, topk});
+        recv_metadata = arena32.narrow(0, 0, tokens * (topk + 2)).view({tokens, topk + 2});
+        metadata = {recv_metadata, expert_counts, expert_offsets, dst_slots, send_counts, snapshot, prefix};
+        if (expand) {
+            token_slots = arena32.narrow(0, at_table, tokens * topk).view({tokens, topk});
+            metadata.push_back(token_slots);  // private eighth entry: slot[t,k] in one lookup
+        }
+        if (ordered) {
+            slot_order = arena64.narrow(0, at_order, order_entries);
+            metadata.push_back(slot_order);  // private ninth entry: assignments in block-wise slot order
         }
 
         int64_t counts[NANOEP_HOST_COUNT_WORDS] = {0, 0, 0, 0};
@@ -742,7 +769,7 @@ DispatchResult dispatch(PeerRuntime& runtime,
         } else {
             allocate_outputs(used_rows, recv_count);
             if (recv_count > 0)
-                launch_permute(metadata, recv_count, expanded_capacity);
+                launch_permute(view_of(metadata), recv_count, expanded_capacity);
         }
         if (tokens > 0 && gap_bound * 8 <= choice_bound)
             runtime.note_output_fill(bound_is_close);
