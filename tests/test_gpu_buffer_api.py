@@ -214,6 +214,24 @@ def test_fresh_dispatch_allocation_orders(device, alignment, at_bound):
         assert torch.equal(replay.topk_weights, fresh.topk_weights)
 
 
+@pytest.mark.parametrize("switch,at_bound", [("0", False), ("1", True)], ids=["always-exact", "at-the-bound"])
+def test_fresh_output_order_can_be_forced(device, monkeypatch, switch, at_bound):
+    """NANOEP_FRESH_OUTPUTS=0 allocates a fresh dispatch's outputs after the counts are known whatever
+    the shapes, =1 at the bound whenever the alignment rule allows (a runtime that has turned to the
+    exact order included): same results."""
+    monkeypatch.setenv("NANOEP_FRESH_OUTPUTS", switch)
+    tokens, experts, topk, hidden = 200, 8, 4, 512
+    idx = cases.routing("dropout", tokens, experts, topk, seed=6)
+    x, w = cases.payload(tokens, hidden, seed=7), cases.gate_weights(tokens, topk)
+    with Buffer(None, EPConfig(experts, topk, hidden, tokens)) as buffer:
+        for expand in (True, False):
+            result = buffer.dispatch(x.to(device), topk_idx=idx.to(device), weights=w.to(device), do_expand=expand, zero_padding=True)
+            assert_dispatch_result(result, x, idx, w, experts, expand, 1, True)
+            if expand:  # some choices are masked: the rows in use are fewer than the bound
+                assert result.x.shape[0] < tokens * topk
+                assert (held_rows(result.x, hidden) >= tokens * topk) == at_bound
+
+
 @pytest.mark.parametrize("expand", [False, True], ids=["compact", "expanded"])
 def test_fresh_dispatch_never_holds_much_more_than_it_uses(device, expand):
     """With many masked choices the upper bound is far above what routing fills.  The call that finds
