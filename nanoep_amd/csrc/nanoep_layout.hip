@@ -455,9 +455,11 @@ __device__ __forceinline__ int64_t wave_inclusive_scan(int64_t value) {
 //
 // kFusedScan: `block_counts` holds the raw block histograms and every workgroup sums them itself
 // (they sit in L2): per column the total over all blocks and the part from the blocks before its
-// own, then the aligned exclusive scan over experts, all in LDS; workgroup 0 also writes the
-// per-expert outputs and the host mailbox (word 0 last).  Otherwise layout_scan_kernel has done
-// that and `block_counts` holds each block's exclusive prefixes.
+// own, then the aligned exclusive scan over experts, all in LDS; the workgroup whose index is
+// `publisher` also writes the per-expert outputs and the host mailbox (word 0 last).  With several
+// blocks that is one more workgroup behind those of the blocks, which has no tokens of its own: the
+// store to host memory and its fence then sit on nobody's way to the token writes.  Otherwise
+// layout_scan_kernel has done that and `block_counts` holds each block's exclusive prefixes.
 //
 // Either way the workgroup also scans its own histogram over experts: that places every
 // assignment of the block in expert-major order inside the block's run of `slot_order`; the runs
@@ -485,7 +487,8 @@ __device__ __forceinline__ void layout_assign_block(const int32_t* block_counts,
                                                     int32_t* __restrict__ recv_metadata,
                                                     int64_t* __restrict__ dst_slots,
                                                     int32_t* __restrict__ token_slots,
-                                                    int64_t* __restrict__ slot_order) {
+                                                    int64_t* __restrict__ slot_order,
+                                                    int publisher) {
     extern __shared__ int32_t assign_lds[];
     __shared__ int64_t wave_padded[kMaxBlockTokens / kWave];
     __shared__ int64_t wave_assigned[kMaxBlockTokens / kWave];
@@ -513,10 +516,10 @@ __device__ __forceinline__ void layout_assign_block(const int32_t* block_counts,
     for (int k = 0; k < kCap; ++k)
         packed[k] = live ? packed_rank[token * num_topk + (k < num_topk ? k : 0)] : -1;
 
-    // workgroup 0 gathers the blocks' routing status; the first word a thread is fetched here, used
+    // the publishing workgroup gathers the blocks' routing status; the first word a thread is fetched here, used
     // behind the histogram loads, so that its round trip is not a second one behind theirs
     int first_status = 0;
-    if (kFusedScan && block == 0 && tid < num_blocks)
+    if (kFusedScan && block == publisher && tid < num_blocks)
         first_status = block_status[tid];
     if (kFusedScan) {
         for (int i = tid; i < 4 * rows; i += threads)
@@ -610,7 +613,7 @@ __device__ __forceinline__ void layout_assign_block(const int32_t* block_counts,
             if ((tid & (kWave - 1)) == 0 && own_sum != 0)
                 atomicAdd(&own_assignments, own_sum);
         }
-        if (block == 0) {
+        if (block == publisher) {
             int bad = first_status;
             for (int b = tid + threads; b < num_blocks; b += threads)
                 bad |= block_status[b];
@@ -685,7 +688,7 @@ __device__ __forceinline__ void layout_assign_block(const int32_t* block_counts,
     for (int e = first; e < last; ++e) {
         if (kFusedScan) {
             const int64_t count = column_total[e];
-            if (block == 0) {
+            if (block == publisher) {
                 expert_counts[e] = count;
                 expert_offsets[e] = running;
             }
@@ -700,10 +703,10 @@ __device__ __forceinline__ void layout_assign_block(const int32_t* block_counts,
     }
     const int64_t received = kFusedScan ? column_total[local_experts] : 0;
     __syncthreads();
-    if (kFusedScan && block == 0 && tid == 0) {
+    if (kFusedScan && block == publisher && tid == 0) {
         // Behind the workgroup's last barrier: the store to host memory and the wait that orders it
-        // hold up this one wavefront's share of the token writes below, not the whole workgroup
-        // (in front of the barrier they were a microsecond of the kernel).
+        // hold up one wavefront, not the whole workgroup (in front of the barrier they were a
+        // microsecond of the kernel).
         expert_offsets[local_experts] = capacity;
         send_counts[0] = received;
         recv_rank_prefix[0] = received;
@@ -733,7 +736,7 @@ __device__ __forceinline__ void layout_assign_block(const int32_t* block_counts,
         if (block == num_blocks - 1)
             for (int64_t i = num_tokens * num_topk + tid; i < capacity_entries; i += threads)
                 slot_order[i] = -1;
-        if (block == 0 && tid == 0)
+        if (block == (kFusedScan ? publisher : 0) && tid == 0)
             slot_order[capacity_entries] = assigned;
     }
     if (live)
@@ -764,11 +767,12 @@ __global__ void __launch_bounds__(kMaxBlockTokens) layout_assign_kernel(const in
                                                             int32_t* recv_metadata,
                                                             int64_t* dst_slots,
                                                             int32_t* token_slots,
-                                                            int64_t* slot_order) {
+                                                            int64_t* slot_order,
+                                                            int publisher) {
     layout_assign_block<kCap, kFusedScan>(block_counts, block_status, num_blocks, num_tokens, num_topk, local_experts,
                                           tokens_per_block, window_blocks, threads, expand, alignment, packed_rank, local_row, expert_counts,
                                           expert_offsets, send_counts, recv_rank_prefix, totals, host_counts, recv_metadata,
-                                          dst_slots, token_slots, slot_order);
+                                          dst_slots, token_slots, slot_order, publisher);
 }
 
 // Whole layout in one launch when all tokens fit one block: the count pass, then (its results are
@@ -802,7 +806,7 @@ __global__ void __launch_bounds__(kMaxBlockTokens) layout_single_block_kernel(co
     __syncthreads();
     layout_assign_block<kCap, true>(block_counts, block_status, 1, num_tokens, num_topk, local_experts, words * 32, 1, threads,
                                     expand, alignment, packed_rank, local_row, expert_counts, expert_offsets, send_counts,
-                                    recv_rank_prefix, nullptr, host_counts, recv_metadata, dst_slots, token_slots, slot_order);
+                                    recv_rank_prefix, nullptr, host_counts, recv_metadata, dst_slots, token_slots, slot_order, 0);
 }
 
 
@@ -874,10 +878,11 @@ int enqueue_layout(const int64_t* topk_idx, int64_t num_tokens, int num_topk, in
         }
         const size_t assign_lds = static_cast<size_t>(experts + 1) * 16;
         if (fused_scan) {
-            layout_assign_kernel<kCap, true><<<blocks, count_threads, assign_lds, stream>>>(
+            // one workgroup more than there are blocks: the publisher
+            layout_assign_kernel<kCap, true><<<blocks + 1, count_threads, assign_lds, stream>>>(
                 ws.block_counts, ws.block_status, blocks, num_tokens, num_topk, experts, tokens_per_block, window_blocks,
                 count_threads, expand, alignment, ws.packed_rank, ws.local_row, expert_counts, expert_offsets, send_counts,
-                recv_rank_prefix, ws.totals, host_counts, recv_metadata, dst_slots, token_slots, slot_order);
+                recv_rank_prefix, ws.totals, host_counts, recv_metadata, dst_slots, token_slots, slot_order, blocks);
             launch_status = hipGetLastError();
             return;
         }
@@ -890,7 +895,7 @@ int enqueue_layout(const int64_t* topk_idx, int64_t num_tokens, int num_topk, in
             layout_assign_kernel<kCap, false><<<blocks, count_threads, assign_lds, stream>>>(
                 ws.block_counts, ws.block_status, blocks, num_tokens, num_topk, experts, tokens_per_block, 1, count_threads,
                 expand, alignment, ws.packed_rank, ws.local_row, expert_counts, expert_offsets, send_counts,
-                recv_rank_prefix, ws.totals, host_counts, recv_metadata, dst_slots, token_slots, slot_order);
+                recv_rank_prefix, ws.totals, host_counts, recv_metadata, dst_slots, token_slots, slot_order, 0);
             launch_status = hipGetLastError();
         }
     });
