@@ -161,11 +161,25 @@ __device__ __forceinline__ void layout_count_block(const int64_t* __restrict__ t
     const int word = local_token >> 5;
     const uint32_t bit = 1u << (local_token & 31);
 
+    typedef int64_t i64x2 __attribute__((ext_vector_type(2)));
+    typedef int32_t i32x4 __attribute__((ext_vector_type(4)));
+    // rows of an even number of ids start 16-byte aligned when the tensor does: two ids a load and a store
+    const bool wide_ids = (num_topk & 1) == 0 && (reinterpret_cast<uintptr_t>(topk_idx) & 15) == 0;
+    const bool wide_snapshot = (num_topk & 1) == 0 && (reinterpret_cast<uintptr_t>(snapshot) & 15) == 0;
     int64_t raw[kCap];
     const int64_t* mine = topk_idx + (live ? token : 0) * num_topk;
+    if (wide_ids) {
 #pragma unroll
-    for (int k = 0; k < kCap; ++k)
-        raw[k] = mine[k < num_topk ? k : 0];
+        for (int k = 0; k < kCap; k += 2) {
+            const i64x2 pair = *reinterpret_cast<const i64x2*>(mine + (k < num_topk ? k : 0));
+            raw[k] = pair.x;
+            raw[k + 1] = pair.y;
+        }
+    } else {
+#pragma unroll
+        for (int k = 0; k < kCap; ++k)
+            raw[k] = mine[k < num_topk ? k : 0];
+    }
 
     for (int i = threadIdx.x; i < rows * stride; i += threads)
         bits[i] = 0;
@@ -180,8 +194,14 @@ __device__ __forceinline__ void layout_count_block(const int64_t* __restrict__ t
         ids[k] = (expert >= 0 && expert < local_experts) ? static_cast<int>(expert) : (expert == -1 ? -1 : -2);
         if (!live || k >= num_topk)
             ids[k] = -1;
-        else
+        else if (!wide_snapshot)
             snapshot[token * num_topk + k] = expert;
+    }
+    if (live && wide_snapshot) {
+#pragma unroll
+        for (int k = 0; k < kCap; k += 2)
+            if (k < num_topk)
+                *reinterpret_cast<i64x2*>(snapshot + token * num_topk + k) = i64x2{raw[k], raw[k + 1]};
     }
 
     int bad = 0;
@@ -218,17 +238,27 @@ __device__ __forceinline__ void layout_count_block(const int64_t* __restrict__ t
 
     if (live) {
         const uint32_t below = bit - 1;
+        int32_t packed[kCap];
 #pragma unroll
         for (int k = 0; k < kCap; ++k) {
             const int id = ids[k];
-            int32_t packed = -1;
+            packed[k] = -1;
             if (id >= 0) {
                 const int rank = prefix[static_cast<size_t>(id) * words + word] +
                                  __popc(bits[static_cast<size_t>(id) * stride + word] & below);
-                packed = (id << kRankBits) | rank;
+                packed[k] = (id << kRankBits) | rank;
             }
-            if (k < num_topk)
-                packed_rank[token * num_topk + k] = packed;
+        }
+        if ((num_topk & 3) == 0 && (reinterpret_cast<uintptr_t>(packed_rank) & 15) == 0) {
+#pragma unroll
+            for (int k = 0; k < kCap; k += 4)
+                if (k < num_topk)
+                    *reinterpret_cast<i32x4*>(packed_rank + token * num_topk + k) = i32x4{packed[k], packed[k + 1], packed[k + 2], packed[k + 3]};
+        } else {
+#pragma unroll
+            for (int k = 0; k < kCap; ++k)
+                if (k < num_topk)
+                    packed_rank[token * num_topk + k] = packed[k];
         }
         const uint32_t received = bits[static_cast<size_t>(local_experts) * stride + word];
         local_row[token] = (received & bit) ? prefix[static_cast<size_t>(local_experts) * words + word] + __popc(received & below) : -1;

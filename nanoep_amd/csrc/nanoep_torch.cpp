@@ -658,7 +658,12 @@ DispatchResult dispatch(PeerRuntime& runtime,
         // host latency, the GPU starts three allocator round trips after the call instead of ten
         // and works while the rest of the bookkeeping is done.
         const int64_t order_entries = ordered ? nanoep_slot_order_entries(tokens, static_cast<int>(topk), local_experts) : 0;
-        const int64_t count64 = 2 * local_experts + 3 + tokens + tokens * topk + order_entries;
+        // offsets of the int64 tensors in the arena; the per-token ones start 16-byte aligned (even
+        // offsets), which lets the layout kernels move two ids a lane at a time
+        const auto even = [](int64_t words) { return (words + 1) / 2 * 2; };
+        const int64_t at_offsets = local_experts, at_send = 2 * local_experts + 1, at_prefix = at_send + 1;
+        const int64_t at_dst = even(at_prefix + 1), at_snapshot = even(at_dst + tokens), at_order = even(at_snapshot + tokens * topk);
+        const int64_t count64 = even(at_order + order_entries);
         const int64_t at_table = (tokens * (topk + 2) + 3) / 4 * 4;  // the slot table starts 16-byte aligned
         const int64_t count32 = at_table + (expand ? tokens * topk : 0);
         const size_t workspace_bytes = nanoep_layout_workspace_bytes(tokens, static_cast<int>(topk), local_experts);
@@ -674,8 +679,6 @@ DispatchResult dispatch(PeerRuntime& runtime,
         auto workspace = torch::empty({static_cast<int64_t>(workspace_bytes)}, int64_options.dtype(torch::kUInt8));
         // arena64: expert_counts [L] | expert_offsets [L+1] | send_counts [1] | recv_rank_prefix [1] |
         //          dst_slots [T] | topk snapshot [T*K] | slot_order;   arena32: recv_metadata [T*(K+2)] | token_slots [T*K]
-        const int64_t at_offsets = local_experts, at_send = 2 * local_experts + 1, at_prefix = at_send + 1, at_dst = at_prefix + 1;
-        const int64_t at_snapshot = at_dst + tokens, at_order = at_snapshot + tokens * topk;
         int64_t* base64 = arena64.data_ptr<int64_t>();
         int32_t* base32 = reinterpret_cast<int32_t*>(base64 + count64);
 
