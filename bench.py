@@ -271,20 +271,27 @@ def measure(workload, args, device, detailed):
     result = {}
     with torch.cuda.stream(stream):
         # fresh dispatch: layout kernels + host wait for N/C + permute, as seen by the caller
+        # (two series: wall clock around call + synchronisation with nothing else in between, then the
+        # same calls between two HIP events, whose recording costs the host a few microseconds)
         fresh_times, fresh_gpu_times = [], []
         fresh_calls = WARMUP_MIN + (4 * rotation if detailed else 20)
-        for call in range(fresh_calls, -1, -1):  # rotating sources like the timed steps; the last call takes xs[0]
-            begin, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-            torch.cuda.synchronize()
-            t0 = time.perf_counter()
-            begin.record(stream)
-            received = buffer.dispatch(xs[call % rotation], topk_idx=idx, weights=weights, do_expand=workload.expand,
-                                       alignment=workload.alignment, zero_padding=workload.zero_padding)
-            end.record(stream)
-            torch.cuda.synchronize()
-            if call < fresh_calls - WARMUP_MIN:
-                fresh_times.append(time.perf_counter() - t0)
-                fresh_gpu_times.append(begin.elapsed_time(end) * 1e-3)
+        for with_events in (False, True):
+            for call in range(fresh_calls, -1, -1):  # rotating sources like the timed steps; the last call takes xs[0]
+                begin, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                torch.cuda.synchronize()
+                t0 = time.perf_counter()
+                if with_events:
+                    begin.record(stream)
+                received = buffer.dispatch(xs[call % rotation], topk_idx=idx, weights=weights, do_expand=workload.expand,
+                                           alignment=workload.alignment, zero_padding=workload.zero_padding)
+                if with_events:
+                    end.record(stream)
+                torch.cuda.synchronize()
+                if call < fresh_calls - WARMUP_MIN:
+                    if with_events:
+                        fresh_gpu_times.append(begin.elapsed_time(end) * 1e-3)
+                    else:
+                        fresh_times.append(time.perf_counter() - t0)
         handle = received.handle
         check_combined = buffer.combine(received.x, handle).x
         torch.cuda.synchronize()
