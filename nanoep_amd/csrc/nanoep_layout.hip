@@ -1042,20 +1042,28 @@ int nanoep_wait_counts(int64_t* host_counts, void* stream_handle, double timeout
     if (host_counts == nullptr || out == nullptr)
         return NANOEP_ERR_INVALID_ARGUMENT;
     auto stream = static_cast<hipStream_t>(stream_handle);
+    // The wait is a plain spin on the mailbox word: the counts usually arrive within microseconds,
+    // and whoever waits for them wants to know at once.  The clock is read every 256 spins; the
+    // stream is only asked how it is doing every 100 us of waiting (the question itself takes the
+    // runtime microseconds, during which a published count would go unnoticed).
     timespec start{};
     clock_gettime(CLOCK_MONOTONIC, &start);
+    double next_stream_check = 100e-6;
     uint64_t spins = 0;
     while (true) {
         const int64_t received = __atomic_load_n(&host_counts[0], __ATOMIC_ACQUIRE);
         if (received >= 0)
             break;
-        if ((++spins & 0x3ff) == 0) {
+        if ((++spins & 0xff) == 0) {
             // the clock first: a caller with no patience left is answered without touching the stream
             timespec now{};
             clock_gettime(CLOCK_MONOTONIC, &now);
             const double elapsed = (now.tv_sec - start.tv_sec) + 1e-9 * (now.tv_nsec - start.tv_nsec);
             if (elapsed > timeout_seconds)
                 return NANOEP_ERR_TIMEOUT;
+            if (elapsed < next_stream_check)
+                continue;
+            next_stream_check = elapsed + 100e-6;
             // A finished (or failed) stream with no published count means the layout never ran.
             const hipError_t state = hipStreamQuery(stream);
             if (state != hipErrorNotReady) {
