@@ -564,6 +564,43 @@ def test_argument_errors(device):
         Buffer(None, EPConfig(4, 2, 128, 8))
 
 
+@pytest.mark.parametrize("seed", range(12))
+def test_randomized_shapes_through_the_api(device, seed):
+    """Odd token counts, expert counts, top-k and alignments through fresh dispatch, replay and
+    combine: the handle's tensors are carved out of one allocation whose sections move with every
+    one of these numbers."""
+    generator = torch.Generator().manual_seed(1000 + seed)
+
+    def pick(options):
+        return options[int(torch.randint(len(options), (1,), generator=generator))]
+
+    topk = pick([1, 2, 3, 4, 5, 7, 8])
+    experts = max(topk, pick([3, 8, 17, 64, 129]))
+    tokens = pick([1, 5, 33, 255, 256, 257, 777, 1500])
+    hidden = pick([256, 512, 1280])
+    alignment = pick([1, 1, 3, 8, 16])
+    kind = pick(["random", "dropout", "sparse", "mixed"])
+    expand = pick([True, True, False])
+    idx = cases.routing(kind, tokens, experts, topk, seed=seed)
+    x, w = cases.payload(tokens, hidden, seed=seed), cases.gate_weights(tokens, topk, seed=seed)
+    with Buffer(None, EPConfig(experts, topk, hidden, tokens + 3)) as buffer:
+        for weighted in (True, False):
+            gate = w if weighted else None
+            fresh = buffer.dispatch(x.to(device), topk_idx=idx.to(device), weights=None if gate is None else gate.to(device),
+                                    do_expand=expand, alignment=alignment, zero_padding=expand)
+            lay = assert_dispatch_result(fresh, x, idx, gate, experts, expand, alignment, expand)
+            assert_handle(fresh.handle, lay, expand, alignment, buffer)
+            replay = buffer.dispatch((x * 2).to(device), weights=None if gate is None else gate.to(device), handle=fresh.handle,
+                                     zero_padding=expand)
+            assert_dispatch_result(replay, x * 2, idx, gate, experts, expand, alignment, expand)
+            combined = buffer.combine(fresh.x, fresh.handle, weights=fresh.topk_weights)
+            want, want_w = oracle.combine(fresh.x.cpu(), lay.recv_metadata(expand), lay.dst_slots, do_expand=expand,
+                                          weights=None if gate is None else fresh.topk_weights.cpu())
+            assert_same_bits(combined.x, want, "combined x")
+            if weighted:
+                assert_same_bits(combined.topk_weights, want_w, "combined weights")
+
+
 def test_fresh_dispatches_of_two_threads_on_one_buffer(device):
     """dispatch runs without the interpreter lock, and a buffer has one mailbox for N and C: fresh
     dispatches of two Python threads take turns at it, and each gets the counts and the layout of
