@@ -201,11 +201,13 @@ __global__ void __launch_bounds__(1024) dispatch_ordered_kernel(const u32x4* __r
         // so that the per-XCD ranges split the real work and not an unused tail.
         // A word that cannot be a count (the layout did not run) walks nothing.
         const int64_t live = uniform_load(live_count);
-        if (live != static_cast<int64_t>(entries)) {
-            entries = live >= 0 && live <= static_cast<int64_t>(source_limit) ? static_cast<uint32_t>(live) : 0u;
+        entries = live >= 0 && live <= static_cast<int64_t>(source_limit) ? static_cast<uint32_t>(live) : 0u;
+        // (one workgroup a list entry: no division by a runtime number on every wavefront's way to its load)
+        if (kWholeRows)
+            copy_blocks = entries;
+        else
             copy_blocks = (rows_per_block == 1 ? entries : (entries + rows_per_block - 1) / rows_per_block) * parts;
-            copy_per_xcd = (copy_blocks + kNumXcds - 1) / kNumXcds;
-        }
+        copy_per_xcd = (copy_blocks + kNumXcds - 1) / kNumXcds;
     }
     if (!kWholeRows && blockIdx.x >= payload_blocks) {
         // The weights of the assignments, one lane per list entry, in workgroups of their own at the
