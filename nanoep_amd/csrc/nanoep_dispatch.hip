@@ -186,6 +186,8 @@ __global__ void __launch_bounds__(1024) dispatch_ordered_kernel(const u32x4* __r
                                                                 uint32_t chunks,      // pieces of kSpan chunks in a row
                                                                 uint32_t topk_magic,  // fast divisor by K
                                                                 uint32_t topk_shift,
+                                                                uint32_t rows_magic,  // fast divisor by rows_per_block
+                                                                uint32_t rows_shift,
                                                                 uint32_t payload_blocks) {  // blocks behind them, if any, move the weights
     NANOEP_FETCH_ARGS_4(x, weights, recv_x, recv_weights);
     NANOEP_FETCH_ARGS_4(slot_order, entries, source_limit, out_rows);
@@ -206,7 +208,7 @@ __global__ void __launch_bounds__(1024) dispatch_ordered_kernel(const u32x4* __r
         if (kWholeRows)
             copy_blocks = entries;
         else
-            copy_blocks = (rows_per_block == 1 ? entries : (entries + rows_per_block - 1) / rows_per_block) * parts;
+            copy_blocks = fast_divide(entries + rows_per_block - 1, rows_magic, rows_shift) * parts;
         copy_per_xcd = (copy_blocks + kNumXcds - 1) / kNumXcds;
     }
     if (!kWholeRows && blockIdx.x >= payload_blocks) {
@@ -464,6 +466,7 @@ int nanoep_dispatch(const void* x, const float* weights, const int32_t* recv_met
     auto stream = static_cast<hipStream_t>(stream_handle);
     if (ordered) {
         const FastDivisor topk_divisor = make_fast_divisor(static_cast<uint32_t>(num_topk));
+        const FastDivisor rows_divisor = make_fast_divisor(blocking.rows_per_block);
 #define NANOEP_LAUNCH_ORDERED_ROWS(DEVICE_COUNT, ZERO_FILL, SPAN, WHOLE_ROWS)                                         \
     dispatch_ordered_kernel<DEVICE_COUNT, ZERO_FILL, SPAN, WHOLE_ROWS><<<grid, block, 0, stream>>>(                  \
         static_cast<const u32x4*>(x), weights, slot_order, live_count, expert_counts, expert_offsets,                \
@@ -474,7 +477,7 @@ int nanoep_dispatch(const void* x, const float* weights, const int32_t* recv_met
         static_cast<uint32_t>(pad_groups_per_expert > 0 ? pad_groups_per_expert : 1), blocking.parts,                \
         parts_divisor.magic, parts_divisor.shift, blocking.chunks_per_block, blocking.rows_per_block,                \
         static_cast<uint32_t>(vectors), static_cast<uint32_t>(chunks), topk_divisor.magic, topk_divisor.shift,       \
-        static_cast<uint32_t>(payload_blocks))
+        rows_divisor.magic, rows_divisor.shift, static_cast<uint32_t>(payload_blocks))
 #define NANOEP_LAUNCH_ORDERED_SPAN(DEVICE_COUNT, ZERO_FILL, SPAN)             \
     do {                                                                      \
         if (whole_rows)                                                       \
