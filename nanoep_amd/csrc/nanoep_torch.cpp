@@ -184,8 +184,8 @@ class PeerRuntime {
     // Share of the routing choices that were valid in the latest fresh expanded dispatch, in 1/65536
     // (65536 before the first one).  A permute that is enqueued before the host knows the count sizes
     // its launch for this share of T * K plus half a percent instead of for all of it (a workgroup
-    // that finds nothing to do costs as much as one that takes a second turn: 0.55 us per percent of
-    // the headline batch either way); any count is handled.
+    // that finds nothing to do costs about as much as one that takes a second turn, so the launch
+    // aims at the count itself); any count is handled.
     int64_t valid_share_65536() const { return valid_share_65536_.load(); }
     void note_valid_share(int64_t assignments, int64_t choices) {
         if (choices > 0)
@@ -196,7 +196,7 @@ class PeerRuntime {
     // dispatches.  A caller that keeps only the reference's seven handle tensors gets them back on
     // a replay of one of those handles: an entry is recognised by the identity of the handle's
     // routing snapshot (the tensor object, its data pointer and version) and of its recv_metadata
-    // storage.  The two tensors are views of the allocations that back the seven public ones.
+    // storage.  The two tensors are views of the allocation that backs the seven public ones.
     // Handles this runtime did not make, or made too long ago, are never matched: their replays
     // follow the handle's own recv_metadata and dst_slots in token order.
     void remember_private(const std::vector<torch::Tensor>& metadata, int64_t alignment) {
