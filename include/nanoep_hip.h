@@ -52,6 +52,33 @@ const char* nanoep_last_hip_error(void);
  * nano_ep/backends/cuda.py:108-109). */
 int nanoep_device_cu_count(int device, int* out_cus);
 
+/* What the launch plans take from the current device: compute units, XCDs (each with its own L2;
+ * workgroups are dealt to them round-robin) and the bytes of one XCD's L2.  A process without a
+ * device gets the MI355X's 256 / 8 / 4 MiB.  The XCDS and L2_BYTES switches below override the
+ * last two.  No counterpart in the reference (its grids are sized by num_sms alone,
+ * csrc/pipeline.cu:20-24).  Any pointer may be NULL. */
+int nanoep_device_topology(int* out_cus, int* out_xcds, int64_t* out_l2_bytes);
+
+/*
+ * Tuning switches.  Each is read once per process from the environment variable NANOEP_<NAME>
+ * (first use of the library); afterwards only these calls change it, so no entry point touches the
+ * environment on its way to a launch.  Meant for tests and sweeps: the defaults are the measured
+ * best.  No counterpart in the reference.
+ *   CHUNKS_PER_BLOCK, ROWS_PER_BLOCK (0: by shape)  workgroup shape of the row kernels
+ *   DISPATCH_ORDER (-1; 0: token-order walk even when the handle has a slot-order list)
+ *   DISPATCH_SPAN (0: by size; 1 | 2 chunks a wavefront of the slot-order walk)
+ *   DISPATCH_SIDE (-1; 0 | 1: weights of that walk in workgroups of their own)
+ *   DISPATCH_WHOLE_ROWS (-1; 0 | 1: one workgroup a list entry)
+ *   LAYOUT_LAUNCHES (0; 2 | 3: layout plan)     WINDOW_TOKENS (0; window of the slot-order list)
+ *   RECALL_ORDER, FRESH_OUTPUTS, REBUILD_ORDER (-1; 0 | 1: host-extension policies)
+ *   XCDS, L2_BYTES (0: ask the device)
+ * nanoep_set_tuning / nanoep_get_tuning return NANOEP_ERR_INVALID_ARGUMENT for an unknown name;
+ * nanoep_reset_tuning reads every switch from the environment again.
+ */
+int nanoep_set_tuning(const char* name, int value);
+int nanoep_get_tuning(const char* name, int* value);
+void nanoep_reset_tuning(void);
+
 /* Byte offsets of the reference's peer window regions; a pure function kept so that a caller
  * written against csrc/bindings.cpp:47-58 / csrc/layout.hpp:59-98 still finds it.
  * out = {signal_offset, count_offset, payload_offset, return_offset, num_bytes}. */
@@ -123,6 +150,35 @@ int nanoep_layout_static(const int64_t* topk_idx, int64_t num_tokens, int num_to
                          int64_t alignment, int expand, int hidden, int32_t* recv_metadata, int64_t* expert_counts,
                          int64_t* expert_offsets, int64_t* dst_slots, int64_t* send_counts, int64_t* topk_snapshot,
                          int64_t* recv_rank_prefix, int32_t* token_slots, int64_t* slot_order, int64_t* host_counts,
+                         void* stream);
+
+/* Tokens of one window of the list nanoep_rebuild_order writes for (T, K, hidden). */
+int nanoep_rebuild_window_tokens(int64_t num_tokens, int num_topk, int hidden);
+
+/* Device scratch needed by nanoep_rebuild_order for (T, K). */
+size_t nanoep_rebuild_workspace_bytes(int64_t num_tokens, int num_topk);
+
+/*
+ * The two private handle tensors of an expanded handle, rebuilt from its public ones alone: for a
+ * handle that comes back with only the seven tensors the reference's operator boundary carries
+ * (csrc/pipeline.cu:357-358, nano_ep/backends/cuda.py:296-304).  The handle is followed as it is
+ * written, whatever order its rows and slots are in (the reference's own helper builds handles in
+ * another order, nano_ep/testing/native_combine.py:62-74):
+ *   token_slots[t][k] = recv_metadata[dst_slots[t]][2 + k], -1 when the token was not sent or the
+ *                       value lies outside [0, expanded_capacity)
+ *   slot_order        = window of consecutive tokens by window, the valid (slot << 32) | (t * K + k)
+ *                       in ascending slot order, -1 from entry A on, A in the buffer's last word
+ * (a window is nanoep_layout_block_tokens' for `hidden`, halved until its T * K entries number at
+ * most 4096: any window size is a valid list, the size only decides the walk's locality).
+ * token_slots is int32 [T, K], slot_order int64 [nanoep_slot_order_entries]; workspace needs
+ * nanoep_rebuild_workspace_bytes.  host_count, when not NULL, is one pinned int64 the host can read:
+ * the call stores -1 there and the device later stores host_tag | A (host_tag: a non-negative number
+ * with its low 32 bits clear, so that a reader can tell this call's answer from an older one's).
+ * Two launches on `stream`; T * K < 2^31, T > 0.
+ */
+int nanoep_rebuild_order(const int32_t* recv_metadata, const int64_t* dst_slots, int64_t recv_count, int64_t expanded_capacity,
+                         int64_t num_tokens, int num_topk, int64_t num_local_experts, int hidden, int32_t* token_slots,
+                         int64_t* slot_order, void* workspace, size_t workspace_bytes, int64_t* host_count, int64_t host_tag,
                          void* stream);
 
 /* Spin on the mailbox until the layout enqueued on `stream` has published its counts

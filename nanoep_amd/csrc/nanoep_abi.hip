@@ -1,46 +1,104 @@
 // Version, status strings, window layout, profiler calibration copy.
 
-#include <unistd.h>
+#include <atomic>
+#include <climits>
+#include <mutex>
 
 #include "nanoep_device.h"
-
-extern char** environ;
 
 namespace nanoep {
 
 thread_local hipError_t g_last_hip_error = hipSuccess;
-thread_local Tuning g_tuning;
-
-void refresh_tuning() {
-    Tuning fresh;
-    struct Switch {
-        const char* name;  // behind the NANOEP_ prefix
-        int* value;
-    };
-    const Switch switches[] = {
-        {"CHUNKS_PER_BLOCK", &fresh.chunks_per_block}, {"ROWS_PER_BLOCK", &fresh.rows_per_block},
-        {"DISPATCH_ORDER", &fresh.dispatch_order},     {"DISPATCH_SPAN", &fresh.dispatch_span},
-        {"DISPATCH_SIDE", &fresh.dispatch_side},       {"DISPATCH_WHOLE_ROWS", &fresh.dispatch_whole_rows},
-        {"LAYOUT_LAUNCHES", &fresh.layout_launches},   {"WINDOW_TOKENS", &fresh.window_tokens},
-    };
-    if (environ != nullptr) {
-        for (char** entry = environ; *entry != nullptr; ++entry) {
-            const char* text = *entry;
-            if (text[0] != 'N' || std::strncmp(text, "NANOEP_", 7) != 0)
-                continue;
-            for (const Switch& item : switches) {
-                const size_t length = std::strlen(item.name);
-                // NANOEP_<NAME>=<number>; an empty value leaves the default
-                if (std::strncmp(text + 7, item.name, length) == 0 && text[7 + length] == '=' && text[8 + length] != '\0')
-                    *item.value = std::atoi(text + 8 + length);
-            }
-        }
-    }
-    g_tuning = fresh;
-}
 
 namespace {
 
+// The switches by name (behind the NANOEP_ prefix in the environment), where they sit in Tuning, and
+// their process-wide values.
+struct SwitchSlot {
+    const char* name;
+    int Tuning::*field;
+};
+
+constexpr SwitchSlot kSwitches[] = {
+    {"CHUNKS_PER_BLOCK", &Tuning::chunks_per_block}, {"ROWS_PER_BLOCK", &Tuning::rows_per_block},
+    {"DISPATCH_ORDER", &Tuning::dispatch_order},     {"DISPATCH_SPAN", &Tuning::dispatch_span},
+    {"DISPATCH_SIDE", &Tuning::dispatch_side},       {"DISPATCH_WHOLE_ROWS", &Tuning::dispatch_whole_rows},
+    {"LAYOUT_LAUNCHES", &Tuning::layout_launches},   {"WINDOW_TOKENS", &Tuning::window_tokens},
+    {"RECALL_ORDER", &Tuning::recall_order},         {"FRESH_OUTPUTS", &Tuning::fresh_outputs},
+    {"REBUILD_ORDER", &Tuning::rebuild_order},       {"XCDS", &Tuning::xcds},
+    {"L2_BYTES", &Tuning::l2_bytes},
+};
+constexpr int kSwitchCount = sizeof(kSwitches) / sizeof(kSwitches[0]);
+
+std::atomic<int> g_switch_values[kSwitchCount];
+std::once_flag g_switches_once;
+
+// NANOEP_<NAME>=<number> in the environment; unset or empty leaves the default.
+void load_switches_from_environment() {
+    const Tuning defaults;
+    for (int i = 0; i < kSwitchCount; ++i) {
+        char variable[64];
+        std::snprintf(variable, sizeof(variable), "NANOEP_%s", kSwitches[i].name);
+        const char* text = std::getenv(variable);
+        g_switch_values[i].store(text != nullptr && *text != '\0' ? std::atoi(text) : defaults.*(kSwitches[i].field),
+                                 std::memory_order_relaxed);
+    }
+}
+
+int find_switch(const char* name) {
+    if (name == nullptr)
+        return -1;
+    for (int i = 0; i < kSwitchCount; ++i)
+        if (std::strcmp(name, kSwitches[i].name) == 0)
+            return i;
+    return -1;
+}
+
+constexpr int kMaxDevices = 64;
+std::mutex g_topology_mutex;
+bool g_topology_known[kMaxDevices] = {};
+Topology g_topology[kMaxDevices];
+
+}  // namespace
+
+Tuning current_tuning() {
+    std::call_once(g_switches_once, load_switches_from_environment);
+    Tuning tuning;
+    for (int i = 0; i < kSwitchCount; ++i)
+        tuning.*(kSwitches[i].field) = g_switch_values[i].load(std::memory_order_relaxed);
+    return tuning;
+}
+
+Topology current_topology(const Tuning& tuning) {
+    Topology topology;  // the MI355X's numbers, for a process without a device
+    int device = -1;
+    if (hipGetDevice(&device) == hipSuccess && device >= 0 && device < kMaxDevices) {
+        std::lock_guard<std::mutex> lock(g_topology_mutex);
+        if (!g_topology_known[device]) {
+            Topology asked;
+            int value = 0;
+            if (hipDeviceGetAttribute(&value, hipDeviceAttributeMultiprocessorCount, device) == hipSuccess && value > 0)
+                asked.cus = value;
+            if (hipDeviceGetAttribute(&value, hipDeviceAttributeNumberOfXccs, device) == hipSuccess && value > 0)
+                asked.xcds = value;
+            // the runtime reports the L2 of one XCD; a part that reports none keeps the default
+            if (hipDeviceGetAttribute(&value, hipDeviceAttributeL2CacheSize, device) == hipSuccess && value >= (1 << 20))
+                asked.l2_bytes = value;
+            g_topology[device] = asked;
+            g_topology_known[device] = true;
+        }
+        topology = g_topology[device];
+    } else {
+        (void)hipGetLastError();  // no device: not an error of the caller's
+    }
+    if (tuning.xcds > 0)
+        topology.xcds = tuning.xcds;
+    if (tuning.l2_bytes > 0)
+        topology.l2_bytes = tuning.l2_bytes;
+    return topology;
+}
+
+namespace {
 
 __global__ void __launch_bounds__(kBlockThreads) copy_vectors_kernel(const u32x4* __restrict__ src,
                                                                     u32x4* __restrict__ dst,
@@ -82,6 +140,40 @@ const char* nanoep_status_string(int status) {
 
 const char* nanoep_last_hip_error(void) {
     return g_last_hip_error == hipSuccess ? "" : hipGetErrorString(g_last_hip_error);
+}
+
+int nanoep_set_tuning(const char* name, int value) {
+    const int at = find_switch(name);
+    if (at < 0)
+        return NANOEP_ERR_INVALID_ARGUMENT;
+    std::call_once(g_switches_once, load_switches_from_environment);
+    g_switch_values[at].store(value, std::memory_order_relaxed);
+    return NANOEP_OK;
+}
+
+int nanoep_get_tuning(const char* name, int* value) {
+    const int at = find_switch(name);
+    if (at < 0 || value == nullptr)
+        return NANOEP_ERR_INVALID_ARGUMENT;
+    std::call_once(g_switches_once, load_switches_from_environment);
+    *value = g_switch_values[at].load(std::memory_order_relaxed);
+    return NANOEP_OK;
+}
+
+void nanoep_reset_tuning(void) {
+    std::call_once(g_switches_once, load_switches_from_environment);
+    load_switches_from_environment();
+}
+
+int nanoep_device_topology(int* out_cus, int* out_xcds, int64_t* out_l2_bytes) {
+    const Topology topology = current_topology(current_tuning());
+    if (out_cus != nullptr)
+        *out_cus = topology.cus;
+    if (out_xcds != nullptr)
+        *out_xcds = topology.xcds;
+    if (out_l2_bytes != nullptr)
+        *out_l2_bytes = topology.l2_bytes;
+    return NANOEP_OK;
 }
 
 int nanoep_device_cu_count(int device, int* out_cus) {

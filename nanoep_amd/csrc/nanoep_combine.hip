@@ -306,7 +306,7 @@ int nanoep_combine(const void* y, const float* weights, const void* bias, const 
                    const int64_t* dst_slots, const int32_t* token_slots, int64_t recv_count, int64_t y_rows,
                    int64_t num_tokens, int hidden, int num_topk, int expand, int multiple_reduction, void* out_x,
                    float* out_weights, int num_cus, void* stream_handle) {
-    refresh_tuning();
+    const Tuning tuning = current_tuning();
     if (hidden <= 0 || hidden % 8 != 0 || num_topk <= 0 || num_topk > kMaxTopk)
         return NANOEP_ERR_INVALID_ARGUMENT;
     if (recv_count < 0 || num_tokens < 0 || recv_count > num_tokens || num_tokens > INT32_MAX || y_rows < 0 ||
@@ -319,7 +319,7 @@ int nanoep_combine(const void* y, const float* weights, const void* bias, const 
         return NANOEP_ERR_INVALID_ARGUMENT;
     if (!aligned16(y) || !aligned16(out_x) || !aligned16(bias))
         return NANOEP_ERR_INVALID_ARGUMENT;
-    const int budget_status = validate_cu_budget(num_cus);
+    const int budget_status = validate_cu_budget(num_cus, current_topology(tuning));
     if (budget_status != NANOEP_OK)
         return budget_status;
     if (num_tokens == 0)
@@ -330,7 +330,7 @@ int nanoep_combine(const void* y, const float* weights, const void* bias, const 
     const int vectors = hidden / 8;
     const int chunks = (vectors + kWave - 1) / kWave;
     // top-1 expanded combines are row copies like the compact ones
-    const RowBlocking blocking = pick_row_blocking(chunks, expand && num_topk > 1 ? kTokenOrderWalk : kRowCopyWalk);
+    const RowBlocking blocking = pick_row_blocking(chunks, expand && num_topk > 1 ? kTokenOrderWalk : kRowCopyWalk, tuning);
     const int64_t blocks = (num_tokens + blocking.rows_per_block - 1) / blocking.rows_per_block * blocking.parts;
     if (blocks >= (int64_t{1} << 31))
         return NANOEP_ERR_INVALID_ARGUMENT;

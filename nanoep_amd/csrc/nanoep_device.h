@@ -70,24 +70,38 @@ extern thread_local hipError_t g_last_hip_error;
 
 inline size_t align_up(size_t value, size_t alignment) { return (value + alignment - 1) / alignment * alignment; }
 
-// Tuning switches of the library, read from the environment (NANOEP_<NAME>; tests and sweeps flip
-// them between calls).  Every entry point of the C ABI reads them afresh with one walk over the
-// environment (refresh_tuning) into this per-thread record; the code below the entry points only
-// looks at the record.  (A getenv per switch and use walked the whole environment a dozen to two
-// dozen times a call, microseconds on the host path of a fresh dispatch.)
+// Tuning switches of the library.  Each is NANOEP_<NAME> in the environment, which is read exactly
+// once per process, on the first use of the library; nanoep_set_tuning changes one afterwards (tests
+// and sweeps do that between calls).  The record is a handful of relaxed atomics: entry points take
+// one snapshot of it (current_tuning) and the code below them only looks at the snapshot.
 struct Tuning {
-    int chunks_per_block = 0;       // NANOEP_CHUNKS_PER_BLOCK: wavefronts along a row in a workgroup, 0 = by shape
-    int rows_per_block = 0;         // NANOEP_ROWS_PER_BLOCK: rows a workgroup, 0 = by shape
-    int dispatch_order = -1;        // NANOEP_DISPATCH_ORDER: 0 forces the token-order walk
-    int dispatch_span = 0;          // NANOEP_DISPATCH_SPAN: 1 | 2 chunks a wavefront of the slot-order walk, 0 = by size
-    int dispatch_side = -1;         // NANOEP_DISPATCH_SIDE: 0 | 1 weights of that walk in workgroups of their own
-    int dispatch_whole_rows = -1;   // NANOEP_DISPATCH_WHOLE_ROWS: 0 | 1 the kernel variant for one workgroup a list entry
-    int layout_launches = 0;        // NANOEP_LAYOUT_LAUNCHES: 2 | 3 forces the layout plan
-    int window_tokens = 0;          // NANOEP_WINDOW_TOKENS: forces the window of the slot-order list
+    int chunks_per_block = 0;       // CHUNKS_PER_BLOCK: wavefronts along a row in a workgroup, 0 = by shape
+    int rows_per_block = 0;         // ROWS_PER_BLOCK: rows a workgroup, 0 = by shape
+    int dispatch_order = -1;        // DISPATCH_ORDER: 0 forces the token-order walk
+    int dispatch_span = 0;          // DISPATCH_SPAN: 1 | 2 chunks a wavefront of the slot-order walk, 0 = by size
+    int dispatch_side = -1;         // DISPATCH_SIDE: 0 | 1 weights of that walk in workgroups of their own
+    int dispatch_whole_rows = -1;   // DISPATCH_WHOLE_ROWS: 0 | 1 the kernel variant for one workgroup a list entry
+    int layout_launches = 0;        // LAYOUT_LAUNCHES: 2 | 3 forces the layout plan
+    int window_tokens = 0;          // WINDOW_TOKENS: forces the window of the slot-order list
+    int recall_order = -1;          // RECALL_ORDER: 0 = seven-tensor handles never get private tensors back (host extension)
+    int fresh_outputs = -1;         // FRESH_OUTPUTS: 0 | 1 where a fresh dispatch's outputs are allocated (host extension)
+    int rebuild_order = -1;         // REBUILD_ORDER: 0 | 1 never / always rebuild the private tensors of a seven-tensor handle
+    int xcds = 0;                   // XCDS: number of XCDs the block remap assumes, 0 = ask the device
+    int l2_bytes = 0;               // L2_BYTES: size of one XCD's L2 the windows are sized for, 0 = ask the device
 };
 
-extern thread_local Tuning g_tuning;  // defined in nanoep_abi.hip
-void refresh_tuning();                // defined in nanoep_abi.hip
+Tuning current_tuning();  // defined in nanoep_abi.hip
+
+// What the launch plans need to know of the device: compute units, XCDs (each with an L2 of its
+// own; workgroups are handed to them round-robin by linear id) and the size of one such L2.
+// Asked of the runtime once per device; a process without a device gets the MI355X's numbers.
+struct Topology {
+    int cus = 256;
+    int xcds = 8;
+    int64_t l2_bytes = int64_t{4} << 20;
+};
+
+Topology current_topology(const Tuning& tuning);  // defined in nanoep_abi.hip
 
 // Calls f with the smallest compile-time bound in {4, 8, 16, 32} that covers num_topk.
 template <typename F>
@@ -126,9 +140,6 @@ __device__ __forceinline__ T uniform_load(const T* p) {
     return *(const __attribute__((address_space(4))) T*)(p);
 }
 
-// Workgroups are handed to the 8 XCDs round-robin by their linear id, and every XCD has its own L2.
-constexpr int kNumXcds = 8;
-
 // n / d for n < 2^31 as one 64-bit multiply and shift: magic = ceil(2^shift / d), shift = 31 + ceil(log2 d).
 struct FastDivisor {
     uint32_t magic;
@@ -146,6 +157,22 @@ inline FastDivisor make_fast_divisor(uint32_t divisor) {
 
 __device__ __forceinline__ uint32_t fast_divide(uint32_t n, uint32_t magic, uint32_t shift) {
     return static_cast<uint32_t>((static_cast<uint64_t>(n) * magic) >> shift);
+}
+
+// Workgroups are handed to the XCDs round-robin by their linear id and every XCD has its own L2, so
+// kernels whose neighbouring work items share data remap the linear id: workgroup b runs on XCD
+// b % count and is the (b / count)-th workgroup there.  count comes from the device (8 on an
+// unpartitioned MI355X), so the division is a multiply-shift by a host-made magic number.
+struct XcdMap {
+    uint32_t count;
+    uint32_t magic;
+    uint32_t shift;
+};
+
+inline XcdMap make_xcd_map(int xcds) {
+    const uint32_t count = xcds > 0 ? static_cast<uint32_t>(xcds) : 1u;
+    const FastDivisor divisor = make_fast_divisor(count);
+    return {count, divisor.magic, divisor.shift};
 }
 
 // Kernel arguments are fetched with scalar loads where they are first used, which strings several
@@ -175,9 +202,9 @@ enum WalkShape {
     kRowCopyWalk,     // compact layouts (plain row copies): single-wavefront workgroups
 };
 
-inline RowBlocking pick_row_blocking(int chunks, WalkShape shape) {
+inline RowBlocking pick_row_blocking(int chunks, WalkShape shape, const Tuning& tuning) {
     RowBlocking blocking{};
-    int per_block = g_tuning.chunks_per_block;
+    int per_block = tuning.chunks_per_block;
     if (per_block < 1 || per_block > kMaxWavesPerBlock) {
         per_block = kDefaultChunksPerBlock;
         if (shape == kSlotOrderWalk) {
@@ -199,7 +226,7 @@ inline RowBlocking pick_row_blocking(int chunks, WalkShape shape) {
     blocking.parts = static_cast<unsigned>((chunks + per_block - 1) / per_block);
     int rows = 1;
     if (blocking.parts == 1) {
-        rows = g_tuning.rows_per_block;
+        rows = tuning.rows_per_block;
         if (rows < 1 || rows * per_block > kMaxWavesPerBlock)
             rows = per_block >= 4 ? 1 : 4 / per_block;
     }
@@ -207,18 +234,8 @@ inline RowBlocking pick_row_blocking(int chunks, WalkShape shape) {
     return blocking;
 }
 
-inline int validate_cu_budget(int num_cus) {
-    int device = 0;
-    NANOEP_HIP_TRY(hipGetDevice(&device));
-    static thread_local int cached_device = -1;
-    static thread_local int cached_cus = 0;
-    if (device != cached_device) {
-        int cus = 0;
-        NANOEP_HIP_TRY(hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, device));
-        cached_device = device;
-        cached_cus = cus;
-    }
-    return (num_cus < 0 || num_cus > cached_cus) ? NANOEP_ERR_INVALID_ARGUMENT : NANOEP_OK;
+inline int validate_cu_budget(int num_cus, const Topology& topology) {
+    return (num_cus < 0 || num_cus > topology.cus) ? NANOEP_ERR_INVALID_ARGUMENT : NANOEP_OK;
 }
 
 inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }

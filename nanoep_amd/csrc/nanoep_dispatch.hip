@@ -74,9 +74,9 @@ __global__ void __launch_bounds__(1024) dispatch_rows_kernel(const u32x4* __rest
                                                              int64_t out_rows,
                                                              uint32_t copy_candidates,  // T*K
                                                              uint32_t copy_blocks,
-                                                             uint32_t copy_per_xcd,  // ceil(copy_blocks / 8)
+                                                             uint32_t copy_per_xcd,  // ceil(copy_blocks / XCDs)
                                                              uint32_t pad_blocks,
-                                                             uint32_t pad_per_xcd,   // ceil(pad_blocks / 8)
+                                                             uint32_t pad_per_xcd,   // ceil(pad_blocks / XCDs)
                                                              uint32_t parts,            // workgroups per candidate group (rows longer than 16 chunks)
                                                              uint32_t parts_magic,      // fast divisor by parts
                                                              uint32_t parts_shift,
@@ -87,19 +87,21 @@ __global__ void __launch_bounds__(1024) dispatch_rows_kernel(const u32x4* __rest
                                                              int vectors,
                                                              int chunks,
                                                              int num_topk,
-                                                             int topk_shift) {  // log2(K) when K is a power of two, else -1
+                                                             int topk_shift,  // log2(K) when K is a power of two, else -1
+                                                             XcdMap xcds) {
     NANOEP_FETCH_ARGS_4(x, weights, recv_x, recv_weights);
     NANOEP_FETCH_ARGS_4(token_slots, copy_blocks, dst_slots, recv_metadata);
     NANOEP_FETCH_ARGS_4(out_rows, recv_count, copy_candidates, copy_per_xcd);
     NANOEP_FETCH_ARGS_4(parts_magic, parts_shift, vectors, chunks);
     NANOEP_FETCH_ARGS_4(num_topk, topk_shift, rows_per_block, chunks_per_block);
+    NANOEP_FETCH_ARGS_4(xcds.count, xcds.magic, xcds.shift, copy_per_xcd);
     // Workgroups are handed to the XCDs round-robin.  Each XCD takes one contiguous range of the
     // copy work followed by one contiguous range of the zero-fill work, so neighbouring work items
     // (which share their source rows) stay behind one L2 and every XCD gets its share of both.
     // (kZeroFill is false when the launch has no zero-fill work: the copy path then carries none of
     // its bookkeeping, which shows in a wavefront that lives about a microsecond)
-    const uint32_t xcd = blockIdx.x % kNumXcds;
-    const uint32_t index_in_xcd = blockIdx.x / kNumXcds;
+    const uint32_t index_in_xcd = fast_divide(blockIdx.x, xcds.magic, xcds.shift);
+    const uint32_t xcd = blockIdx.x - index_in_xcd * xcds.count;
     const bool copy_work = !kZeroFill || index_in_xcd < copy_per_xcd;
     uint32_t block = xcd * copy_per_xcd + index_in_xcd;
     if (kZeroFill && !copy_work)
@@ -188,12 +190,14 @@ __global__ void __launch_bounds__(1024) dispatch_ordered_kernel(const u32x4* __r
                                                                 uint32_t topk_shift,
                                                                 uint32_t rows_magic,  // fast divisor by rows_per_block
                                                                 uint32_t rows_shift,
-                                                                uint32_t payload_blocks) {  // blocks behind them, if any, move the weights
+                                                                uint32_t payload_blocks,  // blocks behind them, if any, move the weights
+                                                                XcdMap xcds) {
     NANOEP_FETCH_ARGS_4(x, weights, recv_x, recv_weights);
     NANOEP_FETCH_ARGS_4(slot_order, entries, source_limit, out_rows);
     NANOEP_FETCH_ARGS_4(copy_blocks, copy_per_xcd, parts, parts_magic);
     NANOEP_FETCH_ARGS_4(parts_shift, chunks_per_block, rows_per_block, vectors);
     NANOEP_FETCH_ARGS_4(chunks, topk_magic, topk_shift, live_count);
+    NANOEP_FETCH_ARGS_4(xcds.count, xcds.magic, xcds.shift, payload_blocks);
     // workgroups per XCD the grid holds for the copy work: with the entry count on the device the live
     // list may be shorter (the rest of the grid leaves at once) or longer (workgroups then take more
     // than one turn, `grid_copy_per_xcd` list positions apart) than what the grid was sized for
@@ -209,7 +213,7 @@ __global__ void __launch_bounds__(1024) dispatch_ordered_kernel(const u32x4* __r
             copy_blocks = entries;
         else
             copy_blocks = fast_divide(entries + rows_per_block - 1, rows_magic, rows_shift) * parts;
-        copy_per_xcd = (copy_blocks + kNumXcds - 1) / kNumXcds;
+        copy_per_xcd = fast_divide(copy_blocks + xcds.count - 1, xcds.magic, xcds.shift);
     }
     if (!kWholeRows && blockIdx.x >= payload_blocks) {
         // The weights of the assignments, one lane per list entry, in workgroups of their own at the
@@ -230,12 +234,13 @@ __global__ void __launch_bounds__(1024) dispatch_ordered_kernel(const u32x4* __r
         }
         return;
     }
-    const uint32_t index_in_xcd = blockIdx.x / kNumXcds;
+    const uint32_t index_in_xcd = fast_divide(blockIdx.x, xcds.magic, xcds.shift);
+    const uint32_t xcd = blockIdx.x - index_in_xcd * xcds.count;
     // the XCD's workgroups up to `copy_turns` copy, the ones behind them clear gap rows
     const uint32_t copy_turns = kDeviceCount && copy_per_xcd > grid_copy_per_xcd ? grid_copy_per_xcd : copy_per_xcd;
     if (kZeroFill && index_in_xcd >= copy_turns) {
         const uint32_t pad_index = index_in_xcd - copy_turns;
-        const uint32_t pad_block = (blockIdx.x % kNumXcds) * pad_per_xcd + pad_index;
+        const uint32_t pad_block = xcd * pad_per_xcd + pad_index;
         if (pad_index < pad_per_xcd && pad_block < pad_blocks)
             zero_fill_gap_rows(pad_block, pad_per_expert, pad_groups_per_expert, chunks_per_block, rows_per_block,
                                expert_counts, expert_offsets, recv_x, recv_weights, out_rows, static_cast<int>(vectors));
@@ -245,7 +250,7 @@ __global__ void __launch_bounds__(1024) dispatch_ordered_kernel(const u32x4* __r
         return;
     // one turn, except where a device-side count found more entries than the grid was sized for
     for (uint32_t at = index_in_xcd; at < copy_per_xcd; at += grid_copy_per_xcd) {
-        const uint32_t block = (blockIdx.x % kNumXcds) * copy_per_xcd + at;
+        const uint32_t block = xcd * copy_per_xcd + at;
         uint32_t candidate, chunk;
         if (kWholeRows) {
             // one workgroup a row, as many wavefronts as the row has pieces: the block is the list entry
@@ -373,7 +378,7 @@ int nanoep_dispatch(const void* x, const float* weights, const int32_t* recv_met
                     int64_t recv_count, int64_t expanded_capacity, int64_t num_tokens, int hidden, int num_topk,
                     int64_t num_local_experts, int64_t alignment, int expand, int zero_padding, void* recv_x,
                     int64_t* recv_topk_idx, float* recv_weights, int num_cus, void* stream_handle) {
-    refresh_tuning();
+    const Tuning tuning = current_tuning();
     if (hidden <= 0 || hidden % 8 != 0 || num_topk <= 0 || num_topk > kMaxTopk || num_local_experts <= 0 || alignment <= 0)
         return NANOEP_ERR_INVALID_ARGUMENT;
     if (recv_count < 0 || num_tokens < 0 || recv_count > num_tokens || num_tokens > INT32_MAX || expanded_capacity < 0 ||
@@ -383,9 +388,11 @@ int nanoep_dispatch(const void* x, const float* weights, const int32_t* recv_met
         return NANOEP_ERR_INVALID_ARGUMENT;
     if (!aligned16(x) || !aligned16(recv_x))
         return NANOEP_ERR_INVALID_ARGUMENT;
-    const int budget_status = validate_cu_budget(num_cus);
+    const Topology topology = current_topology(tuning);
+    const int budget_status = validate_cu_budget(num_cus, topology);
     if (budget_status != NANOEP_OK)
         return budget_status;
+    const XcdMap xcds = make_xcd_map(topology.xcds);
     const int64_t out_rows = expand ? expanded_capacity : recv_count;
     if (recv_count == 0 || out_rows == 0)
         return NANOEP_OK;  // nothing was received: the outputs have no rows to write
@@ -402,7 +409,7 @@ int nanoep_dispatch(const void* x, const float* weights, const int32_t* recv_met
     // The walk is used whenever the handle carries the list.  With cache-resident sources and fewer
     // than eight token blocks the token-order walk is up to 15 % faster, but with cold sources it is
     // 25-60 % slower at every size, so the list decides.
-    const int order_switch = g_tuning.dispatch_order;  // 0 forces the token-order walk
+    const int order_switch = tuning.dispatch_order;  // 0 forces the token-order walk
     const bool ordered = expand && slot_order != nullptr && order_bound > 0 && order_switch != 0;
     if (ordered && (slot_order_entries > order_bound || num_tokens * num_topk >= (int64_t{1} << 31)))
         return NANOEP_ERR_INVALID_ARGUMENT;
@@ -427,13 +434,13 @@ int nanoep_dispatch(const void* x, const float* weights, const int32_t* recv_met
     if (ordered) {
         const bool short_rows = chunks == 2;
         span = short_rows || static_cast<int64_t>(num_tokens) * hidden * 2 > kLastLevelCacheBytes ? 2 : 1;
-        const int forced_span = g_tuning.dispatch_span;
+        const int forced_span = tuning.dispatch_span;
         if (forced_span == 1 || forced_span == 2)
             span = forced_span;
         chunks = (chunks + span - 1) / span;
     }
     const WalkShape walk = ordered ? kSlotOrderWalk : expand ? kTokenOrderWalk : kRowCopyWalk;
-    const RowBlocking blocking = pick_row_blocking(chunks, walk);
+    const RowBlocking blocking = pick_row_blocking(chunks, walk, tuning);
     const int64_t waves = static_cast<int64_t>(blocking.chunks_per_block) * blocking.rows_per_block;
     const int64_t copy_candidates = ordered ? slot_order_entries : expand ? num_tokens * num_topk : num_tokens;
     const int64_t copy_blocks = (copy_candidates + blocking.rows_per_block - 1) / blocking.rows_per_block * blocking.parts;
@@ -441,10 +448,10 @@ int nanoep_dispatch(const void* x, const float* weights, const int32_t* recv_met
     const int64_t pad_per_expert = !pad ? 0 : (alignment - 1 < expanded_capacity ? alignment - 1 : expanded_capacity);
     const int64_t pad_groups_per_expert = (pad_per_expert + waves - 1) / waves;
     const int64_t pad_blocks = num_local_experts * pad_groups_per_expert;
-    if (copy_candidates >= (int64_t{1} << 31) || copy_blocks + pad_blocks >= (int64_t{1} << 31) - 2 * kNumXcds)
+    if (copy_candidates >= (int64_t{1} << 31) || copy_blocks + pad_blocks >= (int64_t{1} << 31) - 2 * int64_t{xcds.count})
         return NANOEP_ERR_INVALID_ARGUMENT;
-    const uint32_t copy_per_xcd = static_cast<uint32_t>((copy_blocks + kNumXcds - 1) / kNumXcds);
-    const uint32_t pad_per_xcd = static_cast<uint32_t>((pad_blocks + kNumXcds - 1) / kNumXcds);
+    const uint32_t copy_per_xcd = static_cast<uint32_t>((copy_blocks + xcds.count - 1) / xcds.count);
+    const uint32_t pad_per_xcd = static_cast<uint32_t>((pad_blocks + xcds.count - 1) / xcds.count);
     int topk_shift = -1;
     if ((num_topk & (num_topk - 1)) == 0)
         for (topk_shift = 0; (1 << topk_shift) < num_topk; ++topk_shift) {
@@ -453,11 +460,11 @@ int nanoep_dispatch(const void* x, const float* weights, const int32_t* recv_met
     // slot-order walk over rows of one or two chunks: one lane per list entry moves the weights, in
     // workgroups at the end of the grid (+3-4 %); longer rows carry the weight on their first wavefront
     // (8192 x 2048 top-8 with alignment 128: 56.0 against 57.0 us).  NANOEP_DISPATCH_SIDE=0|1 overrides.
-    const int side_switch = g_tuning.dispatch_side;
+    const int side_switch = tuning.dispatch_side;
     const bool side_weights = ordered && recv_weights != nullptr && (side_switch < 0 ? row_chunks <= 2 : side_switch != 0);
     const int64_t side_lanes = side_weights ? copy_candidates : 0;
     const int64_t side_blocks = (side_lanes + kWave * waves - 1) / (kWave * waves);
-    const int64_t payload_blocks = (int64_t{copy_per_xcd} + pad_per_xcd) * kNumXcds;
+    const int64_t payload_blocks = (int64_t{copy_per_xcd} + pad_per_xcd) * xcds.count;
     if (payload_blocks + side_blocks >= (int64_t{1} << 31))
         return NANOEP_ERR_INVALID_ARGUMENT;
     const dim3 grid(static_cast<unsigned>(payload_blocks + side_blocks));
@@ -477,7 +484,7 @@ int nanoep_dispatch(const void* x, const float* weights, const int32_t* recv_met
         static_cast<uint32_t>(pad_groups_per_expert > 0 ? pad_groups_per_expert : 1), blocking.parts,                \
         parts_divisor.magic, parts_divisor.shift, blocking.chunks_per_block, blocking.rows_per_block,                \
         static_cast<uint32_t>(vectors), static_cast<uint32_t>(chunks), topk_divisor.magic, topk_divisor.shift,       \
-        rows_divisor.magic, rows_divisor.shift, static_cast<uint32_t>(payload_blocks))
+        rows_divisor.magic, rows_divisor.shift, static_cast<uint32_t>(payload_blocks), xcds)
 #define NANOEP_LAUNCH_ORDERED_SPAN(DEVICE_COUNT, ZERO_FILL, SPAN)             \
     do {                                                                      \
         if (whole_rows)                                                       \
@@ -496,7 +503,7 @@ int nanoep_dispatch(const void* x, const float* weights, const int32_t* recv_met
         // division to find its entry and piece (4096 x 7168: 81.5 -> 80.4 us, with alignment 128
         // 100.6 -> 96.9 us, 8192 x 5120: 123.1 -> 120.3 us).  Rows of four pieces are better off
         // with the general path (8192 x 2048 with cache-resident sources: 37.6 against 38.3 us).
-        const int whole_rows_switch = g_tuning.dispatch_whole_rows;
+        const int whole_rows_switch = tuning.dispatch_whole_rows;
         const bool whole_rows = blocking.parts == 1 && blocking.rows_per_block == 1 &&
                                 blocking.chunks_per_block == static_cast<unsigned>(chunks) && side_blocks == 0 &&
                                 (whole_rows_switch < 0 ? chunks >= 5 : whole_rows_switch != 0);
@@ -534,7 +541,7 @@ int nanoep_dispatch(const void* x, const float* weights, const int32_t* recv_met
         static_cast<uint32_t>(pad_blocks), pad_per_xcd, blocking.parts, parts_divisor.magic, parts_divisor.shift,    \
         blocking.chunks_per_block, blocking.rows_per_block, static_cast<uint32_t>(pad_per_expert),                   \
         static_cast<uint32_t>(pad_groups_per_expert > 0 ? pad_groups_per_expert : 1), vectors, chunks, num_topk,     \
-        topk_shift)
+        topk_shift, xcds)
         const bool table = token_slots != nullptr;
         if (table && pad_blocks > 0)
             NANOEP_LAUNCH_ROWS(kLookupTable, true);

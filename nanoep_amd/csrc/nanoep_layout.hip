@@ -17,9 +17,21 @@ namespace {
 
 // Largest block of tokens a layout workgroup handles (one thread per token).
 constexpr int kMaxBlockTokens = 256;
-// An XCD's L2: the rows of one token block should fit it, since the dispatch walks the slot-order
-// list block by block and wants every re-use of a source row to hit that cache.
-constexpr int64_t kXcdL2Bytes = int64_t{4} << 20;
+// What the launch plans below depend on besides the batch: the forced settings and the device's XCD
+// count and L2 size (the rows of one window should fit an XCD's L2, since the dispatch walks the
+// slot-order list window by window and wants every re-use of a source row to hit that cache).
+struct Knobs {
+    int window_tokens;
+    int layout_launches;
+    int xcds;
+    int64_t l2_bytes;
+};
+
+Knobs current_knobs() {
+    const Tuning tuning = current_tuning();
+    const Topology topology = current_topology(tuning);
+    return {tuning.window_tokens, tuning.layout_launches, topology.xcds, topology.l2_bytes};
+}
 
 // Most blocks for which every assignment workgroup scans the block histograms itself.
 constexpr int kFusedScanMaxBlocks = 1024;
@@ -31,22 +43,23 @@ constexpr int kMaxWindowTokens = 1024;
 //    XCD's L2: 512 tokens up to 4096 elements, 256 up to 8192 (and when it is not known), then 128, 64.
 //    Rows of up to 1024 elements take 1024 tokens (half the L2: at 2048 elements a 1024-token window
 //    measured 8 % slower than a 512-token one, at 1024 and 512 elements 5 and 7 % faster).
-//  * The dispatch hands every XCD whole windows when there are at least eight of them (sixteen for
-//    1024-token windows): batches of more than 256 tokens take smaller windows (down to 64 tokens)
-//    to get there.
-int layout_window_tokens(int64_t tokens_total, int hidden) {
-    // NANOEP_WINDOW_TOKENS forces a window: any multiple of 32 up to 256 (one layout workgroup), or 512 / 1024
-    const int forced = g_tuning.window_tokens;
+//  * The dispatch hands every XCD whole windows when there are at least as many as XCDs (twice as
+//    many for 1024-token windows): batches of more than 256 tokens take smaller windows (down to 64
+//    tokens) to get there.
+// (sizes above are those of a 4 MiB L2 and 8 XCDs)
+int layout_window_tokens(int64_t tokens_total, int hidden, const Knobs& knobs) {
+    // WINDOW_TOKENS forces a window: any multiple of 32 up to 256 (one layout workgroup), or 512 / 1024
+    const int forced = knobs.window_tokens;
     if (forced >= 32 && forced % 32 == 0 && (forced <= 256 || forced == 512 || forced == 1024) && tokens_total > 256)
         return forced;
     int window = 256;
     if (hidden > 0)
         for (window = kMaxWindowTokens;
-             window > 64 && static_cast<int64_t>(window) * hidden * 2 > (window > 512 ? kXcdL2Bytes / 2 : kXcdL2Bytes); window /= 2) {
+             window > 64 && static_cast<int64_t>(window) * hidden * 2 > (window > 512 ? knobs.l2_bytes / 2 : knobs.l2_bytes); window /= 2) {
         }
     if (tokens_total <= 256 && window > 256)
         window = 256;  // one layout block: the whole layout is then a single launch
-    while (tokens_total > 256 && window > 64 && (tokens_total + window - 1) / window < (window > 512 ? 16 : 8))
+    while (tokens_total > 256 && window > 64 && (tokens_total + window - 1) / window < (window > 512 ? 2 * knobs.xcds : knobs.xcds))
         window /= 2;
     return window;
 }
@@ -55,10 +68,10 @@ int layout_window_tokens(int64_t tokens_total, int hidden) {
 // the LDS bit matrix ((L+1) rows of tokens/32 words plus a 16-bit prefix per word) asks for it.  A
 // window of 512 tokens is two workgroups' worth: the assignment pass orders the list by windows from
 // the block histograms (a 512-token workgroup makes the dispatch as fast and the layout 5 us slower).
-int layout_tokens_per_block(int64_t tokens_total, int64_t local_experts, int hidden) {
+int layout_tokens_per_block(int64_t tokens_total, int64_t local_experts, int hidden, const Knobs& knobs) {
     if (static_cast<size_t>(local_experts + 1) * 16 > kLayoutLdsBudget)  // four int32 arrays of the assignment kernel
         return 0;
-    const int window = layout_window_tokens(tokens_total, hidden);
+    const int window = layout_window_tokens(tokens_total, hidden, knobs);
     for (int tokens = window < kMaxBlockTokens ? window : kMaxBlockTokens; tokens >= 32; tokens = tokens / 2 / 32 * 32) {
         const size_t words = static_cast<size_t>(tokens / 32);
         if (static_cast<size_t>(local_experts + 1) * (words * 6 + 4) <= kLayoutLdsBudget)
@@ -69,28 +82,28 @@ int layout_tokens_per_block(int64_t tokens_total, int64_t local_experts, int hid
 
 // Layout blocks per window.  Windows of several blocks need every assignment workgroup to see the
 // block histograms (the two-launch plan); with a separate scan launch the window is the block.
-int layout_window_blocks(int64_t tokens_total, int64_t local_experts, int hidden, bool fused_scan) {
-    const int per_block = layout_tokens_per_block(tokens_total, local_experts, hidden);
-    const int window = layout_window_tokens(tokens_total, hidden);
+int layout_window_blocks(int64_t tokens_total, int64_t local_experts, int hidden, bool fused_scan, const Knobs& knobs) {
+    const int per_block = layout_tokens_per_block(tokens_total, local_experts, hidden, knobs);
+    const int window = layout_window_tokens(tokens_total, hidden, knobs);
     return per_block == 0 || !fused_scan || window <= per_block ? 1 : window / per_block;
 }
 
 // Whether the layout of this batch runs as two launches (see nanoep_layout).
-bool layout_uses_fused_scan(int64_t tokens_total, int64_t local_experts, int hidden) {
-    const int per_block = layout_tokens_per_block(tokens_total, local_experts, hidden);
+bool layout_uses_fused_scan(int64_t tokens_total, int64_t local_experts, int hidden, const Knobs& knobs) {
+    const int per_block = layout_tokens_per_block(tokens_total, local_experts, hidden, knobs);
     if (per_block == 0 || tokens_total == 0)
         return false;
     const int64_t blocks = (tokens_total + per_block - 1) / per_block;
-    const int forced = g_tuning.layout_launches;
+    const int forced = knobs.layout_launches;
     if (forced == 3)
         return false;
     return forced == 2 || blocks <= kFusedScanMaxBlocks;
 }
 
 // Smallest block any `hidden` can lead to for this batch: what the workspace is sized for.
-int layout_smallest_block(int64_t tokens_total, int64_t local_experts) {
-    const int narrow = layout_tokens_per_block(tokens_total, local_experts, 1 << 20);
-    const int wide = layout_tokens_per_block(tokens_total, local_experts, 8);
+int layout_smallest_block(int64_t tokens_total, int64_t local_experts, const Knobs& knobs) {
+    const int narrow = layout_tokens_per_block(tokens_total, local_experts, 1 << 20, knobs);
+    const int wide = layout_tokens_per_block(tokens_total, local_experts, 8, knobs);
     return narrow < wide ? narrow : wide;
 }
 
@@ -103,8 +116,8 @@ struct LayoutWorkspace {
     size_t bytes;
 };
 
-LayoutWorkspace carve_layout_workspace(void* base, int64_t tokens, int topk, int64_t local_experts) {
-    const int per_block = layout_smallest_block(tokens, local_experts);
+LayoutWorkspace carve_layout_workspace(void* base, int64_t tokens, int topk, int64_t local_experts, const Knobs& knobs) {
+    const int per_block = layout_smallest_block(tokens, local_experts, knobs);
     const int64_t blocks = per_block == 0 ? 0 : (tokens + per_block - 1) / per_block;
     auto* cursor = static_cast<uint8_t*>(base);
     size_t offset = 0;
@@ -845,7 +858,7 @@ int check_layout_arguments(const int64_t* topk_idx, int64_t num_tokens, int num_
                            int expand, int hidden, const int32_t* recv_metadata, const int64_t* expert_counts,
                            const int64_t* expert_offsets, const int64_t* dst_slots, const int64_t* send_counts,
                            const int64_t* topk_snapshot, const int64_t* recv_rank_prefix, const int64_t* slot_order,
-                           const int64_t* host_counts) {
+                           const int64_t* host_counts, const Knobs& knobs) {
     if (num_tokens < 0 || num_tokens > INT32_MAX || num_topk <= 0 || num_topk > kMaxTopk || num_local_experts <= 0 ||
         num_local_experts >= (int64_t{1} << (31 - kRankBits)) || alignment <= 0 || alignment > (int64_t{1} << 31) || hidden < 0)
         return NANOEP_ERR_INVALID_ARGUMENT;
@@ -857,7 +870,7 @@ int check_layout_arguments(const int64_t* topk_idx, int64_t num_tokens, int num_
     // the slot-order list packs token * K + k into 32 bits and only exists for the expanded layout
     if (slot_order != nullptr && (!expand || num_tokens * num_topk >= (int64_t{1} << 31)))
         return NANOEP_ERR_INVALID_ARGUMENT;
-    if (layout_tokens_per_block(num_tokens, num_local_experts, hidden) == 0)
+    if (layout_tokens_per_block(num_tokens, num_local_experts, hidden, knobs) == 0)
         return NANOEP_ERR_INVALID_ARGUMENT;
     return NANOEP_OK;
 }
@@ -867,8 +880,8 @@ int enqueue_layout(const int64_t* topk_idx, int64_t num_tokens, int num_topk, in
                    int expand, int hidden, int32_t* recv_metadata, int64_t* expert_counts, int64_t* expert_offsets,
                    int64_t* dst_slots, int64_t* send_counts, int64_t* topk_snapshot, int64_t* recv_rank_prefix,
                    int32_t* token_slots, int64_t* slot_order, const LayoutWorkspace& ws, int64_t* host_counts,
-                   void* stream_handle) {
-    const int tokens_per_block = layout_tokens_per_block(num_tokens, num_local_experts, hidden);
+                   void* stream_handle, const Knobs& knobs) {
+    const int tokens_per_block = layout_tokens_per_block(num_tokens, num_local_experts, hidden, knobs);
     const int64_t blocks64 = (num_tokens + tokens_per_block - 1) / tokens_per_block;
     const int blocks = static_cast<int>(blocks64);
     const int experts = static_cast<int>(num_local_experts);
@@ -876,15 +889,17 @@ int enqueue_layout(const int64_t* topk_idx, int64_t num_tokens, int num_topk, in
     auto stream = static_cast<hipStream_t>(stream_handle);
 
     __atomic_store_n(&host_counts[0], int64_t{-1}, __ATOMIC_RELEASE);
-    const int count_threads = tokens_per_block < kWave ? kWave : tokens_per_block;
+    // whole wavefronts: the kernels' scans take a wavefront's sums from its last lane (a forced window of
+    // 96, 160 or 224 tokens would otherwise leave the experts of a trailing half wavefront out)
+    const int count_threads = (tokens_per_block + kWave - 1) / kWave * kWave;
     // Two launches while every block can afford to sum the block histograms itself (blocks x (L+1)
     // loads from L2, spread over the workgroup): measured faster than the single-workgroup scan up to
     // 1024 blocks whatever the expert count (8192 tokens, 256 experts: 21 against 27 us; 262144
     // tokens: 159 against 198 us).  Beyond, the blocks^2 loads lose (2^20 tokens, 8 experts: 124
     // against 67 us) and a third launch does the scan once.
-    const bool fused_scan = layout_uses_fused_scan(num_tokens, num_local_experts, hidden);
-    const int forced_launches = g_tuning.layout_launches;
-    const int window_blocks = layout_window_blocks(num_tokens, num_local_experts, hidden, fused_scan);
+    const bool fused_scan = layout_uses_fused_scan(num_tokens, num_local_experts, hidden, knobs);
+    const int forced_launches = knobs.layout_launches;
+    const int window_blocks = layout_window_blocks(num_tokens, num_local_experts, hidden, fused_scan, knobs);
     hipError_t launch_status = hipSuccess;
     with_topk_cap(num_topk, [&](auto cap) {
         constexpr int kCap = decltype(cap)::value;
@@ -933,6 +948,167 @@ int enqueue_layout(const int64_t* topk_idx, int64_t num_tokens, int num_topk, in
     return NANOEP_OK;
 }
 
+// ---- The private handle tensors rebuilt from a handle's own public ones -------------------------
+//
+// A handle that went through a caller keeping only the reference's seven tensors has lost the slot
+// table and the slot-order list.  Both are functions of dst_slots and recv_metadata alone:
+// token_slots[t][k] = recv_metadata[dst_slots[t]][2 + k] (-1 when the token was not sent or the slot
+// lies outside [0, C)), and the list is, window of consecutive tokens by window, the valid (slot,
+// t * K + k) pairs in ascending slot order.  Nothing here looks at the routing ids or assumes the
+// slots were made by this library: the handle is followed as it is written.
+
+// Largest number of list entries one window may hold here: the sort runs in LDS, 8 bytes an entry.
+constexpr int kRebuildMaxWindowEntries = 4096;
+constexpr int kRebuildThreads = 1024;
+
+// Tokens of one window of a rebuilt list: the layout's own choice for this batch, halved until a
+// window's T * K entries fit the sort.
+int rebuild_window_tokens(int64_t tokens_total, int num_topk, int hidden, const Knobs& knobs) {
+    int window = layout_window_tokens(tokens_total, hidden, knobs);
+    if (window > kMaxWindowTokens)
+        window = kMaxWindowTokens;
+    while (window > 32 && static_cast<int64_t>(window) * num_topk > kRebuildMaxWindowEntries)
+        window /= 2;
+    return window;
+}
+
+// One workgroup per window: the slot table of the window's tokens and the number of valid entries.
+__global__ void __launch_bounds__(kRebuildThreads) rebuild_table_kernel(const int32_t* __restrict__ recv_metadata,  // [N][K+2]
+                                                                       const int64_t* __restrict__ dst_slots,     // [T]
+                                                                       int64_t recv_count,
+                                                                       int64_t out_rows,
+                                                                       int64_t num_tokens,
+                                                                       int num_topk,
+                                                                       int window_tokens,
+                                                                       int32_t* __restrict__ token_slots,  // [T][K]
+                                                                       int32_t* __restrict__ window_counts) {
+    __shared__ int valid_entries;
+    if (threadIdx.x == 0)
+        valid_entries = 0;
+    __syncthreads();
+    const int64_t first = static_cast<int64_t>(blockIdx.x) * window_tokens * num_topk;
+    const int64_t batch_end = num_tokens * num_topk;
+    const int64_t window_end = first + static_cast<int64_t>(window_tokens) * num_topk;
+    const int64_t end = window_end < batch_end ? window_end : batch_end;
+    int mine = 0;
+    for (int64_t flat = first + threadIdx.x; flat < end; flat += kRebuildThreads) {
+        const int64_t token = flat / num_topk;
+        const int k = static_cast<int>(flat - token * num_topk);
+        const int64_t row = dst_slots[token];
+        int32_t slot = -1;
+        if (row >= 0 && row < recv_count)
+            slot = recv_metadata[row * (num_topk + 2) + 2 + k];
+        if (slot < 0 || slot >= out_rows)
+            slot = -1;
+        token_slots[flat] = slot;
+        mine += slot >= 0;
+    }
+#pragma unroll
+    for (int distance = kWave / 2; distance > 0; distance /= 2)
+        mine += __shfl_xor(mine, distance, kWave);
+    if ((threadIdx.x & (kWave - 1)) == 0 && mine != 0)
+        atomicAdd(&valid_entries, mine);
+    __syncthreads();
+    if (threadIdx.x == 0)
+        window_counts[blockIdx.x] = valid_entries;
+}
+
+// One workgroup per window: sorts the window's (slot, source) pairs in LDS (bitonic network over
+// `sort_size` keys, a power of two; masked choices sort behind everything as the largest key) and
+// writes the valid ones where the list has room for them: behind the entries of all earlier
+// windows.  The rest of the buffer reads -1 up to the count word, as the layout leaves it.
+__global__ void __launch_bounds__(kRebuildThreads) rebuild_order_kernel(const int32_t* __restrict__ token_slots,    // [T][K]
+                                                                       const int32_t* __restrict__ window_counts,  // [windows]
+                                                                       int64_t num_tokens,
+                                                                       int num_topk,
+                                                                       int window_tokens,
+                                                                       int num_windows,
+                                                                       int sort_size,
+                                                                       int64_t* __restrict__ slot_order,
+                                                                       int64_t capacity_entries,
+                                                                       int64_t* host_count,  // pinned, or null
+                                                                       int64_t host_tag) {
+    extern __shared__ int64_t sort_keys[];
+    __shared__ int64_t before_sum;
+    __shared__ int64_t total_sum;
+    const int window = blockIdx.x;
+    const int tid = threadIdx.x;
+    if (tid == 0) {
+        before_sum = 0;
+        total_sum = 0;
+    }
+    const int64_t first = static_cast<int64_t>(window) * window_tokens * num_topk;
+    const int64_t batch_end = num_tokens * num_topk;
+    const int64_t window_end = first + static_cast<int64_t>(window_tokens) * num_topk;
+    const int64_t end = window_end < batch_end ? window_end : batch_end;
+    for (int i = tid; i < sort_size; i += kRebuildThreads) {
+        const int64_t flat = first + i;
+        int64_t key = INT64_MAX;
+        if (flat < end) {
+            const int32_t slot = token_slots[flat];
+            if (slot >= 0)
+                key = (static_cast<int64_t>(slot) << 32) | static_cast<int64_t>(static_cast<uint32_t>(flat));
+        }
+        sort_keys[i] = key;
+    }
+    __syncthreads();
+    // valid entries of the windows before this one, and of all windows
+    int64_t before = 0, total = 0;
+    for (int w = tid; w < num_windows; w += kRebuildThreads) {
+        const int count = window_counts[w];
+        total += count;
+        before += w < window ? count : 0;
+    }
+#pragma unroll
+    for (int distance = kWave / 2; distance > 0; distance /= 2) {
+        before += __shfl_xor(before, distance, kWave);
+        total += __shfl_xor(total, distance, kWave);
+    }
+    if ((tid & (kWave - 1)) == 0 && total != 0) {
+        atomicAdd(reinterpret_cast<unsigned long long*>(&before_sum), static_cast<unsigned long long>(before));
+        atomicAdd(reinterpret_cast<unsigned long long*>(&total_sum), static_cast<unsigned long long>(total));
+    }
+    for (int size = 2; size <= sort_size; size *= 2) {
+        for (int stride = size / 2; stride > 0; stride /= 2) {
+            for (int i = tid; i < sort_size; i += kRebuildThreads) {
+                const int partner = i ^ stride;
+                if (partner > i) {
+                    const bool ascending = (i & size) == 0;
+                    const int64_t a = sort_keys[i], b = sort_keys[partner];
+                    if ((a > b) == ascending) {
+                        sort_keys[i] = b;
+                        sort_keys[partner] = a;
+                    }
+                }
+            }
+            __syncthreads();
+        }
+    }
+    __syncthreads();
+    const int64_t assigned_before = before_sum;
+    const int64_t assigned = total_sum;
+    const int own = window_counts[window];
+    for (int i = tid; i < own; i += kRebuildThreads)
+        slot_order[assigned_before + i] = sort_keys[i];
+    // the unused tail: every window clears as many entries as it has masked choices, the last one also
+    // what lies between the batch's last choice and the count word
+    const int64_t own_entries = end - first;
+    int64_t* tail = slot_order + assigned + (first - assigned_before);
+    for (int64_t i = tid; i < own_entries - own; i += kRebuildThreads)
+        tail[i] = -1;
+    if (window == num_windows - 1) {
+        for (int64_t i = batch_end + tid; i < capacity_entries; i += kRebuildThreads)
+            slot_order[i] = -1;
+        if (tid == 0) {
+            slot_order[capacity_entries] = assigned;
+            if (host_count != nullptr) {
+                __threadfence_system();
+                __hip_atomic_store(host_count, host_tag | assigned, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_SYSTEM);
+            }
+        }
+    }
+}
+
 // Address of this file's `scratch` array on the current device, resolved once per device (each GPU
 // holds its own copy at its own address).
 constexpr int kMaxDevices = 64;
@@ -964,27 +1140,25 @@ using namespace nanoep;
 extern "C" {
 
 size_t nanoep_layout_workspace_bytes(int64_t num_tokens, int num_topk, int64_t num_local_experts) {
-    refresh_tuning();
     if (num_tokens < 0 || num_topk <= 0 || num_local_experts <= 0)
         return 0;
-    return carve_layout_workspace(nullptr, num_tokens, num_topk, num_local_experts).bytes;
+    return carve_layout_workspace(nullptr, num_tokens, num_topk, num_local_experts, current_knobs()).bytes;
 }
 
 int nanoep_layout_block_tokens(int64_t num_tokens, int64_t num_local_experts, int hidden) {
-    refresh_tuning();
     if (num_local_experts <= 0 || num_tokens < 0 || hidden < 0)
         return 0;
+    const Knobs knobs = current_knobs();
     // tokens the slot-order list is ordered by: the layout workgroup's tokens times the blocks of a window
-    const int per_block = layout_tokens_per_block(num_tokens, num_local_experts, hidden);
-    const bool fused = layout_uses_fused_scan(num_tokens, num_local_experts, hidden);
-    return per_block * layout_window_blocks(num_tokens, num_local_experts, hidden, fused);
+    const int per_block = layout_tokens_per_block(num_tokens, num_local_experts, hidden, knobs);
+    const bool fused = layout_uses_fused_scan(num_tokens, num_local_experts, hidden, knobs);
+    return per_block * layout_window_blocks(num_tokens, num_local_experts, hidden, fused, knobs);
 }
 
 int64_t nanoep_slot_order_entries(int64_t num_tokens, int num_topk, int64_t num_local_experts) {
-    refresh_tuning();
     if (num_tokens < 0 || num_topk <= 0 || num_local_experts <= 0)
         return 0;
-    if (layout_smallest_block(num_tokens, num_local_experts) == 0 || num_tokens == 0)
+    if (layout_smallest_block(num_tokens, num_local_experts, current_knobs()) == 0 || num_tokens == 0)
         return 0;
     // whole blocks of any size the layout may take, then the count word
     return (num_tokens + kMaxBlockTokens - 1) / kMaxBlockTokens * kMaxBlockTokens * num_topk + 1;
@@ -995,20 +1169,20 @@ int nanoep_layout(const int64_t* topk_idx, int64_t num_tokens, int num_topk, int
                   int64_t* expert_offsets, int64_t* dst_slots, int64_t* send_counts, int64_t* topk_snapshot,
                   int64_t* recv_rank_prefix, int32_t* token_slots, int64_t* slot_order, void* workspace,
                   size_t workspace_bytes, int64_t* host_counts, void* stream_handle) {
-    refresh_tuning();
+    const Knobs knobs = current_knobs();
     const int status = check_layout_arguments(topk_idx, num_tokens, num_topk, num_local_experts, alignment, expand, hidden,
                                               recv_metadata, expert_counts, expert_offsets, dst_slots, send_counts, topk_snapshot,
-                                              recv_rank_prefix, slot_order, host_counts);
+                                              recv_rank_prefix, slot_order, host_counts, knobs);
     if (status != NANOEP_OK)
         return status;
     if (workspace == nullptr)
         return NANOEP_ERR_INVALID_ARGUMENT;
-    const LayoutWorkspace ws = carve_layout_workspace(workspace, num_tokens, num_topk, num_local_experts);
+    const LayoutWorkspace ws = carve_layout_workspace(workspace, num_tokens, num_topk, num_local_experts, knobs);
     if (ws.bytes > workspace_bytes)
         return NANOEP_ERR_WORKSPACE;
     return enqueue_layout(topk_idx, num_tokens, num_topk, num_local_experts, alignment, expand, hidden, recv_metadata, expert_counts,
                           expert_offsets, dst_slots, send_counts, topk_snapshot, recv_rank_prefix, token_slots, slot_order, ws,
-                          host_counts, stream_handle);
+                          host_counts, stream_handle, knobs);
 }
 
 int nanoep_layout_static(const int64_t* topk_idx, int64_t num_tokens, int num_topk, int64_t num_local_experts,
@@ -1016,14 +1190,14 @@ int nanoep_layout_static(const int64_t* topk_idx, int64_t num_tokens, int num_to
                          int64_t* expert_offsets, int64_t* dst_slots, int64_t* send_counts, int64_t* topk_snapshot,
                          int64_t* recv_rank_prefix, int32_t* token_slots, int64_t* slot_order, int64_t* host_counts,
                          void* stream_handle) {
-    refresh_tuning();
+    const Knobs knobs = current_knobs();
     const int status = check_layout_arguments(topk_idx, num_tokens, num_topk, num_local_experts, alignment, expand, hidden,
                                               recv_metadata, expert_counts, expert_offsets, dst_slots, send_counts, topk_snapshot,
-                                              recv_rank_prefix, slot_order, host_counts);
+                                              recv_rank_prefix, slot_order, host_counts, knobs);
     if (status != NANOEP_OK)
         return status;
     // the size is checked before any device is touched
-    if (carve_layout_workspace(nullptr, num_tokens, num_topk, num_local_experts).bytes > NANOEP_STATIC_SCRATCH_BYTES)
+    if (carve_layout_workspace(nullptr, num_tokens, num_topk, num_local_experts, knobs).bytes > NANOEP_STATIC_SCRATCH_BYTES)
         return NANOEP_ERR_SCRATCH_LIMIT;
     void* base = nullptr;
     const int scratch_status = static_scratch_of_current_device(&base);
@@ -1031,10 +1205,59 @@ int nanoep_layout_static(const int64_t* topk_idx, int64_t num_tokens, int num_to
         return scratch_status;
     // Nothing in the workspace has to start at zero: the count pass writes every histogram row, status
     // word, rank entry and receive row that the later passes of the same call read.
-    const LayoutWorkspace ws = carve_layout_workspace(base, num_tokens, num_topk, num_local_experts);
+    const LayoutWorkspace ws = carve_layout_workspace(base, num_tokens, num_topk, num_local_experts, knobs);
     return enqueue_layout(topk_idx, num_tokens, num_topk, num_local_experts, alignment, expand, hidden, recv_metadata, expert_counts,
                           expert_offsets, dst_slots, send_counts, topk_snapshot, recv_rank_prefix, token_slots, slot_order, ws,
-                          host_counts, stream_handle);
+                          host_counts, stream_handle, knobs);
+}
+
+size_t nanoep_rebuild_workspace_bytes(int64_t num_tokens, int num_topk) {
+    if (num_tokens < 0 || num_topk <= 0 || num_topk > kMaxTopk)
+        return 0;
+    // one int32 per window of the smallest size a rebuilt list takes
+    return align_up(static_cast<size_t>((num_tokens + 31) / 32) * 4, 256) + 256;
+}
+
+int nanoep_rebuild_window_tokens(int64_t num_tokens, int num_topk, int hidden) {
+    if (num_tokens < 0 || num_topk <= 0 || num_topk > kMaxTopk || hidden < 0)
+        return 0;
+    return rebuild_window_tokens(num_tokens, num_topk, hidden, current_knobs());
+}
+
+int nanoep_rebuild_order(const int32_t* recv_metadata, const int64_t* dst_slots, int64_t recv_count, int64_t expanded_capacity,
+                         int64_t num_tokens, int num_topk, int64_t num_local_experts, int hidden, int32_t* token_slots,
+                         int64_t* slot_order, void* workspace, size_t workspace_bytes, int64_t* host_count, int64_t host_tag,
+                         void* stream_handle) {
+    if (num_tokens <= 0 || num_tokens > INT32_MAX || num_topk <= 0 || num_topk > kMaxTopk || num_local_experts <= 0 || hidden < 0 ||
+        recv_count < 0 || recv_count > num_tokens || expanded_capacity < 0 || expanded_capacity > INT32_MAX ||
+        num_tokens * num_topk >= (int64_t{1} << 31))
+        return NANOEP_ERR_INVALID_ARGUMENT;
+    if (dst_slots == nullptr || token_slots == nullptr || slot_order == nullptr || workspace == nullptr ||
+        (recv_count > 0 && recv_metadata == nullptr) || host_tag < 0 || (host_tag & 0xffffffffll) != 0)
+        return NANOEP_ERR_INVALID_ARGUMENT;
+    const Knobs knobs = current_knobs();
+    if (layout_smallest_block(num_tokens, num_local_experts, knobs) == 0)
+        return NANOEP_ERR_INVALID_ARGUMENT;  // no slot-order buffer exists for this geometry
+    if (nanoep_rebuild_workspace_bytes(num_tokens, num_topk) > workspace_bytes)
+        return NANOEP_ERR_WORKSPACE;
+    const int window = rebuild_window_tokens(num_tokens, num_topk, hidden, knobs);
+    const int64_t windows = (num_tokens + window - 1) / window;
+    int sort_size = 2;
+    while (sort_size < window * num_topk)
+        sort_size *= 2;
+    const int64_t capacity_entries = (num_tokens + kMaxBlockTokens - 1) / kMaxBlockTokens * kMaxBlockTokens * num_topk;
+    auto* window_counts = static_cast<int32_t*>(workspace);
+    auto stream = static_cast<hipStream_t>(stream_handle);
+    if (host_count != nullptr)
+        __atomic_store_n(host_count, int64_t{-1}, __ATOMIC_RELEASE);
+    rebuild_table_kernel<<<static_cast<unsigned>(windows), kRebuildThreads, 0, stream>>>(
+        recv_metadata, dst_slots, recv_count, expanded_capacity, num_tokens, num_topk, window, token_slots, window_counts);
+    NANOEP_HIP_TRY(hipGetLastError());
+    rebuild_order_kernel<<<static_cast<unsigned>(windows), kRebuildThreads, static_cast<size_t>(sort_size) * 8, stream>>>(
+        token_slots, window_counts, num_tokens, num_topk, window, static_cast<int>(windows), sort_size, slot_order, capacity_entries,
+        host_count, host_tag);
+    NANOEP_HIP_TRY(hipGetLastError());
+    return NANOEP_OK;
 }
 
 int nanoep_wait_counts(int64_t* host_counts, void* stream_handle, double timeout_seconds,
@@ -1059,8 +1282,19 @@ int nanoep_wait_counts(int64_t* host_counts, void* stream_handle, double timeout
             timespec now{};
             clock_gettime(CLOCK_MONOTONIC, &now);
             const double elapsed = (now.tv_sec - start.tv_sec) + 1e-9 * (now.tv_nsec - start.tv_nsec);
-            if (elapsed > timeout_seconds)
+            if (elapsed > timeout_seconds) {
+                // a last look at the mailbox, and at a stream that may have failed rather than stalled
+                if (__atomic_load_n(&host_counts[0], __ATOMIC_ACQUIRE) >= 0)
+                    break;
+                if (stream != nullptr) {
+                    const hipError_t state = hipStreamQuery(stream);
+                    if (state != hipSuccess && state != hipErrorNotReady) {
+                        g_last_hip_error = state;
+                        return NANOEP_ERR_HIP;
+                    }
+                }
                 return NANOEP_ERR_TIMEOUT;
+            }
             if (elapsed < next_stream_check)
                 continue;
             next_stream_check = elapsed + 100e-6;

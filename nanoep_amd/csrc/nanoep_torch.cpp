@@ -45,10 +45,17 @@ constexpr double kCountTimeoutSeconds = 60.0;
 // Fresh expanded dispatches whose private handle tensors the runtime keeps for callers that hand
 // back only the reference's seven.
 constexpr size_t kRememberedHandles = 4;
+// Seven-tensor handles whose private tensors were rebuilt from the handle itself and are kept for
+// its later replays.
+constexpr size_t kRebuiltHandles = 64;
+// Rebuilding pays from this many payload bytes written per replay on (below, the token-order walk's
+// loss is smaller than what the two extra launches cost a handle that is replayed once or twice).
+constexpr int64_t kRebuildPayloadBytes = int64_t{48} << 20;
 
-int env_switch(const char* name) {  // -1: not set
-    const char* text = std::getenv(name);
-    return text == nullptr || *text == '\0' ? -1 : std::atoi(text);
+// One of the library's tuning switches (no environment access: the library read it once).
+int tuning_switch(const char* name) {
+    int value = -1;
+    return nanoep_get_tuning(name, &value) == NANOEP_OK ? value : -1;
 }
 
 void check_status(int status, const char* what) {
@@ -103,11 +110,18 @@ class PeerRuntime {
         host_counts_ = static_cast<int64_t*>(mailbox);
         for (int i = 0; i < NANOEP_HOST_COUNT_WORDS; ++i)
             host_counts_[i] = -1;
+        void* words = nullptr;
+        check_hip(hipHostMalloc(&words, kRebuiltHandles * sizeof(int64_t), hipHostMallocMapped | hipHostMallocCoherent), "hipHostMalloc");
+        rebuilt_counts_ = static_cast<int64_t*>(words);
+        for (size_t i = 0; i < kRebuiltHandles; ++i)
+            rebuilt_counts_[i] = -1;
     }
 
     ~PeerRuntime() {
         if (host_counts_ != nullptr)
             (void)hipHostFree(host_counts_);
+        if (rebuilt_counts_ != nullptr)
+            (void)hipHostFree(rebuilt_counts_);
     }
 
     PeerRuntime(const PeerRuntime&) = delete;
@@ -259,8 +273,111 @@ class PeerRuntime {
 
     void forget_private() {
         std::deque<RememberedHandle> retired;
+        std::array<std::shared_ptr<RebuiltHandle>, kRebuiltHandles> retired_rebuilt;
         std::lock_guard<std::mutex> lock(private_mutex_);
         retired.swap(remembered_);
+        retired_rebuilt.swap(rebuilt_);
+    }
+
+    // The private tensors of a seven-tensor handle, rebuilt from the handle's own dst_slots and
+    // recv_metadata (nanoep_rebuild_order) and kept for its later replays.  An entry is recognised
+    // like a remembered one, and in addition by the identity and version of the two tensors it was
+    // built from: a handle edited through torch is rebuilt.  `count` is where the device publishes the
+    // number of list entries (tagged, so that a late store of an entry that used this word before is
+    // never taken for this one's): until it is there, replays read the count on the device.
+    struct RebuiltHandle {
+        c10::weak_intrusive_ptr<c10::TensorImpl> snapshot;
+        uint32_t snapshot_version = 0, metadata_version = 0, slots_version = 0;
+        const void* snapshot_data = nullptr;
+        const void* metadata_data = nullptr;
+        const void* slots_data = nullptr;
+        int64_t rows = 0, capacity = 0;
+        torch::Tensor table, order;  // views of one allocation
+        c10::Event ready{c10::DeviceType::CUDA};
+        hipStream_t made_on = nullptr;
+        int64_t* count = nullptr;  // pinned host word
+        int64_t tag = 0;
+
+        explicit RebuiltHandle(const torch::Tensor& snapshot_tensor) : snapshot(snapshot_tensor.getIntrusivePtr()) {}
+
+        // the number of list entries once the device has published it, else -1
+        int64_t published_entries() const {
+            const int64_t word = __atomic_load_n(count, __ATOMIC_ACQUIRE);
+            return word >= 0 && (word & ~int64_t{0xffffffff}) == tag ? (word & int64_t{0xffffffff}) : -1;
+        }
+    };
+
+    std::shared_ptr<RebuiltHandle> find_rebuilt(const std::vector<torch::Tensor>& metadata, int64_t capacity) const {
+        std::lock_guard<std::mutex> lock(private_mutex_);
+        if (closed_.load() || metadata.size() != 7)
+            return nullptr;
+        for (const auto& entry : rebuilt_) {
+            if (!entry)
+                continue;
+            const auto alive = entry->snapshot.lock();
+            if (alive && alive.get() == metadata[5].unsafeGetTensorImpl() && metadata[5].data_ptr() == entry->snapshot_data &&
+                tensor_version(metadata[5]) == entry->snapshot_version && metadata[0].data_ptr() == entry->metadata_data &&
+                tensor_version(metadata[0]) == entry->metadata_version && metadata[3].data_ptr() == entry->slots_data &&
+                tensor_version(metadata[3]) == entry->slots_version && metadata[0].size(0) == entry->rows && capacity == entry->capacity)
+                return entry;
+        }
+        return nullptr;
+    }
+
+    // A new entry for this handle (tensors not yet set, not yet findable), with a count word and tag of
+    // its own.  It takes the place of an entry whose handle is gone, else of the oldest one;
+    // publish_rebuilt makes it findable once its tensors are there.
+    std::shared_ptr<RebuiltHandle> new_rebuilt(const std::vector<torch::Tensor>& metadata, int64_t capacity) {
+        auto entry = std::make_shared<RebuiltHandle>(metadata[5]);
+        entry->snapshot_version = tensor_version(metadata[5]);
+        entry->metadata_version = tensor_version(metadata[0]);
+        entry->slots_version = tensor_version(metadata[3]);
+        entry->snapshot_data = metadata[5].data_ptr();
+        entry->metadata_data = metadata[0].data_ptr();
+        entry->slots_data = metadata[3].data_ptr();
+        entry->rows = metadata[0].size(0);
+        entry->capacity = capacity;
+        std::shared_ptr<RebuiltHandle> retired;  // released after the lock
+        std::lock_guard<std::mutex> lock(private_mutex_);
+        size_t at = kRebuiltHandles;
+        for (size_t i = 0; i < kRebuiltHandles && at == kRebuiltHandles; ++i)
+            if (!rebuilt_[i] || rebuilt_[i]->snapshot.expired())
+                at = i;
+        if (at == kRebuiltHandles)
+            at = next_rebuilt_++ % kRebuiltHandles;
+        entry->count = rebuilt_counts_ + at;
+        entry->tag = (++rebuilt_generation_ & 0x3fffffff) << 32;
+        retired = std::move(rebuilt_[at]);
+        ++rebuilds_;
+        return entry;
+    }
+
+    void publish_rebuilt(const std::shared_ptr<RebuiltHandle>& entry) {
+        std::shared_ptr<RebuiltHandle> retired;  // released after the lock
+        std::lock_guard<std::mutex> lock(private_mutex_);
+        if (closed_.load())
+            return;
+        retired = std::move(rebuilt_[entry->count - rebuilt_counts_]);
+        rebuilt_[entry->count - rebuilt_counts_] = entry;
+    }
+
+    // number of seven-tensor handles whose private tensors were rebuilt (for tests)
+    int64_t rebuilds() const {
+        std::lock_guard<std::mutex> lock(private_mutex_);
+        return rebuilds_;
+    }
+
+    // Scratch of the layout kernels, kept between fresh dispatches (they take turns at the mailbox and
+    // a turn ends when the layout has published its counts, but its last workgroups may still be reading
+    // the scratch: the buffer is only handed out again to a call on the stream it was last used on,
+    // where the launches are ordered; a call on another stream gets a buffer of its own, which is then
+    // the one that is kept).  Called with the mailbox held.
+    torch::Tensor layout_workspace(size_t bytes, hipStream_t stream, const torch::TensorOptions& options) {
+        if (!workspace_.defined() || static_cast<size_t>(workspace_.numel()) < bytes || workspace_stream_ != stream) {
+            workspace_ = torch::empty({static_cast<int64_t>(bytes)}, options);
+            workspace_stream_ = stream;
+        }
+        return workspace_;
     }
 
     py::bytes export_local_handle() const {
@@ -320,6 +437,10 @@ class PeerRuntime {
         TORCH_CHECK(mappings_closed_, "Call close_peer_mappings() before close()");
         window_ = torch::Tensor();
         forget_private();
+        {
+            std::lock_guard<std::mutex> lock(counts_mutex_);
+            workspace_ = torch::Tensor();
+        }
         closed_.store(true);
     }
 
@@ -349,6 +470,13 @@ class PeerRuntime {
     std::atomic<bool> prefers_exact_outputs_{false};
     std::atomic<int64_t> valid_share_65536_{65536};
     std::deque<RememberedHandle> remembered_;  // newest first
+    std::array<std::shared_ptr<RebuiltHandle>, kRebuiltHandles> rebuilt_;
+    int64_t* rebuilt_counts_ = nullptr;  // pinned, one word per entry of rebuilt_
+    size_t next_rebuilt_ = 0;
+    int64_t rebuilt_generation_ = 0;
+    int64_t rebuilds_ = 0;
+    torch::Tensor workspace_;
+    hipStream_t workspace_stream_ = nullptr;
     mutable int64_t private_recalls_ = 0;
     mutable std::mutex private_mutex_;
     int64_t last_barrier_epoch_ = 0;
@@ -518,6 +646,41 @@ void order_comm_after_inputs(const Stream& comm, const Stream& compute, int64_t 
     }
 }
 
+// The private tensors of a seven-tensor expanded handle the runtime does not remember: found among
+// the ones rebuilt earlier, or rebuilt now on `stream` (the current stream of the allocator).
+std::shared_ptr<PeerRuntime::RebuiltHandle> private_tensors_of(PeerRuntime& runtime, const std::vector<torch::Tensor>& metadata,
+                                                               int64_t capacity, int64_t tokens, int64_t topk, int64_t local_experts,
+                                                               int64_t hidden, const Stream& stream) {
+    auto entry = runtime.find_rebuilt(metadata, capacity);
+    if (entry) {
+        if (entry->made_on != stream.stream()) {
+            // built on another stream: wait for it unless it is long done, and tell the allocator
+            if (!entry->ready.query())
+                stream.unwrap().wait(entry->ready);
+            entry->order.record_stream(stream.unwrap());  // the table is a view of the same allocation
+        }
+        return entry;
+    }
+    entry = runtime.new_rebuilt(metadata, capacity);
+    const int64_t order_words = nanoep_slot_order_entries(tokens, static_cast<int>(topk), local_experts);
+    const size_t workspace_bytes = nanoep_rebuild_workspace_bytes(tokens, static_cast<int>(topk));
+    const int64_t table_words = (tokens * topk + 1) / 2;
+    const int64_t workspace_words = static_cast<int64_t>((workspace_bytes + 7) / 8);
+    // one allocation: slot-order buffer | slot table | the rebuild's scratch
+    auto storage = torch::empty({order_words + table_words + workspace_words}, metadata[3].options());
+    entry->order = storage.narrow(0, 0, order_words);
+    entry->table = storage.narrow(0, order_words, table_words).view(torch::kInt32).narrow(0, 0, tokens * topk).view({tokens, topk});
+    check_status(nanoep_rebuild_order(metadata[0].data_ptr<int32_t>(), metadata[3].data_ptr<int64_t>(), metadata[0].size(0), capacity, tokens,
+                                      static_cast<int>(topk), local_experts, static_cast<int>(hidden), entry->table.data_ptr<int32_t>(),
+                                      entry->order.data_ptr<int64_t>(), storage.data_ptr<int64_t>() + order_words + table_words,
+                                      static_cast<size_t>(workspace_words) * 8, entry->count, entry->tag, stream.stream()),
+                 "rebuild_order");
+    entry->made_on = stream.stream();
+    entry->ready.record(stream.unwrap());
+    runtime.publish_rebuilt(entry);
+    return entry;
+}
+
 }  // namespace
 
 using DispatchResult =
@@ -637,13 +800,37 @@ DispatchResult dispatch(PeerRuntime& runtime,
         // A handle that went through the reference's Python class carries the seven tensors of the
         // reference only.  If it is one of this runtime's latest fresh dispatches, the runtime still
         // has its private tensors and the payload takes the slot-order walk
-        // (NANOEP_RECALL_ORDER=0 switches that off).  Any other seven-tensor handle is followed as it
+        // (the RECALL_ORDER switch set to 0 turns that off).  Any other seven-tensor handle is followed as it
         // is written, in token order through its own dst_slots and recv_metadata: whatever row and
         // slot order it describes is the order the rows land in.
-        if (expand && recv_count > 0 && env_switch("NANOEP_RECALL_ORDER") != 0)
-            runtime.recall_private(metadata, alignment);
-        if (recv_count > 0)
-            launch_permute(view_of(metadata), recv_count, expanded_capacity);
+        bool has_private = metadata.size() > 7;
+        if (expand && recv_count > 0 && !has_private && tuning_switch("RECALL_ORDER") != 0)
+            has_private = runtime.recall_private(metadata, alignment);
+        if (recv_count > 0) {
+            HandleView view = view_of(metadata);
+            // A seven-tensor handle the runtime does not remember: its private tensors are rebuilt from
+            // the handle as it is written (one integer pass, two launches) and kept for its later
+            // replays, where the payload is large enough for the slot-order walk to pay for that
+            // (the REBUILD_ORDER switch: 0 never, 1 always).  Not under stream capture: a captured
+            // replay must not depend on when the rebuilt tensors are dropped.
+            const int rebuild_switch = tuning_switch("REBUILD_ORDER");
+            const bool worth_it = rebuild_switch >= 0 ? rebuild_switch != 0 : expanded_capacity * hidden * 2 >= kRebuildPayloadBytes;
+            std::shared_ptr<PeerRuntime::RebuiltHandle> rebuilt;
+            if (expand && !has_private && worth_it && tokens * topk < (int64_t{1} << 31) &&
+                nanoep_slot_order_entries(tokens, static_cast<int>(topk), local_experts) > 0) {
+                hipStreamCaptureStatus capture = hipStreamCaptureStatusNone;
+                check_hip(hipStreamIsCapturing(comm.stream(), &capture), "hipStreamIsCapturing");
+                if (capture == hipStreamCaptureStatusNone)
+                    rebuilt = private_tensors_of(runtime, metadata, expanded_capacity, tokens, topk, local_experts, hidden, comm);
+            }
+            if (rebuilt) {
+                view.token_slots = rebuilt->table.data_ptr<int32_t>();
+                view.slot_order = rebuilt->order.data_ptr<int64_t>();
+                const int64_t entries = rebuilt->published_entries();
+                view.order_entries = entries >= 0 ? entries : -1;
+            }
+            launch_permute(view, recv_count, expanded_capacity, /*count_on_device=*/rebuilt && view.order_entries < 0);
+        }
     } else {
         hipStreamCaptureStatus capture = hipStreamCaptureStatusNone;
         check_hip(hipStreamIsCapturing(comm.stream(), &capture), "hipStreamIsCapturing");
@@ -676,7 +863,6 @@ DispatchResult dispatch(PeerRuntime& runtime,
             arena64 = torch::empty({count64 + (count32 + 1) / 2}, int64_options);
             return 0;
         });
-        auto workspace = torch::empty({static_cast<int64_t>(workspace_bytes)}, int64_options.dtype(torch::kUInt8));
         // arena64: expert_counts [L] | expert_offsets [L+1] | send_counts [1] | recv_rank_prefix [1] |
         //          dst_slots [T] | topk snapshot [T*K] | slot_order;   arena32: recv_metadata [T*(K+2)] | token_slots [T*K]
         int64_t* base64 = arena64.data_ptr<int64_t>();
@@ -685,6 +871,7 @@ DispatchResult dispatch(PeerRuntime& runtime,
         // From here until the counts have been read this call owns the runtime's mailbox; a fresh
         // dispatch of another thread on the same runtime waits here for its turn.
         PeerRuntime::CountsTurn turn(runtime);
+        const auto workspace = runtime.layout_workspace(workspace_bytes, comm.stream(), int64_options.dtype(torch::kUInt8));
         const int layout_status =
             nanoep_layout(routing.data_ptr<int64_t>(), tokens, static_cast<int>(topk), local_experts, alignment, expand ? 1 : 0,
                           static_cast<int>(hidden), base32, base64, base64 + at_offsets, base64 + at_dst, base64 + at_send, base64 + at_snapshot,
@@ -706,7 +893,7 @@ DispatchResult dispatch(PeerRuntime& runtime,
         const int64_t choice_bound = expand ? tokens * topk : tokens;
         const int64_t gap_bound = expand ? local_experts * (alignment - 1) : 0;
         const int64_t row_bound = choice_bound + gap_bound;
-        const int order_switch = env_switch("NANOEP_FRESH_OUTPUTS");  // 0: always exact, 1: at the bound whenever the rule allows
+        const int order_switch = tuning_switch("FRESH_OUTPUTS");  // 0: always exact, 1: at the bound whenever the rule allows
         const bool speculative = tokens > 0 && gap_bound * 8 <= choice_bound && row_bound <= std::numeric_limits<int32_t>::max() &&
                                  order_switch != 0 && (order_switch == 1 || !runtime.prefers_exact_outputs());
         if (speculative) {
@@ -720,8 +907,20 @@ DispatchResult dispatch(PeerRuntime& runtime,
             fresh.order_entries = order_entries > 0 ? -1 : 0;
             fresh.expert_counts = base64;
             fresh.expert_offsets = base64 + at_offsets;
-            allocate_outputs(row_bound, tokens);
-            launch_permute(fresh, tokens, row_bound, /*count_on_device=*/true);
+            try {
+                allocate_outputs(row_bound, tokens);
+                launch_permute(fresh, tokens, row_bound, /*count_on_device=*/true);
+            } catch (...) {
+                // The layout is under way and will publish its counts whatever went wrong here (most
+                // likely the allocation at the bound): the turn at the mailbox is settled before the
+                // error leaves, so the runtime stays usable.  Only counts that never arrive latch it.
+                int64_t unused[NANOEP_HOST_COUNT_WORDS] = {0, 0, 0, 0};
+                try {
+                    turn.wait(comm.stream(), kCountTimeoutSeconds, unused);
+                } catch (...) {
+                }
+                throw;
+            }
         }
 
         arena32 = arena64.narrow(0, count64, (count32 + 1) / 2).view(torch::kInt32);
@@ -866,14 +1065,29 @@ CombineResult combine(PeerRuntime& runtime,
     if (source_tokens > 0) {
         // a seven-tensor handle of the latest fresh dispatch gets its slot table back from the runtime
         std::vector<torch::Tensor> handle;
-        if (expand && metadata.size() == 7 && env_switch("NANOEP_RECALL_ORDER") != 0) {
+        if (expand && metadata.size() == 7 && tuning_switch("RECALL_ORDER") != 0) {
             handle = metadata;
             runtime.recall_private(handle, -1);
         }
         const auto& lookup = handle.size() > 7 ? handle : metadata;
+        const int32_t* table = slot_table(lookup, source_tokens, topk, expand);
+        // ... or the table a replayed dispatch of this handle had rebuilt
+        std::shared_ptr<PeerRuntime::RebuiltHandle> rebuilt;
+        if (table == nullptr && expand && metadata.size() == 7 && recv_count > 0 && tuning_switch("REBUILD_ORDER") != 0) {
+            hipStreamCaptureStatus capture = hipStreamCaptureStatusNone;
+            check_hip(hipStreamIsCapturing(comm.stream(), &capture), "hipStreamIsCapturing");
+            if (capture == hipStreamCaptureStatusNone && (rebuilt = runtime.find_rebuilt(metadata, x.size(0)))) {
+                if (rebuilt->made_on != comm.stream()) {
+                    if (!rebuilt->ready.query())
+                        comm.unwrap().wait(rebuilt->ready);
+                    rebuilt->order.record_stream(comm.unwrap());
+                }
+                table = rebuilt->table.data_ptr<int32_t>();
+            }
+        }
         check_status(nanoep_combine(x.data_ptr(), weights.has_value() ? weights->data_ptr<float>() : nullptr,
                                     bias.has_value() ? bias->data_ptr() : nullptr, metadata[0].data_ptr<int32_t>(),
-                                    metadata[3].data_ptr<int64_t>(), slot_table(lookup, source_tokens, topk, expand), recv_count,
+                                    metadata[3].data_ptr<int64_t>(), table, recv_count,
                                     x.size(0), source_tokens, static_cast<int>(hidden),
                                     static_cast<int>(topk), expand ? 1 : 0, allow_multiple_reduction ? 1 : 0, combined_x.data_ptr(),
                                     weights.has_value() ? combined_weights.data_ptr<float>() : nullptr, cu_budget, comm.stream()),
@@ -936,6 +1150,7 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, module) {
         .def("barrier", &nanoep::PeerRuntime::barrier_at)
         .def("close_peer_mappings", &nanoep::PeerRuntime::close_peer_mappings)
         .def("private_recalls", &nanoep::PeerRuntime::private_recalls)
+        .def("rebuilds", &nanoep::PeerRuntime::rebuilds)
         .def("counts_failed", &nanoep::PeerRuntime::counts_failed)
         .def("prefers_exact_outputs", &nanoep::PeerRuntime::prefers_exact_outputs)
         .def("valid_share_65536", &nanoep::PeerRuntime::valid_share_65536)

@@ -3,8 +3,8 @@ every compute call goes through the C ABI of nanoep_amd/libnanoep_hip.so."""
 
 from __future__ import annotations
 
+import contextlib
 import ctypes
-import os
 import re
 from pathlib import Path
 
@@ -51,6 +51,14 @@ def lib() -> ctypes.CDLL:
         handle.nanoep_dispatch.argtypes = [p, p, p, p, p, p, i64, p, p, i64, i64, i64, i, i, i64, i64, i, i, p, p, p, i, p]
         handle.nanoep_combine.argtypes = [p, p, p, p, p, p, i64, i64, i64, i, i, i, i, p, p, i, p]
         handle.nanoep_copy_bytes.argtypes = [p, p, sz, p]
+        handle.nanoep_rebuild_window_tokens.argtypes = [i64, i, i]
+        handle.nanoep_rebuild_workspace_bytes.restype = sz
+        handle.nanoep_rebuild_workspace_bytes.argtypes = [i64, i]
+        handle.nanoep_rebuild_order.argtypes = [p, p, i64, i64, i64, i, i64, i, p, p, p, sz, p, i64, p]
+        handle.nanoep_set_tuning.argtypes = [ctypes.c_char_p, i]
+        handle.nanoep_get_tuning.argtypes = [ctypes.c_char_p, ctypes.POINTER(i)]
+        handle.nanoep_reset_tuning.restype = None
+        handle.nanoep_device_topology.argtypes = [ctypes.POINTER(i), ctypes.POINTER(i), ctypes.POINTER(i64)]
         _lib = handle
     return _lib
 
@@ -73,6 +81,31 @@ def ptr(tensor: torch.Tensor | None):
 
 def stream_handle() -> int:
     return torch.cuda.current_stream().cuda_stream
+
+
+def get_tuning(name: str) -> int:
+    value = ctypes.c_int(0)
+    check(lib().nanoep_get_tuning(name.encode(), ctypes.byref(value)))
+    return value.value
+
+
+@contextlib.contextmanager
+def forced_tuning(switches: dict):
+    """Sets the given tuning switches (None: leave alone) through the C ABI and puts the previous values back."""
+    previous = {name: get_tuning(name) for name, value in switches.items() if value is not None}
+    try:
+        for name in previous:
+            check(lib().nanoep_set_tuning(name.encode(), int(switches[name])))
+        yield
+    finally:
+        for name, value in previous.items():
+            check(lib().nanoep_set_tuning(name.encode(), value))
+
+
+def device_topology() -> tuple[int, int, int]:
+    cus, xcds, l2 = ctypes.c_int(0), ctypes.c_int(0), ctypes.c_int64(0)
+    check(lib().nanoep_device_topology(ctypes.byref(cus), ctypes.byref(xcds), ctypes.byref(l2)))
+    return cus.value, xcds.value, l2.value
 
 
 def window_layout(ranks, tokens, hidden, topk, experts, multi=False) -> list[int]:
@@ -133,6 +166,25 @@ def layout(topk_idx: torch.Tensor, num_local_experts: int, alignment: int, expan
     return metadata, counts
 
 
+def rebuild_order(metadata, counts, num_local_experts, hidden, *, host_tag=None):
+    """The private tensors of an expanded handle rebuilt from its recv_metadata and dst_slots alone
+    (nanoep_rebuild_order): returns (token_slots, slot_order, published word or None)."""
+    recv_metadata, dst_slots = metadata[0], metadata[3]
+    device = dst_slots.device
+    tokens = dst_slots.shape[0]
+    topk = recv_metadata.shape[1] - 2
+    table = torch.full((tokens, topk), -9, dtype=torch.int32, device=device)
+    order = torch.full((lib().nanoep_slot_order_entries(tokens, topk, num_local_experts),), -7, dtype=torch.int64, device=device)
+    nbytes = lib().nanoep_rebuild_workspace_bytes(tokens, topk)
+    workspace = torch.empty(nbytes, dtype=torch.uint8, device=device)
+    word = torch.full((1,), -5, dtype=torch.int64).pin_memory() if host_tag is not None else None
+    check(lib().nanoep_rebuild_order(ptr(recv_metadata), ptr(dst_slots), counts[0], counts[1], tokens, topk, num_local_experts, hidden,
+                                     ptr(table), ptr(order), ptr(workspace), nbytes, None if word is None else word.data_ptr(),
+                                     0 if host_tag is None else host_tag, stream_handle()))
+    torch.cuda.current_stream().synchronize()
+    return table, order, None if word is None else int(word[0])
+
+
 def token_slots_of(metadata, use_table=True):
     return metadata[7] if use_table and len(metadata) > 7 else None
 
@@ -146,7 +198,7 @@ def dispatch(x, weights, metadata, counts, num_local_experts, alignment, expand,
     """Returns (recv_x, recv_topk_idx | None, recv_weights | None) through nanoep_dispatch.
 
     walk="forced" sets the library's switch for the slot-order walk explicitly, walk="auto" leaves
-    the environment alone (the library then walks the list whenever it is given one).  span=1|2
+    the switch alone (the library then walks the list whenever it is given one).  span=1|2
     forces the number of chunks a wavefront of that walk moves (the library picks it by source size).
     whole_rows=0|1 forces or forbids that walk's kernel variant for one workgroup a list entry (the
     library takes it for rows of five pieces and more whose workgroup covers the row).
@@ -176,32 +228,15 @@ def dispatch(x, weights, metadata, counts, num_local_experts, alignment, expand,
         order_entries = counts[2]
     else:
         order_entries = -1 if order_count == "device" else -int(order_count[1])
-    previous = os.environ.pop("NANOEP_DISPATCH_ORDER", None)
-    previous_span = os.environ.pop("NANOEP_DISPATCH_SPAN", None)
-    previous_rows = os.environ.pop("NANOEP_DISPATCH_WHOLE_ROWS", None)
-    if whole_rows is not None:
-        os.environ["NANOEP_DISPATCH_WHOLE_ROWS"] = str(int(whole_rows))
-    if walk == "forced":
-        os.environ["NANOEP_DISPATCH_ORDER"] = "1"
-    if span is not None:
-        os.environ["NANOEP_DISPATCH_SPAN"] = str(span)
-    try:
+    switches = {"DISPATCH_ORDER": 1 if walk == "forced" else None, "DISPATCH_SPAN": span,
+                "DISPATCH_WHOLE_ROWS": None if whole_rows is None else int(whole_rows)}
+    with forced_tuning(switches):
         status = lib().nanoep_dispatch(
             ptr(x), ptr(weights), ptr(recv_metadata), ptr(dst_slots), ptr(token_slots_of(metadata, use_table)),
             ptr(order), order_entries, ptr(expert_counts), ptr(expert_offsets), received, capacity,
             tokens, hidden, topk, num_local_experts, alignment, int(expand), int(zero_padding), ptr(recv_x),
             ptr(recv_idx), ptr(recv_w), num_cus, stream_handle(),
         )
-    finally:
-        os.environ.pop("NANOEP_DISPATCH_ORDER", None)
-        os.environ.pop("NANOEP_DISPATCH_SPAN", None)
-        os.environ.pop("NANOEP_DISPATCH_WHOLE_ROWS", None)
-        if previous_rows is not None:
-            os.environ["NANOEP_DISPATCH_WHOLE_ROWS"] = previous_rows
-        if previous is not None:
-            os.environ["NANOEP_DISPATCH_ORDER"] = previous
-        if previous_span is not None:
-            os.environ["NANOEP_DISPATCH_SPAN"] = previous_span
     check(status)
     return recv_x, recv_idx, recv_w
 

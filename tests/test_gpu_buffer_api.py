@@ -125,11 +125,11 @@ def test_readme_round_trip_with_a_gloo_control_group(device):
     ],
 )
 @pytest.mark.parametrize("walk", ["slot-order", "token-order"])
-def test_fresh_and_cached_replay(device, monkeypatch, walk, expand, zero_padding, weighted, kind, hidden, alignment):
+def test_fresh_and_cached_replay(device, tuning, walk, expand, zero_padding, weighted, kind, hidden, alignment):
     # the library walks the slot-order list of its own handles (fresh: device-side entry count,
     # replay: exact count); the switch covers the token-order walk with the slot table as well
     if walk == "token-order":
-        monkeypatch.setenv("NANOEP_DISPATCH_ORDER", "0")
+        tuning("DISPATCH_ORDER", "0")
     tokens, experts, topk = 19, 3, 3
     idx = cases.routing(kind, tokens, experts, topk, seed=2)
     x = cases.payload(tokens, hidden)
@@ -215,11 +215,11 @@ def test_fresh_dispatch_allocation_orders(device, alignment, at_bound):
 
 
 @pytest.mark.parametrize("switch,at_bound", [("0", False), ("1", True)], ids=["always-exact", "at-the-bound"])
-def test_fresh_output_order_can_be_forced(device, monkeypatch, switch, at_bound):
-    """NANOEP_FRESH_OUTPUTS=0 allocates a fresh dispatch's outputs after the counts are known whatever
+def test_fresh_output_order_can_be_forced(device, tuning, switch, at_bound):
+    """The FRESH_OUTPUTS switch at 0 allocates a fresh dispatch's outputs after the counts are known whatever
     the shapes, =1 at the bound whenever the alignment rule allows (a runtime that has turned to the
     exact order included): same results."""
-    monkeypatch.setenv("NANOEP_FRESH_OUTPUTS", switch)
+    tuning("FRESH_OUTPUTS", switch)
     tokens, experts, topk, hidden = 200, 8, 4, 512
     idx = cases.routing("dropout", tokens, experts, topk, seed=6)
     x, w = cases.payload(tokens, hidden, seed=7), cases.gate_weights(tokens, topk)
@@ -296,13 +296,13 @@ def test_headline_shapes_hold_at_most_a_quarter_more_than_they_use(device):
 
 @pytest.mark.parametrize("recall", [False, True], ids=["no-recall", "recall"])
 @pytest.mark.parametrize("tokens,hidden", [(2048, 4096), (37, 512)], ids=["16MiB", "small"])
-def test_replay_with_only_the_reference_handle_tensors(device, monkeypatch, tokens, hidden, recall):
+def test_replay_with_only_the_reference_handle_tensors(device, tuning, tokens, hidden, recall):
     """A handle that carries just the reference's seven tensors (as one that went through the
     reference's own Python class would) replays to the same bytes.  While it is one of the buffer's
     latest fresh dispatches the runtime hands its private tensors back (recall); otherwise the
     payload follows the handle's own dst_slots and recv_metadata in token order."""
     if not recall:
-        monkeypatch.setenv("NANOEP_RECALL_ORDER", "0")
+        tuning("RECALL_ORDER", "0")
     experts, topk, alignment = 16, 4, 8
     idx = cases.routing("dropout", tokens, experts, topk, seed=9)
     x, w = cases.payload(tokens, hidden, seed=4), cases.gate_weights(tokens, topk)
@@ -402,6 +402,96 @@ def test_a_foreign_seven_tensor_handle_is_followed_as_written(device):
         want, want_cw = oracle.combine(want_x, meta, dst, do_expand=True, weights=want_w)
         assert_same_bits(combined, want, "combine through the foreign handle")
         assert_same_bits(restored, want_cw, "weights restored through the foreign handle")
+
+
+def reversed_handle(lay, idx):
+    """The handle of `lay` with reversed receive rows and reversed slots inside every expert segment:
+    coherent, and in another order than this library's own (the reference's expert_inputs builds its
+    handles this way, nano_ep/testing/native_combine.py:62-74)."""
+    meta = lay.recv_metadata(True).flip(0).contiguous()
+    slots = meta[:, 2:].clone().to(torch.int64)
+    expert_of = torch.bucketize(slots.clamp(min=0), lay.expert_offsets[1:], right=True)
+    mirrored = lay.expert_offsets[expert_of] + lay.expert_counts[expert_of] - 1 - (slots - lay.expert_offsets[expert_of])
+    meta[:, 2:] = torch.where(slots >= 0, mirrored, slots).to(torch.int32)
+    dst = torch.where(lay.dst_slots >= 0, lay.recv_count - 1 - lay.dst_slots, lay.dst_slots)
+    return [meta, lay.expert_counts, lay.expert_offsets, dst, lay.send_counts, idx.clone(), lay.recv_rank_prefix]
+
+
+def test_a_reversed_handle_at_the_headline_shape_is_rebuilt_once_and_followed(device, tuning):
+    """4096 x 7168, 256 experts, top-8 with masked choices, and a seven-tensor handle in reversed order:
+    the runtime rebuilds the private tensors from the handle itself at the first replay and keeps
+    them, every replay lands its rows where the handle says (vectorised closed form of the handle,
+    which for the reversed handle is the oracle's dispatch with every expert segment mirrored), the
+    walk that never rebuilds writes the same bytes, and combine brings the rows back."""
+    tokens, experts, topk, hidden, alignment = 4096, 256, 8, 7168, 1
+    idx = cases.routing("dropout", tokens, experts, topk, seed=31)
+    lay = oracle.layout(idx, experts, alignment)
+    public = reversed_handle(lay, idx)
+    meta, dst = public[0], public[3]
+    native = load_extension()
+    cus = torch.cuda.get_device_properties(device).multi_processor_count
+
+    def expected(x, w):
+        rows = meta[:, 1].to(torch.int64)[:, None].expand(-1, topk)
+        slots = meta[:, 2:].to(torch.int64)
+        live = slots >= 0
+        want_x = torch.zeros((lay.expanded_capacity, hidden), dtype=torch.bfloat16)
+        want_w = torch.zeros(lay.expanded_capacity, dtype=torch.float32)
+        want_x[slots[live]] = x[rows[live]]
+        ks = torch.arange(topk)[None, :].expand_as(slots)
+        want_w[slots[live]] = w[rows[live], ks[live]]
+        return want_x, want_w
+
+    with Buffer(None, EPConfig(experts, topk, hidden, tokens)) as buffer:
+        handle = [t.to(device) for t in public]
+        stream = buffer.comm_stream.cuda_stream
+        first = None
+        for step in (1, 2, 3):
+            x = cases.payload(tokens, hidden, seed=40 + step)
+            w = cases.gate_weights(tokens, topk, seed=step)
+            if step == 3:
+                tuning("REBUILD_ORDER", 0)  # the token-order walk through the handle's own tensors
+            outputs, returned, (received, capacity), event = native.dispatch(
+                buffer._runtime, x.to(device), handle[5], w.to(device), experts, tokens, alignment, handle, lay.expanded_capacity,
+                False, True, True, cus, stream, -1, False)
+            assert all(a is b for a, b in zip(returned, handle)) and len(returned) == 7
+            want_x, want_w = expected(x, w)
+            assert_same_bits(outputs[0], want_x, f"replay {step} rows follow the handle")
+            assert_same_bits(outputs[2], want_w, f"replay {step} weights follow the handle")
+            assert buffer._runtime.rebuilds() == 1
+            first = first or (outputs, want_x, want_w)
+        tuning("REBUILD_ORDER", -1)
+        outputs, want_x, want_w = first
+        (combined, restored), _ = native.combine(buffer._runtime, outputs[0], handle, outputs[2], None, tokens, True, False, cus,
+                                                 stream, -1, False)
+        want, want_cw = oracle.combine(want_x, meta, dst, do_expand=True, weights=want_w)
+        assert_same_bits(combined, want, "combine through the reversed handle")
+        assert_same_bits(restored, want_cw, "weights restored through the reversed handle")
+        assert buffer._runtime.rebuilds() == 1
+        # editing the handle through torch makes it another handle: it is rebuilt
+        handle[3].copy_(handle[3])
+        native.dispatch(buffer._runtime, x.to(device), handle[5], None, experts, tokens, alignment, handle, lay.expanded_capacity,
+                        False, True, False, cus, stream, -1, False)
+        assert buffer._runtime.rebuilds() == 2
+
+
+def test_the_fifth_oldest_handle_of_a_buffer_still_takes_the_slot_order_walk(device):
+    """A caller that keeps five seven-tensor handles alive (one per layer, say): the runtime
+    remembers the private tensors of its latest four, the oldest one has them rebuilt from the
+    handle itself, once, and every replay equals the oracle."""
+    tokens, experts, topk, hidden, alignment = 2048, 32, 4, 4096, 16
+    x, w = cases.payload(tokens, hidden, seed=8), cases.gate_weights(tokens, topk)
+    with Buffer(None, EPConfig(experts, topk, hidden, tokens)) as buffer:
+        routings = [cases.routing("dropout", tokens, experts, topk, seed=50 + layer) for layer in range(5)]
+        bare = []
+        for idx in routings:
+            fresh = buffer.dispatch(x.to(device), topk_idx=idx.to(device), weights=w.to(device), do_expand=True, alignment=alignment)
+            bare.append(dataclasses.replace(fresh.handle, token_slots=None, slot_order=None))
+        for _ in range(2):
+            for layer in (4, 3, 2, 1, 0):
+                replay = buffer.dispatch(x.to(device), weights=w.to(device), handle=bare[layer], zero_padding=True)
+                assert_dispatch_result(replay, x, routings[layer], w, experts, True, alignment, True)
+        assert buffer._runtime.rebuilds() == 1 and buffer._runtime.private_recalls() == 8
 
 
 @pytest.mark.parametrize("expand", [False, True], ids=["compact", "expanded"])

@@ -352,10 +352,10 @@ def test_topk_range(device, topk, experts, hidden, expand):
 )
 @pytest.mark.parametrize("expand", [False, True], ids=["compact", "expanded"])
 @pytest.mark.parametrize("hidden", [0, 2048, 16384, 40000], ids=["windows-256", "windows-512", "windows-128", "windows-64"])
-def test_both_layout_launch_plans(device, monkeypatch, hidden, launches, tokens, experts, topk, kind, alignment, expand):
+def test_both_layout_launch_plans(device, tuning, hidden, launches, tokens, experts, topk, kind, alignment, expand):
     """The layout runs as two launches (every block scans the block histograms itself) or three
     (single-workgroup scan), chosen by size; both plans must give the oracle's handle."""
-    monkeypatch.setenv("NANOEP_LAYOUT_LAUNCHES", launches)
+    tuning("LAYOUT_LAUNCHES", launches)
     idx = cases.routing(kind, tokens, experts, topk, seed=5)
     metadata, counts = cabi.layout(idx.to(device), experts, alignment, expand, hidden=hidden)
     assert_layout(metadata, counts, oracle.layout(idx, experts, alignment), expand, hidden)
@@ -371,15 +371,20 @@ def test_windows_of_1024_tokens(device, tokens, experts, topk, hidden):
     run_dispatch_combine(device, idx, hidden, experts, 8, True, True, True, seed=3)
 
 
-@pytest.mark.parametrize("window,tokens", [(96, 1000), (160, 4096), (192, 4096), (224, 2000), (512, 1500)])
-def test_forced_window_sizes(device, monkeypatch, window, tokens):
-    """NANOEP_WINDOW_TOKENS orders the slot-order list by windows of any multiple of 32 tokens up to
+@pytest.mark.parametrize(
+    "window,tokens,experts",
+    [(96, 1000, 24), (160, 4096, 24), (192, 4096, 24), (224, 2000, 24), (512, 1500, 24),
+     # windows that are not whole wavefronts, with experts that fall to the threads of the last, partial one
+     (96, 1000, 72), (96, 1000, 96), (96, 1000, 256), (160, 4096, 160), (160, 4096, 256), (224, 2000, 200), (224, 2000, 256)],
+)
+def test_forced_window_sizes(device, tuning, window, tokens, experts):
+    """The WINDOW_TOKENS switch orders the slot-order list by windows of any multiple of 32 tokens up to
     256 (one layout workgroup each; the last one ragged, and more workgroups' worth of tokens than
     the list buffer, which is sized by blocks of 256, has room for beyond the batch)."""
-    monkeypatch.setenv("NANOEP_WINDOW_TOKENS", str(window))
-    assert cabi.lib().nanoep_layout_block_tokens(tokens, 24, 512) == window
-    idx = cases.routing("dropout", tokens, 24, 4, seed=window)
-    run_dispatch_combine(device, idx, 512, 24, 8, True, True, True, seed=5)
+    tuning("WINDOW_TOKENS", str(window))
+    assert cabi.lib().nanoep_layout_block_tokens(tokens, experts, 512) == window
+    idx = cases.routing("dropout", tokens, experts, 4, seed=window)
+    run_dispatch_combine(device, idx, 512, experts, 8, True, True, True, seed=5)
 
 
 @pytest.mark.parametrize(
@@ -608,6 +613,108 @@ def test_reversed_handle_order_is_honoured(device):
             live = torch.zeros(lay.expanded_capacity, dtype=torch.bool)
             live[slots[slots >= 0]] = True
             assert (got_x[~live].view(torch.int16) == 0).all() and (got_xw[~live] == 0).all()
+
+
+def expected_slot_order(table: torch.Tensor, window: int, entries: int):
+    """Closed form of a slot-order buffer: window of consecutive tokens by window, the valid
+    (slot << 32) | (t * K + k) ascending, -1 up to the count word, the count."""
+    tokens, topk = table.shape
+    flat = table.flatten().to(torch.int64)
+    packed = (flat << 32) | torch.arange(flat.numel(), dtype=torch.int64)
+    parts = []
+    for first in range(0, tokens, window):
+        span = slice(first * topk, (first + window) * topk)
+        parts.append(packed[span][flat[span] >= 0].sort().values)
+    assigned = int((flat >= 0).sum())
+    parts.append(torch.full((entries - 1 - assigned,), -1, dtype=torch.int64))
+    parts.append(torch.tensor([assigned], dtype=torch.int64))
+    return torch.cat(parts)
+
+
+@pytest.mark.parametrize(
+    "tokens,experts,topk,kind,alignment,hidden",
+    [
+        pytest.param(19, 3, 3, "mixed", 4, 256, id="one-window"),
+        pytest.param(1000, 16, 4, "dropout", 8, 512, id="ragged-last-window"),
+        pytest.param(4096, 256, 8, "dropout", 1, 7168, id="headline-routing"),
+        pytest.param(4096, 8, 2, "random", 1, 4096, id="mixtral-routing"),
+        pytest.param(8192, 128, 8, "biased", 128, 2048, id="qwen3-routing"),
+        pytest.param(3000, 40, 17, "sparse", 3, 1024, id="odd-topk-window-halved"),
+        pytest.param(700, 64, 32, "random", 1, 256, id="top-32"),
+        pytest.param(2500, 8, 1, "dropout", 16, 8192, id="top-1"),
+        pytest.param(600, 8, 2, "masked", 1, 512, id="nothing-received"),
+    ],
+)
+def test_private_tensors_rebuilt_from_the_public_ones(device, tokens, experts, topk, kind, alignment, hidden):
+    """nanoep_rebuild_order reads nothing but recv_metadata and dst_slots, and gives the layout's own
+    slot table back bit for bit, and a slot-order list that is the closed form for its window size
+    (the layout's own list when both take the same window); the dispatch that walks the rebuilt pair
+    writes the same bytes, with the count from the host and from the device."""
+    idx = cases.routing(kind, tokens, experts, topk, seed=17)
+    metadata, counts = cabi.layout(idx.to(device), experts, alignment, True, hidden=hidden)
+    public = metadata[:7]
+    tag = 5 << 32
+    table, order, word = cabi.rebuild_order(public, counts, experts, hidden, host_tag=tag)
+    assert torch.equal(table.cpu(), metadata[7].cpu())
+    window = cabi.lib().nanoep_rebuild_window_tokens(tokens, topk, hidden)
+    assert window * topk <= 4096 and window >= 32
+    assert torch.equal(order.cpu(), expected_slot_order(metadata[7].cpu(), window, order.numel()))
+    assert word == tag | counts[2]
+    if window == cabi.lib().nanoep_layout_block_tokens(tokens, experts, hidden):
+        assert torch.equal(order.cpu(), metadata[8].cpu())
+    if counts[0] == 0:
+        return
+    x, w = cases.payload(tokens, hidden, seed=3), cases.gate_weights(tokens, topk)
+    want_x, _, want_w = cabi.dispatch(x.to(device), w.to(device), public, counts, experts, alignment, True, True, poison=POISON)
+    rebuilt = public + [table, order]
+    for order_count in ("exact", "device"):
+        got_x, _, got_w = cabi.dispatch(x.to(device), w.to(device), rebuilt, counts, experts, alignment, True, True, poison=POISON,
+                                        order_count=order_count)
+        assert torch.equal(got_x.view(torch.int16), want_x.view(torch.int16))
+        assert torch.equal(got_w.view(torch.int32), want_w.view(torch.int32))
+
+
+def test_rebuild_follows_a_handle_in_another_order(device):
+    """A coherent handle with reversed receive rows and reversed slots inside every expert segment
+    (as the reference's expert_inputs builds them, nano_ep/testing/native_combine.py:62-74), plus
+    slots outside the capacity that must be dropped: the rebuilt pair says what the handle says."""
+    tokens, experts, topk, hidden, alignment = 1500, 12, 4, 512, 4
+    idx = cases.routing("dropout", tokens, experts, topk, seed=23)
+    lay = oracle.layout(idx, experts, alignment)
+    meta = lay.recv_metadata(True).flip(0).contiguous()
+    slots = meta[:, 2:].clone().to(torch.int64)
+    expert_of = torch.bucketize(slots.clamp(min=0), lay.expert_offsets[1:], right=True)
+    mirrored = lay.expert_offsets[expert_of] + lay.expert_counts[expert_of] - 1 - (slots - lay.expert_offsets[expert_of])
+    meta[:, 2:] = torch.where(slots >= 0, mirrored, slots).to(torch.int32)
+    meta[5, 2] = lay.expanded_capacity  # one past the last row: not a slot
+    meta[7, 3] = -3
+    dst = torch.where(lay.dst_slots >= 0, lay.recv_count - 1 - lay.dst_slots, lay.dst_slots)
+    dst[int(meta[11, 1]), 0] = lay.recv_count  # a token pointing past the receive rows is not sent
+    want_table = torch.full((tokens, topk), -1, dtype=torch.int32)
+    for token in range(tokens):
+        row = int(dst[token, 0])
+        if 0 <= row < lay.recv_count:
+            values = meta[row, 2:]
+            want_table[token] = torch.where((values >= 0) & (values < lay.expanded_capacity), values, torch.full_like(values, -1))
+    public = [meta.to(device), lay.expert_counts.to(device), lay.expert_offsets.to(device), dst.to(device)]
+    counts = (lay.recv_count, lay.expanded_capacity, 0, 0)
+    table, order, _ = cabi.rebuild_order(public, counts, experts, hidden)
+    assert torch.equal(table.cpu(), want_table)
+    window = cabi.lib().nanoep_rebuild_window_tokens(tokens, topk, hidden)
+    assert torch.equal(order.cpu(), expected_slot_order(want_table, window, order.numel()))
+    x, w = cases.payload(tokens, hidden, seed=5), cases.gate_weights(tokens, topk)
+    want_x, _, want_w = cabi.dispatch(x.to(device), w.to(device), public, counts, experts, alignment, True, True, poison=POISON)
+    got_x, _, got_w = cabi.dispatch(x.to(device), w.to(device), public + [None, None, None, table, order], counts, experts, alignment,
+                                    True, True, poison=POISON, order_count="device")
+    assert torch.equal(got_x.view(torch.int16), want_x.view(torch.int16))
+    assert torch.equal(got_w.view(torch.int32), want_w.view(torch.int32))
+    # every row the table names holds its token; the rows of the dropped entries are nobody's and keep the poison
+    live = want_table >= 0
+    rows = want_table[live].to(torch.int64)
+    source = torch.arange(tokens)[:, None].expand(-1, topk)[live]
+    assert_bits_equal(got_x.cpu()[rows], x[source], "rows follow the rebuilt table")
+    dropped = [int(mirrored[row, k]) for row, k in [(5, 0), (7, 1)] + [(11, k) for k in range(topk)] if slots[row, k] >= 0]
+    assert dropped and (got_x.cpu()[torch.tensor(dropped)].view(torch.uint8) == POISON).all()
 
 
 def test_window_layout_known_answer():
