@@ -108,6 +108,76 @@ __global__ void __launch_bounds__(kBlockThreads) copy_vectors_kernel(const u32x4
         dst[i] = src[i];
 }
 
+// Plain streams in the shape of the row kernels: one workgroup per destination row, one wavefront
+// per 1 KiB chunk of it, one 128-bit access per lane, nontemporal stores, workgroups dealt to the XCDs
+// in contiguous ranges.  They move the bytes of a dispatch or a combine with addresses that are a
+// closed form of the workgroup index and no lookups: what such a launch attains is the ceiling a
+// permute of the same bytes can approach.
+//   kStreamRead   : reads src row r (nothing is written unless a lane holds an impossible value)
+//   kStreamFill   : writes dst row r
+//   kStreamFanOut : every source row is written kFan times.  Rows go in windows of `window` source
+//                   rows: destination row r = w * window * kFan + p * window + i holds source row
+//                   w * window + i (kFan passes over a window that can stay in an XCD's L2, as the
+//                   slot-order walk makes them; window == 1: kFan neighbours share a row).
+//   kStreamFanIn  : destination row w * window + i is the integer sum of the kFan source rows
+//                   w * window * kFan + p * window + i (kFan linear streams per window).
+enum StreamKind { kStreamRead = 0, kStreamFill = 1, kStreamFanOut = 2, kStreamFanIn = 3 };
+
+template <int kKind, int kFan>
+__global__ void __launch_bounds__(1024) stream_probe_kernel(const u32x4* __restrict__ src,
+                                                            u32x4* __restrict__ dst,
+                                                            uint32_t dst_rows,
+                                                            uint32_t row_vectors,
+                                                            uint32_t window,
+                                                            uint32_t span_magic,  // fast divisor by window * kFan
+                                                            uint32_t span_shift,
+                                                            uint32_t window_magic,  // fast divisor by window
+                                                            uint32_t window_shift,
+                                                            uint32_t blocks_per_xcd,
+                                                            XcdMap xcds) {
+    NANOEP_FETCH_ARGS_4(src, dst, dst_rows, row_vectors);
+    NANOEP_FETCH_ARGS_4(window, span_magic, span_shift, blocks_per_xcd);
+    NANOEP_FETCH_ARGS_4(xcds.count, xcds.magic, xcds.shift, window_magic);
+    const uint32_t index_in_xcd = fast_divide(blockIdx.x, xcds.magic, xcds.shift);
+    const uint32_t xcd = blockIdx.x - index_in_xcd * xcds.count;
+    const uint32_t row = xcd * blocks_per_xcd + index_in_xcd;
+    if (index_in_xcd >= blocks_per_xcd || row >= dst_rows)
+        return;
+    const uint32_t vector = __builtin_amdgcn_readfirstlane(threadIdx.y) * kWave + threadIdx.x;
+    const bool in_row = vector < row_vectors;
+    const uint32_t at = in_row ? vector : 0u;
+    u32x4* out = dst + static_cast<uint64_t>(row) * row_vectors + vector;
+    if (kKind == kStreamRead) {
+        const u32x4 data = load_vec<true>(src + static_cast<uint64_t>(row) * row_vectors + at);
+        if (data.x == 0x7fc1a5a5u && data.y == 0x12345678u && data.z == 0x9abcdef0u && in_row)
+            store_vec<true>(out, data);
+    } else if (kKind == kStreamFill) {
+        const u32x4 data = {row, vector, 0u, 0u};
+        if (in_row)
+            store_vec<true>(out, data);
+    } else if (kKind == kStreamFanOut) {
+        const uint32_t in_window = fast_divide(row, span_magic, span_shift);
+        const uint32_t rest = row - in_window * window * kFan;
+        const uint32_t from = in_window * window + (rest - fast_divide(rest, window_magic, window_shift) * window);
+        const u32x4 data = src[static_cast<uint64_t>(from) * row_vectors + at];
+        if (in_row)
+            store_vec<true>(out, data);
+    } else {
+        const uint32_t in_window = fast_divide(row, window_magic, window_shift);
+        const uint64_t first = static_cast<uint64_t>(in_window) * window * kFan + (row - in_window * window);
+        u32x4 data[kFan];
+#pragma unroll
+        for (int p = 0; p < kFan; ++p)
+            data[p] = load_vec<true>(src + (first + static_cast<uint64_t>(p) * window) * row_vectors + at);
+        u32x4 sum = data[0];
+#pragma unroll
+        for (int p = 1; p < kFan; ++p)
+            sum += data[p];
+        if (in_row)
+            store_vec<true>(out, sum);
+    }
+}
+
 }  // namespace
 }  // namespace nanoep
 
@@ -209,6 +279,64 @@ int nanoep_window_layout(int ranks, int64_t max_tokens, int hidden, int topk, in
     out[2] = payload_offset;
     out[3] = payload_offset;
     out[4] = up32(payload_offset + (wire_bytes > return_bytes ? wire_bytes : return_bytes));
+    return NANOEP_OK;
+}
+
+int nanoep_stream_probe(int kind, const void* src, void* dst, int64_t dst_rows, int hidden, int fan, int64_t window,
+                        void* stream_handle) {
+    if (kind < kStreamRead || kind > kStreamFanIn || hidden <= 0 || hidden % 8 != 0 || hidden > 8192 || dst_rows <= 0 ||
+        dst_rows >= (int64_t{1} << 31) - 64 || window < 1 || window * fan >= (int64_t{1} << 31) || !aligned16(src) || !aligned16(dst))
+        return NANOEP_ERR_INVALID_ARGUMENT;
+    if (fan != 1 && fan != 2 && fan != 4 && fan != 7 && fan != 8)
+        return NANOEP_ERR_INVALID_ARGUMENT;
+    if ((kind != kStreamFill && src == nullptr) || dst == nullptr)
+        return NANOEP_ERR_INVALID_ARGUMENT;
+    // whole windows only: every destination row then has all its source rows
+    if (kind == kStreamFanOut ? dst_rows % (window * fan) != 0 : kind == kStreamFanIn && dst_rows % window != 0)
+        return NANOEP_ERR_INVALID_ARGUMENT;
+    const Topology topology = current_topology(current_tuning());
+    const XcdMap xcds = make_xcd_map(topology.xcds);
+    const uint32_t row_vectors = static_cast<uint32_t>(hidden / 8);
+    const uint32_t chunks = (row_vectors + kWave - 1) / kWave;
+    const uint32_t per_xcd = static_cast<uint32_t>((dst_rows + xcds.count - 1) / xcds.count);
+    const FastDivisor span_divisor = make_fast_divisor(static_cast<uint32_t>(window * fan));
+    const FastDivisor window_divisor = make_fast_divisor(static_cast<uint32_t>(window));
+    const dim3 grid(per_xcd * xcds.count), block(kWave, chunks, 1);
+    auto stream = static_cast<hipStream_t>(stream_handle);
+#define NANOEP_LAUNCH_STREAM(KIND, FAN)                                                                                  \
+    stream_probe_kernel<KIND, FAN><<<grid, block, 0, stream>>>(                                                          \
+        static_cast<const u32x4*>(src), static_cast<u32x4*>(dst), static_cast<uint32_t>(dst_rows), row_vectors,          \
+        static_cast<uint32_t>(window), span_divisor.magic, span_divisor.shift, window_divisor.magic, window_divisor.shift, \
+        per_xcd, xcds)
+#define NANOEP_LAUNCH_STREAM_FAN(KIND)         \
+    switch (fan) {                             \
+        case 1:                                \
+            NANOEP_LAUNCH_STREAM(KIND, 1);     \
+            break;                             \
+        case 2:                                \
+            NANOEP_LAUNCH_STREAM(KIND, 2);     \
+            break;                             \
+        case 4:                                \
+            NANOEP_LAUNCH_STREAM(KIND, 4);     \
+            break;                             \
+        case 7:                                \
+            NANOEP_LAUNCH_STREAM(KIND, 7);     \
+            break;                             \
+        default:                               \
+            NANOEP_LAUNCH_STREAM(KIND, 8);     \
+            break;                             \
+    }
+    if (kind == kStreamRead)
+        NANOEP_LAUNCH_STREAM(kStreamRead, 1);
+    else if (kind == kStreamFill)
+        NANOEP_LAUNCH_STREAM(kStreamFill, 1);
+    else if (kind == kStreamFanOut)
+        NANOEP_LAUNCH_STREAM_FAN(kStreamFanOut)
+    else
+        NANOEP_LAUNCH_STREAM_FAN(kStreamFanIn)
+#undef NANOEP_LAUNCH_STREAM_FAN
+#undef NANOEP_LAUNCH_STREAM
+    NANOEP_HIP_TRY(hipGetLastError());
     return NANOEP_OK;
 }
 
