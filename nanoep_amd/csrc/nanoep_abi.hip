@@ -26,7 +26,7 @@ constexpr SwitchSlot kSwitches[] = {
     {"LAYOUT_LAUNCHES", &Tuning::layout_launches},   {"WINDOW_TOKENS", &Tuning::window_tokens},
     {"RECALL_ORDER", &Tuning::recall_order},         {"FRESH_OUTPUTS", &Tuning::fresh_outputs},
     {"REBUILD_ORDER", &Tuning::rebuild_order},       {"XCDS", &Tuning::xcds},
-    {"L2_BYTES", &Tuning::l2_bytes},
+    {"L2_BYTES", &Tuning::l2_bytes},                 {"DISPATCH_PREFETCH", &Tuning::dispatch_prefetch},
 };
 constexpr int kSwitchCount = sizeof(kSwitches) / sizeof(kSwitches[0]);
 

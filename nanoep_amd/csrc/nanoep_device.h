@@ -81,6 +81,7 @@ struct Tuning {
     int dispatch_span = 0;          // DISPATCH_SPAN: 1 | 2 chunks a wavefront of the slot-order walk, 0 = by size
     int dispatch_side = -1;         // DISPATCH_SIDE: 0 | 1 weights of that walk in workgroups of their own
     int dispatch_whole_rows = -1;   // DISPATCH_WHOLE_ROWS: 0 | 1 the kernel variant for one workgroup a list entry
+    int dispatch_prefetch = -1;     // DISPATCH_PREFETCH: 0 | 1 window-wise source prefetch in the slot-order walk
     int layout_launches = 0;        // LAYOUT_LAUNCHES: 2 | 3 forces the layout plan
     int window_tokens = 0;          // WINDOW_TOKENS: forces the window of the slot-order list
     int recall_order = -1;          // RECALL_ORDER: 0 = seven-tensor handles never get private tensors back (host extension)

@@ -110,6 +110,16 @@ def run_dispatch_combine(device, idx, hidden, experts, alignment, expand, zero_p
                 )
                 assert torch.equal(rows_x.view(torch.int16), got_x.view(torch.int16))
                 assert rows_w is None or torch.equal(rows_w.view(torch.int32), got_w.view(torch.int32))
+        # ... so must the walk with and without its window-wise source prefetch, in both kernel variants
+        for prefetch in (0, 1):
+            for whole_rows in (0, 1):
+                for order_count in ("exact", "device"):
+                    fetched_x, _, fetched_w = cabi.dispatch(
+                        x.to(device), None if w is None else w.to(device), metadata, counts, experts, alignment, expand, zero_padding,
+                        num_cus=num_cus, poison=POISON, prefetch=prefetch, whole_rows=whole_rows, order_count=order_count,
+                    )
+                    assert torch.equal(fetched_x.view(torch.int16), got_x.view(torch.int16))
+                    assert fetched_w is None or torch.equal(fetched_w.view(torch.int32), got_w.view(torch.int32))
         # ... so must the same call with the library's switches left alone
         auto_x, _, auto_w = cabi.dispatch(
             x.to(device), None if w is None else w.to(device), metadata, counts, experts, alignment, expand, zero_padding,
@@ -405,11 +415,11 @@ def test_device_side_count_with_a_launch_sized_for_another_count(device, tokens,
     assignments = counts[2]
     want_x, _, want_w = cabi.dispatch(x, w, metadata, counts, experts, alignment, True, True, poison=POISON)
     for expected in (2, 9, assignments // 3, assignments - 1, assignments, assignments + 1, tokens * topk, tokens * topk + 1000):
-        for span in (1, 2):
+        for span, prefetch in ((1, 0), (2, 0), (1, 1), (2, 1)):
             got_x, _, got_w = cabi.dispatch(x, w, metadata, counts, experts, alignment, True, True, poison=POISON,
-                                            order_count=("device", expected), span=span)
-            assert torch.equal(got_x.view(torch.int16), want_x.view(torch.int16)), (expected, span)
-            assert torch.equal(got_w.view(torch.int32), want_w.view(torch.int32)), (expected, span)
+                                            order_count=("device", expected), span=span, prefetch=prefetch)
+            assert torch.equal(got_x.view(torch.int16), want_x.view(torch.int16)), (expected, span, prefetch)
+            assert torch.equal(got_w.view(torch.int32), want_w.view(torch.int32)), (expected, span, prefetch)
 
 
 @pytest.mark.parametrize("use_order", [True, False], ids=["slot-order", "token-order"])
