@@ -231,9 +231,10 @@ int nanoep_combine(const void* y, const float* weights, const void* bias, const 
                    float* out_weights, int num_cus, void* stream);
 
 /*
- * Plain streams in the shape of the row kernels (one workgroup per destination row of `hidden` bf16
- * elements, one wavefront per KiB, addresses a closed form of the workgroup index, no lookups): the
- * measured ceiling for a permute of the same bytes.  No counterpart in the reference.
+ * Plain streams in the shape of the row kernels (one wavefront per KiB of a destination row of
+ * `hidden` bf16 elements, workgroups of waves_per_block consecutive KiB, 0: a workgroup per row;
+ * addresses a closed form of the workgroup index, no lookups): the measured ceiling for a permute of
+ * the same bytes.  No counterpart in the reference.
  *   kind 0: read dst_rows rows of src (dst is only written if a lane reads one impossible bit pattern)
  *   kind 1: fill dst_rows rows of dst
  *   kind 2: fan-out.  Source rows go in windows of `window` rows, each written `fan` times in `fan`
@@ -244,7 +245,7 @@ int nanoep_combine(const void* y, const float* weights, const void* bias, const 
  * hidden <= 8192; fan 1, 2, 4, 7 or 8; dst_rows a multiple of window * fan (kind 2) or window (kind 3).
  */
 int nanoep_stream_probe(int kind, const void* src, void* dst, int64_t dst_rows, int hidden, int fan, int64_t window,
-                        void* stream);
+                        int waves_per_block, void* stream);
 
 /* Plain 16-byte-vector device copy of `bytes` (multiple of 16); the known-size kernel used to
  * scale the profiler's HBM byte counters.  No counterpart in the reference. */

@@ -108,9 +108,10 @@ __global__ void __launch_bounds__(kBlockThreads) copy_vectors_kernel(const u32x4
         dst[i] = src[i];
 }
 
-// Plain streams in the shape of the row kernels: one workgroup per destination row, one wavefront
-// per 1 KiB chunk of it, one 128-bit access per lane, nontemporal stores, workgroups dealt to the XCDs
-// in contiguous ranges.  They move the bytes of a dispatch or a combine with addresses that are a
+// Plain streams in the shape of the row kernels: one wavefront per 1 KiB chunk of a destination row,
+// workgroups of a chosen number of consecutive chunks (a whole row, a part of one, or several short
+// rows), one 128-bit access per lane, nontemporal stores, workgroups dealt to the XCDs in contiguous
+// ranges.  They move the bytes of a dispatch or a combine with addresses that are a
 // closed form of the workgroup index and no lookups: what such a launch attains is the ceiling a
 // permute of the same bytes can approach.
 //   kStreamRead   : reads src row r (nothing is written unless a lane holds an impossible value)
@@ -134,16 +135,23 @@ __global__ void __launch_bounds__(1024) stream_probe_kernel(const u32x4* __restr
                                                             uint32_t window_magic,  // fast divisor by window
                                                             uint32_t window_shift,
                                                             uint32_t blocks_per_xcd,
+                                                            uint32_t chunks,  // 1 KiB chunks of a row
+                                                            uint32_t chunks_magic,
+                                                            uint32_t chunks_shift,
                                                             XcdMap xcds) {
     NANOEP_FETCH_ARGS_4(src, dst, dst_rows, row_vectors);
     NANOEP_FETCH_ARGS_4(window, span_magic, span_shift, blocks_per_xcd);
     NANOEP_FETCH_ARGS_4(xcds.count, xcds.magic, xcds.shift, window_magic);
+    NANOEP_FETCH_ARGS_4(chunks, chunks_magic, chunks_shift, window_shift);
     const uint32_t index_in_xcd = fast_divide(blockIdx.x, xcds.magic, xcds.shift);
     const uint32_t xcd = blockIdx.x - index_in_xcd * xcds.count;
-    const uint32_t row = xcd * blocks_per_xcd + index_in_xcd;
-    if (index_in_xcd >= blocks_per_xcd || row >= dst_rows)
+    if (index_in_xcd >= blocks_per_xcd)
         return;
-    const uint32_t vector = __builtin_amdgcn_readfirstlane(threadIdx.y) * kWave + threadIdx.x;
+    const uint32_t unit = (xcd * blocks_per_xcd + index_in_xcd) * blockDim.y + __builtin_amdgcn_readfirstlane(threadIdx.y);
+    const uint32_t row = fast_divide(unit, chunks_magic, chunks_shift);
+    if (row >= dst_rows)
+        return;
+    const uint32_t vector = (unit - row * chunks) * kWave + threadIdx.x;
     const bool in_row = vector < row_vectors;
     const uint32_t at = in_row ? vector : 0u;
     u32x4* out = dst + static_cast<uint64_t>(row) * row_vectors + vector;
@@ -283,11 +291,11 @@ int nanoep_window_layout(int ranks, int64_t max_tokens, int hidden, int topk, in
 }
 
 int nanoep_stream_probe(int kind, const void* src, void* dst, int64_t dst_rows, int hidden, int fan, int64_t window,
-                        void* stream_handle) {
+                        int waves_per_block, void* stream_handle) {
     if (kind < kStreamRead || kind > kStreamFanIn || hidden <= 0 || hidden % 8 != 0 || hidden > 8192 || dst_rows <= 0 ||
         dst_rows >= (int64_t{1} << 31) - 64 || window < 1 || window * fan >= (int64_t{1} << 31) || !aligned16(src) || !aligned16(dst))
         return NANOEP_ERR_INVALID_ARGUMENT;
-    if (fan != 1 && fan != 2 && fan != 4 && fan != 7 && fan != 8)
+    if ((fan != 1 && fan != 2 && fan != 4 && fan != 7 && fan != 8) || waves_per_block < 0 || waves_per_block > kMaxWavesPerBlock)
         return NANOEP_ERR_INVALID_ARGUMENT;
     if ((kind != kStreamFill && src == nullptr) || dst == nullptr)
         return NANOEP_ERR_INVALID_ARGUMENT;
@@ -298,16 +306,22 @@ int nanoep_stream_probe(int kind, const void* src, void* dst, int64_t dst_rows, 
     const XcdMap xcds = make_xcd_map(topology.xcds);
     const uint32_t row_vectors = static_cast<uint32_t>(hidden / 8);
     const uint32_t chunks = (row_vectors + kWave - 1) / kWave;
-    const uint32_t per_xcd = static_cast<uint32_t>((dst_rows + xcds.count - 1) / xcds.count);
+    // 0: a workgroup per row (rows of up to 16 chunks), else that many consecutive chunks a workgroup
+    const uint32_t waves = waves_per_block > 0 ? static_cast<uint32_t>(waves_per_block) : (chunks < kMaxWavesPerBlock ? chunks : kMaxWavesPerBlock);
+    const int64_t blocks = (dst_rows * chunks + waves - 1) / waves;
+    if (blocks >= (int64_t{1} << 31) - 64 || dst_rows * chunks >= (int64_t{1} << 31))
+        return NANOEP_ERR_INVALID_ARGUMENT;
+    const uint32_t per_xcd = static_cast<uint32_t>((blocks + xcds.count - 1) / xcds.count);
     const FastDivisor span_divisor = make_fast_divisor(static_cast<uint32_t>(window * fan));
     const FastDivisor window_divisor = make_fast_divisor(static_cast<uint32_t>(window));
-    const dim3 grid(per_xcd * xcds.count), block(kWave, chunks, 1);
+    const FastDivisor chunks_divisor = make_fast_divisor(chunks);
+    const dim3 grid(per_xcd * xcds.count), block(kWave, waves, 1);
     auto stream = static_cast<hipStream_t>(stream_handle);
 #define NANOEP_LAUNCH_STREAM(KIND, FAN)                                                                                  \
     stream_probe_kernel<KIND, FAN><<<grid, block, 0, stream>>>(                                                          \
         static_cast<const u32x4*>(src), static_cast<u32x4*>(dst), static_cast<uint32_t>(dst_rows), row_vectors,          \
         static_cast<uint32_t>(window), span_divisor.magic, span_divisor.shift, window_divisor.magic, window_divisor.shift, \
-        per_xcd, xcds)
+        per_xcd, chunks, chunks_divisor.magic, chunks_divisor.shift, xcds)
 #define NANOEP_LAUNCH_STREAM_FAN(KIND)         \
     switch (fan) {                             \
         case 1:                                \

@@ -195,6 +195,28 @@ class PeerRuntime {
     bool prefers_exact_outputs() const { return prefers_exact_outputs_.load(); }
     void note_output_fill(bool bound_was_close) { prefers_exact_outputs_.store(!bound_was_close); }
 
+    // Rows the latest fresh dispatch of a geometry ended up using.  Where the upper bound of the output
+    // shapes is not close (large alignment gaps), a fresh dispatch of the same geometry allocates its
+    // outputs for that many rows plus an eighth, launches its permute behind the layout and keeps the
+    // result if the rows in use fit and fill at least four fifths of it; otherwise it permutes again
+    // into exact outputs, as a first call of a geometry does.  Read and written with the mailbox held.
+    struct OutputForecast {
+        int64_t tokens = -1, topk = 0, experts = 0, alignment = 0, hidden = 0;
+        bool expand = false;
+        int64_t used_rows = 0;
+    };
+    int64_t forecast_rows(const OutputForecast& key) const {
+        const OutputForecast& seen = forecast_;
+        if (seen.tokens != key.tokens || seen.topk != key.topk || seen.experts != key.experts || seen.alignment != key.alignment ||
+            seen.hidden != key.hidden || seen.expand != key.expand || seen.used_rows <= 0)
+            return 0;
+        return seen.used_rows + (seen.used_rows + 7) / 8;
+    }
+    void note_used_rows(OutputForecast key, int64_t used_rows) {
+        key.used_rows = used_rows;
+        forecast_ = key;
+    }
+
     // Share of the routing choices that were valid in the latest fresh expanded dispatch, in 1/65536
     // (65536 before the first one).  A permute that is enqueued before the host knows the count sizes
     // its launch for this share of T * K plus half a percent instead of for all of it (a workgroup
@@ -468,6 +490,7 @@ class PeerRuntime {
     std::atomic<bool> counts_pending_{false};
     std::atomic<bool> counts_failed_{false};
     std::atomic<bool> prefers_exact_outputs_{false};
+    OutputForecast forecast_;
     std::atomic<int64_t> valid_share_65536_{65536};
     std::deque<RememberedHandle> remembered_;  // newest first
     std::array<std::shared_ptr<RebuiltHandle>, kRebuiltHandles> rebuilt_;
@@ -893,9 +916,21 @@ DispatchResult dispatch(PeerRuntime& runtime,
         const int64_t choice_bound = expand ? tokens * topk : tokens;
         const int64_t gap_bound = expand ? local_experts * (alignment - 1) : 0;
         const int64_t row_bound = choice_bound + gap_bound;
-        const int order_switch = tuning_switch("FRESH_OUTPUTS");  // 0: always exact, 1: at the bound whenever the rule allows
-        const bool speculative = tokens > 0 && gap_bound * 8 <= choice_bound && row_bound <= std::numeric_limits<int32_t>::max() &&
-                                 order_switch != 0 && (order_switch == 1 || !runtime.prefers_exact_outputs());
+        const int order_switch = tuning_switch("FRESH_OUTPUTS");  // 0: always exact, 1: at the bound whenever the rule allows it
+        const bool bound_rule = gap_bound * 8 <= choice_bound;
+        PeerRuntime::OutputForecast geometry;
+        geometry.tokens = tokens, geometry.topk = topk, geometry.experts = local_experts, geometry.alignment = alignment;
+        geometry.hidden = hidden, geometry.expand = expand;
+        // rows the outputs are allocated for ahead of the counts: the bound where it is close, else what
+        // the latest call of this geometry used plus an eighth, else nothing (the exact order)
+        int64_t early_rows = 0;
+        if (tokens > 0 && order_switch != 0 && row_bound <= std::numeric_limits<int32_t>::max()) {
+            if (bound_rule && (order_switch == 1 || !runtime.prefers_exact_outputs()))
+                early_rows = row_bound;
+            else if (!bound_rule)
+                early_rows = std::min(row_bound, runtime.forecast_rows(geometry));
+        }
+        const bool speculative = early_rows > 0;
         if (speculative) {
             // enqueued straight from the arena's pointers: the tensors of the handle are made below,
             // while the GPU works
@@ -908,8 +943,8 @@ DispatchResult dispatch(PeerRuntime& runtime,
             fresh.expert_counts = base64;
             fresh.expert_offsets = base64 + at_offsets;
             try {
-                allocate_outputs(row_bound, tokens);
-                launch_permute(fresh, tokens, row_bound, /*count_on_device=*/true);
+                allocate_outputs(early_rows, tokens);
+                launch_permute(fresh, tokens, early_rows, /*count_on_device=*/true);
             } catch (...) {
                 // The layout is under way and will publish its counts whatever went wrong here (most
                 // likely the allocation at the bound): the turn at the mailbox is settled before the
@@ -962,7 +997,10 @@ DispatchResult dispatch(PeerRuntime& runtime,
         const int64_t used_rows = expand ? expanded_capacity : recv_count;
         const bool bound_is_close = used_rows * 5 >= row_bound * 4;  // the bound holds at most 1.25 x the rows in use
         TORCH_CHECK(used_rows <= row_bound, "receive rows exceed their upper bound");
-        if (speculative && bound_is_close) {
+        // the early outputs are kept when every row in use has a place in them and they hold at most 1.25 x those rows
+        const bool early_outputs_fit = speculative && used_rows <= early_rows && used_rows * 5 >= early_rows * 4;
+        runtime.note_used_rows(geometry, used_rows);
+        if (early_outputs_fit) {
             out_x = out_x.narrow(0, 0, used_rows);
             if (!expand)
                 out_indices = out_indices.narrow(0, 0, recv_count);
@@ -973,7 +1011,7 @@ DispatchResult dispatch(PeerRuntime& runtime,
             if (recv_count > 0)
                 launch_permute(view_of(metadata), recv_count, expanded_capacity);
         }
-        if (tokens > 0 && gap_bound * 8 <= choice_bound)
+        if (tokens > 0 && bound_rule)
             runtime.note_output_fill(bound_is_close);
         if (expand)
             runtime.remember_private(metadata, alignment);

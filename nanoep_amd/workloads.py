@@ -42,6 +42,14 @@ WORKLOADS = {
                           "8192 x 2048, 128 experts top-8 with per-expert bias, expanded, alignment 128, zero_padding, "
                           "async_op with the consumer waiting on the completion event, combine returning the weights",
                           async_op=True, combine_weights=True),
+    # short payload rows: one and two 1 KiB chunks a row
+    "short-rows-512": Workload("short-rows-512", 32768, 512, 64, 8, "softmax-topk-dropout", True, 1, True,
+                               "32768 x 512, 64 experts top-8, 10% of choices masked, expanded + zero_padding"),
+    "short-rows-1024": Workload("short-rows-1024", 32768, 1024, 64, 8, "softmax-topk-dropout", True, 1, True,
+                                "32768 x 1024, 64 experts top-8, 10% of choices masked, expanded + zero_padding"),
+    # the one shape the reference publishes latencies for (its chart: 256 tokens, hidden 4096, top-8, expanded, 2 GPUs)
+    "latency-256": Workload("latency-256", 256, 4096, 64, 8, "softmax-topk-dropout", True, 1, False,
+                            "256 x 4096, 64 experts top-8, 10% of choices masked, expanded: a latency point, not a bandwidth one"),
 }
 
 

@@ -214,6 +214,36 @@ def test_fresh_dispatch_allocation_orders(device, alignment, at_bound):
         assert torch.equal(replay.topk_weights, fresh.topk_weights)
 
 
+def test_fresh_dispatch_with_large_alignment_gaps_allocates_by_what_the_last_call_used(device):
+    """Alignment 64 on 8 experts: the upper bound of the shapes is far from what routing fills, so the
+    first call of a geometry allocates after the counts are known.  The next one allocates for what
+    that call used plus an eighth, ahead of the counts, and keeps the result when the rows in use fit
+    and fill four fifths of it; a batch that uses far fewer rows, or more than were allocated, is
+    permuted again into exact outputs.  Every result is the oracle's and holds at most 1.25 times its rows."""
+    tokens, experts, topk, hidden, alignment = 300, 8, 4, 512, 64
+    x, w = cases.payload(tokens, hidden, seed=2), cases.gate_weights(tokens, topk)
+    dense = cases.routing("random", tokens, experts, topk, seed=1)
+    similar = cases.routing("random", tokens, experts, topk, seed=2)
+    sparse = dense.clone()
+    sparse[tokens // 3:] = -1
+    with Buffer(None, EPConfig(experts, topk, hidden, tokens)) as buffer:
+        held = []
+        for idx in (dense, similar, sparse, sparse, dense, dense):
+            result = buffer.dispatch(x.to(device), topk_idx=idx.to(device), weights=w.to(device), do_expand=True,
+                                     alignment=alignment, zero_padding=True)
+            assert_dispatch_result(result, x, idx, w, experts, True, alignment, True)
+            assert result.x.untyped_storage().nbytes() <= 1.25 * result.x.nbytes + 512
+            held.append(held_rows(result.x, hidden) - result.x.shape[0])
+            replay = buffer.dispatch(x.to(device), weights=w.to(device), handle=result.handle, zero_padding=True)
+            assert torch.equal(replay.x.view(torch.int16), result.x.view(torch.int16))
+        # first of a geometry: exact; same fill: early outputs kept; far fewer rows: exact; same again: early;
+        # far more rows than allocated: exact; same again: early
+        assert [extra > 0 for extra in held] == [False, True, False, True, False, True]
+        # another geometry (other alignment) starts over
+        other = buffer.dispatch(x.to(device), topk_idx=dense.to(device), do_expand=True, alignment=32)
+        assert held_rows(other.x, hidden) == other.x.shape[0]
+
+
 @pytest.mark.parametrize("switch,at_bound", [("0", False), ("1", True)], ids=["always-exact", "at-the-bound"])
 def test_fresh_output_order_can_be_forced(device, tuning, switch, at_bound):
     """The FRESH_OUTPUTS switch at 0 allocates a fresh dispatch's outputs after the counts are known whatever
