@@ -97,6 +97,11 @@ class CudaBuffer:
         self._handle = self._runtime.export_local_handle()
         self._runtime.import_peer_handles([self._handle])
         self._comm_stream = torch.cuda.Stream(device=self._device)
+        # Calls with a compute-unit budget below the whole device run on a stream of the runtime's whose
+        # kernels are confined to that many CUs (see _stream_for); `_active_stream` is the stream the
+        # latest call ran on, which the next call's stream is ordered behind.
+        self._budget_streams: dict[int, torch.cuda.Stream] = {}
+        self._active_stream = self._comm_stream
         self._closed = False
 
     @staticmethod
@@ -133,6 +138,25 @@ class CudaBuffer:
         if self._auto_num_sms is None:
             self._auto_num_sms = whole
         return self._auto_num_sms
+
+    def _stream_for(self, budget: int) -> torch.cuda.Stream:
+        """The stream a call with this compute-unit budget is handed.  The whole device: the buffer's
+        communication stream.  Less: a stream created with a CU mask of about `budget` compute units,
+        the same number on every XCD (the MI355X-native form of the reference's SM budget,
+        nano_ep/backends/cuda.py:233-244, csrc/pipeline.cu:20-24); such a call runs there whether it is
+        asynchronous or not.  All of a buffer's calls stay ordered one behind the other: a call whose
+        stream differs from the previous call's waits for it."""
+        stream = self._comm_stream
+        if 0 < budget < self._device_sms:
+            stream = self._budget_streams.get(budget)
+            if stream is None:
+                raw = self._runtime.budget_stream(budget)
+                stream = torch.cuda.ExternalStream(raw, device=self._device) if raw else self._comm_stream
+                self._budget_streams[budget] = stream
+        if stream is not self._active_stream:
+            stream.wait_stream(self._active_stream)
+            self._active_stream = stream
+        return stream
 
     # ------------------------------------------------------------------ dispatch
 
@@ -189,7 +213,7 @@ class CudaBuffer:
             geometry.num_experts, geometry.num_max_tokens_per_rank, slot_alignment,
             known_tensors, known_capacity,
             self._allow_multiple_reduction, expand, zero_padding, budget,
-            self._comm_stream.cuda_stream, _raw_event(previous_event), async_op,
+            self._stream_for(budget).cuda_stream, _raw_event(previous_event), async_op,
         )
         if not replay:
             handle = self._new_handle(metadata, received, capacity, expand, slot_alignment, x.dtype, budget)
@@ -286,7 +310,7 @@ class CudaBuffer:
             (combined, restored), completed = self._backend.combine(
                 self._runtime, x, metadata, weights, bias,
                 self._config.num_max_tokens_per_rank, expand, self._allow_multiple_reduction, budget,
-                self._comm_stream.cuda_stream, _raw_event(previous_event), async_op,
+                self._stream_for(budget).cuda_stream, _raw_event(previous_event), async_op,
             )
             event = CudaEvent(completed, keepalive=(self, x, handle, weights, bias)) if async_op else None
         return NativeCombineResult(x=combined, topk_weights=None if weights is None else restored, event=event)
@@ -295,8 +319,14 @@ class CudaBuffer:
 
     @property
     def comm_stream(self) -> torch.cuda.Stream:
-        """The stream asynchronous dispatch and combine kernels are launched on."""
+        """The stream asynchronous dispatch and combine kernels are launched on (calls with a
+        compute-unit budget below the whole device: `budget_stream`)."""
         return self._comm_stream
+
+    def budget_stream(self, num_sms: int) -> torch.cuda.Stream:
+        """The stream calls with this compute-unit budget run on."""
+        self._require_open()
+        return self._stream_for(self._resolve_num_sms(num_sms, None))
 
     def close(self):
         """Drain the GPU and release the runtime.  A second call does nothing; dispatch and combine
@@ -304,6 +334,8 @@ class CudaBuffer:
         if self._closed:
             return
         torch.cuda.synchronize(self._device)
+        self._budget_streams.clear()
+        self._active_stream = self._comm_stream
         self._runtime.close_peer_mappings()
         self._runtime.close()
         self._closed = True

@@ -402,6 +402,60 @@ class PeerRuntime {
         return workspace_;
     }
 
+    // The stream for calls with a compute-unit budget below the whole device (the reference sizes its
+    // cooperative grids with num_sms, csrc/pipeline.cu:20-24, so that communication kernels leave
+    // compute units to the caller's own kernels; these kernels are sized by the work, so the budget
+    // is enforced where the hardware offers it: a stream created with a CU mask).  Returns the raw
+    // handle of a stream whose kernels run on about `cus` compute units, the same number on every
+    // XCD; 0 when the budget is the whole device or the device's shape does not allow an even mask.
+    // The streams are made on first use, shared by all runtimes of the process and never destroyed:
+    // the caching allocator remembers the streams a block was used on and visits them when the block
+    // is freed, which may be long after the buffer that used them is closed.
+    //
+    // Which mask bit is which CU differs between descriptions of the interface (bit i on XCD i mod N,
+    // or XCDs one after the other), so the mask is one that gives every XCD the same number of CUs
+    // under both readings: with N XCDs of P CUs, bit P*a + N*b + c is set when (a + c) mod N < t.
+    // That confines the budget to steps of P (32 of 256 on an MI355X), rounded down, at least one step.
+    int64_t budget_stream(int cus) {
+        TORCH_CHECK(!closed_.load(), "PeerRuntime is closed");
+        int device_cus = 0, xcds = 0;
+        check_status(nanoep_device_topology(&device_cus, &xcds, nullptr), "device_topology");
+        if (cus <= 0 || cus >= device_cus || xcds <= 1 || device_cus % xcds != 0 || (device_cus / xcds) % xcds != 0)
+            return 0;
+        const int per_xcd = device_cus / xcds;
+        const int steps = std::max(1, cus / per_xcd);  // of `per_xcd` CUs each: per_xcd / xcds on every XCD
+        if (steps >= xcds)
+            return 0;
+        static std::mutex streams_mutex;
+        static std::vector<std::tuple<int, int, hipStream_t>> streams;  // (device, steps, stream)
+        std::lock_guard<std::mutex> lock(streams_mutex);
+        for (const auto& made : streams)
+            if (std::get<0>(made) == device_ && std::get<1>(made) == steps)
+                return reinterpret_cast<int64_t>(std::get<2>(made));
+        std::vector<uint32_t> mask((device_cus + 31) / 32, 0u);
+        for (int bit = 0; bit < device_cus; ++bit) {
+            const int a = bit / per_xcd, c = bit % xcds;
+            if ((a + c) % xcds < steps)
+                mask[bit / 32] |= 1u << (bit % 32);
+        }
+        DeviceGuard guard(static_cast<c10::DeviceIndex>(device_));
+        hipStream_t stream = nullptr;
+        check_hip(hipExtStreamCreateWithCUMask(&stream, static_cast<uint32_t>(mask.size()), mask.data()), "hipExtStreamCreateWithCUMask");
+        streams.emplace_back(device_, steps, stream);
+        return reinterpret_cast<int64_t>(stream);
+    }
+
+    // compute units a budget stream's kernels can run on (what budget_stream rounds `cus` to)
+    int budget_stream_cus(int cus) const {
+        int device_cus = 0, xcds = 0;
+        check_status(nanoep_device_topology(&device_cus, &xcds, nullptr), "device_topology");
+        if (cus <= 0 || cus >= device_cus || xcds <= 1 || device_cus % xcds != 0 || (device_cus / xcds) % xcds != 0)
+            return device_cus;
+        const int per_xcd = device_cus / xcds;
+        const int steps = std::max(1, cus / per_xcd);
+        return steps >= xcds ? device_cus : steps * per_xcd;
+    }
+
     py::bytes export_local_handle() const {
         std::string tag(64, '\0');
         tag.replace(0, 9, "nanoep-r1");
@@ -459,6 +513,7 @@ class PeerRuntime {
         TORCH_CHECK(mappings_closed_, "Call close_peer_mappings() before close()");
         window_ = torch::Tensor();
         forget_private();
+
         {
             std::lock_guard<std::mutex> lock(counts_mutex_);
             workspace_ = torch::Tensor();
@@ -646,9 +701,10 @@ bool same_queue(const Stream& a, const Stream& b) { return a.stream() == b.strea
 // A synchronous call must leave its results ordered on the caller's stream, so it runs there
 // directly instead of bouncing through the communication stream with two cross-stream events; it
 // still comes after everything enqueued earlier on the communication stream.
-Stream work_stream(int64_t comm_handle, const Stream& compute, c10::DeviceIndex device, bool async_op) {
+Stream work_stream(int64_t comm_handle, const Stream& compute, c10::DeviceIndex device, bool async_op, bool budgeted) {
     const auto comm = external_stream(comm_handle, device);
-    if (async_op || same_queue(comm, compute))
+    // (a call with a compute-unit budget runs on the stream it was handed: that stream carries the CU mask)
+    if (async_op || budgeted || same_queue(comm, compute))
         return comm;
     // While the caller's stream is being captured into a graph no other stream may be queried;
     // a captured call is ordered by the graph alone.
@@ -742,7 +798,7 @@ DispatchResult dispatch(PeerRuntime& runtime,
     const int64_t local_experts = num_experts;
 
     const auto compute = c10::hip::getCurrentHIPStreamMasqueradingAsCUDA(device);
-    const auto comm = work_stream(comm_stream, compute, device, async_op);
+    const auto comm = work_stream(comm_stream, compute, device, async_op, cu_budget != 0);
     order_comm_after_inputs(comm, compute, previous_event, async_op);
 
     StreamGuard comm_guard(comm.unwrap());
@@ -1087,7 +1143,7 @@ CombineResult combine(PeerRuntime& runtime,
     const int cu_budget = resolve_cu_budget(num_sms, device);
 
     const auto compute = c10::hip::getCurrentHIPStreamMasqueradingAsCUDA(device);
-    const auto comm = work_stream(comm_stream, compute, device, async_op);
+    const auto comm = work_stream(comm_stream, compute, device, async_op, cu_budget != 0);
     order_comm_after_inputs(comm, compute, previous_event, async_op);
     StreamGuard comm_guard(comm.unwrap());
 
@@ -1189,6 +1245,8 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, module) {
         .def("close_peer_mappings", &nanoep::PeerRuntime::close_peer_mappings)
         .def("private_recalls", &nanoep::PeerRuntime::private_recalls)
         .def("rebuilds", &nanoep::PeerRuntime::rebuilds)
+        .def("budget_stream", &nanoep::PeerRuntime::budget_stream)
+        .def("budget_stream_cus", &nanoep::PeerRuntime::budget_stream_cus)
         .def("counts_failed", &nanoep::PeerRuntime::counts_failed)
         .def("prefers_exact_outputs", &nanoep::PeerRuntime::prefers_exact_outputs)
         .def("valid_share_65536", &nanoep::PeerRuntime::valid_share_65536)

@@ -13,8 +13,12 @@ from nanoep_amd.config import EPConfig as ConfigAlias
 
 
 class FakeStream:
-    def __init__(self, handle):
+    def __init__(self, handle, device=None):
         self.cuda_stream = handle
+        self.waited_for = []
+
+    def wait_stream(self, other):
+        self.waited_for.append(other.cuda_stream)
 
 
 class FakeTensor:
@@ -92,8 +96,12 @@ def context(monkeypatch):
     buffer._auto_num_sms = None
     buffer._closed = False
     buffer._world_size = 1
-    buffer._runtime = object()
+    # budgets of 64 compute units and more get a stream of their own from the runtime
+    buffer._runtime = SimpleNamespace(budget_stream=lambda cus: 1000 + cus if cus >= 64 else 0)
+    monkeypatch.setattr(api.torch.cuda, "ExternalStream", FakeStream)
     buffer._comm_stream = FakeStream(11)
+    buffer._budget_streams = {}
+    buffer._active_stream = buffer._comm_stream
     buffer._backend = SimpleNamespace(dispatch=dispatch, combine=combine)
     buffer._allow_multiple_reduction = False
     return SimpleNamespace(buffer=buffer, calls=calls, tensor=FakeTensor,
@@ -163,6 +171,27 @@ def test_cached_dispatch_forwards_the_handle(context, expand, weighted, asynchro
     assert cached == old_metadata and capacity == first.handle.layout.expanded_capacity
     assert alignment == 4 and got_expand is expand and zero_padding is False and got_async is asynchronous
     assert num_sms == 24  # the handle's saved budget is inherited
+
+
+def test_a_compute_unit_budget_picks_the_stream_and_keeps_the_calls_in_order(context):
+    """A call with a budget below the whole device is handed the runtime's stream for that budget
+    (sync or async), the others the communication stream; a call whose stream differs from the
+    previous call's is ordered behind it."""
+    buffer = context.buffer
+    x = context.tensor("x", torch.zeros((2, 256), dtype=torch.bfloat16))
+    streams = lambda: [call.args[13] if call.kind == "dispatch" else call.args[9] for call in context.calls]
+    first = buffer.dispatch(x, topk_idx=context.indices, do_expand=True, num_sms=64, async_op=True)
+    assert streams() == [1064] and buffer._budget_streams[64].waited_for == [11]
+    buffer.dispatch(x, handle=first.handle)  # inherits the handle's budget
+    assert streams() == [1064, 1064] and buffer._budget_streams[64].waited_for == [11]
+    payload = context.tensor("y", torch.zeros((first.handle.layout.expanded_capacity, 256), dtype=torch.bfloat16))
+    buffer.combine(payload, first.handle, num_sms=256)  # the whole device: the communication stream, behind the budget stream
+    assert streams()[-1] == 11 and buffer._comm_stream.waited_for == [1064]
+    buffer.combine(payload, first.handle, num_sms=128)
+    assert streams()[-1] == 1128 and buffer._budget_streams[128].waited_for == [11]
+    buffer.dispatch(x, topk_idx=context.indices, num_sms=24)  # the runtime has no stream for so few: the communication stream
+    assert streams()[-1] == 11 and buffer._comm_stream.waited_for == [1064, 1128]
+    assert buffer.budget_stream(64) is buffer._budget_streams[64]
 
 
 def test_dispatch_argument_rules(context):

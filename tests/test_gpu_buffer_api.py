@@ -524,6 +524,56 @@ def test_the_fifth_oldest_handle_of_a_buffer_still_takes_the_slot_order_walk(dev
         assert buffer._runtime.rebuilds() == 1 and buffer._runtime.private_recalls() == 8
 
 
+def test_a_compute_unit_budget_confines_the_kernels_and_changes_no_result(device):
+    """num_sms below the device's compute units: the call runs on a stream created with a CU mask of
+    about that many units (the same number on every XCD).  Results are the oracle's whatever the
+    budget, synchronous or not, calls with different budgets stay ordered one behind the other, and
+    the kernel time grows as the budget shrinks (a 16 MiB payload on a quarter of the device takes
+    well over twice as long as on all of it)."""
+    tokens, experts, topk, hidden, alignment = 2048, 16, 4, 4096, 8
+    idx = cases.routing("dropout", tokens, experts, topk, seed=4)
+    x, w = cases.payload(tokens, hidden, seed=5), cases.gate_weights(tokens, topk)
+    cus = torch.cuda.get_device_properties(device).multi_processor_count
+    with Buffer(None, EPConfig(experts, topk, hidden, tokens)) as buffer:
+        quarter = cus // 4
+        assert buffer._runtime.budget_stream_cus(quarter) == quarter and buffer._runtime.budget_stream(cus) == 0
+        assert buffer.budget_stream(quarter) is not buffer.comm_stream and buffer.budget_stream(cus) is buffer.comm_stream
+        fresh = buffer.dispatch(x.to(device), topk_idx=idx.to(device), weights=w.to(device), do_expand=True, alignment=alignment,
+                                zero_padding=True, num_sms=quarter)
+        lay = assert_dispatch_result(fresh, x, idx, w, experts, True, alignment, True)
+        assert fresh.handle.num_sms == quarter
+        for budget, asynchronous in ((quarter, True), (cus, True), (cus // 2, False), (None, False), (cus, False), (quarter, True)):
+            replay = buffer.dispatch((x * 2).to(device), weights=w.to(device), handle=fresh.handle, zero_padding=True,
+                                     num_sms=budget, async_op=asynchronous)
+            if asynchronous:
+                replay.event.current_stream_wait()
+            assert_dispatch_result(replay, x * 2, idx, w, experts, True, alignment, True)
+            combined = buffer.combine(replay.x, fresh.handle, weights=replay.topk_weights, num_sms=budget, async_op=asynchronous)
+            if asynchronous:
+                combined.event.current_stream_wait()
+            want, want_w = oracle.combine(replay.x.cpu(), lay.recv_metadata(True), lay.dst_slots, do_expand=True, weights=replay.topk_weights.cpu())
+            assert_same_bits(combined.x, want, f"combine with budget {budget}")
+            assert_same_bits(combined.topk_weights, want_w, f"combine weights with budget {budget}")
+
+        def kernel_us(budget):
+            stream = buffer.budget_stream(budget)
+            payload = x.to(device)
+            with torch.cuda.stream(stream):
+                for _ in range(5):
+                    buffer.dispatch(payload, handle=fresh.handle, num_sms=budget)
+                begin, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                torch.cuda.synchronize()
+                begin.record(stream)
+                for _ in range(20):
+                    buffer.dispatch(payload, handle=fresh.handle, num_sms=budget)
+                end.record(stream)
+                torch.cuda.synchronize()
+            return begin.elapsed_time(end) * 1e3 / 20
+
+        whole, confined = kernel_us(cus), kernel_us(quarter)
+        assert confined > 2 * whole, (whole, confined)
+
+
 @pytest.mark.parametrize("expand", [False, True], ids=["compact", "expanded"])
 def test_async_streams_and_previous_event(device, expand):
     tokens, experts, topk, hidden = 301, 16, 4, 1024
