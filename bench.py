@@ -61,6 +61,9 @@ def parse_args():
                              "it is a specification, not a performance path)")
     parser.add_argument("--regions", type=int, default=REGIONS)
     parser.add_argument("--region-launches", type=int, default=REGION_LAUNCHES)
+    parser.add_argument("--series", choices=["all", "basic", "streams"], default="all",
+                        help="`basic`: only fresh dispatches and the cold step / dispatch / combine series (what a profiler run wants: "
+                             "every launch of a kernel name is then the same work); `streams`: only the plain streams")
     parser.add_argument("--no-calibration", dest="calibration", action="store_false",
                         help="skip the plain streams (nanoep_stream_probe) that give every roofline entry its frac_of_stream_ceiling")
     parser.add_argument("--calibration-copy-mib", type=int, default=0,
@@ -358,6 +361,24 @@ def roofline_entry(kernel, workload_name, nbytes, median_us, min_us, ceiling=Non
     return entry
 
 
+def measure_streams(workload, args, device):
+    """Only the plain streams of one workload's bytes (`--series streams`)."""
+    import torch
+
+    from nanoep_amd import Buffer, EPConfig, workloads
+
+    x_cpu, idx_cpu, w_cpu = workloads.make_inputs(workload, seed=0)
+    with Buffer(None, EPConfig(workload.experts, workload.topk, workload.hidden, workload.tokens)) as buffer:
+        layout = buffer.dispatch(x_cpu.to(device), topk_idx=idx_cpu.to(device), do_expand=workload.expand,
+                                 alignment=workload.alignment).handle.layout
+        received, capacity, assignments = layout.recv_count, layout.expanded_capacity, int(layout.expert_counts.sum().item())
+    torch.cuda.empty_cache()
+    return {"received_rows": received, "assignments": assignments, "expanded_capacity": capacity,
+            "timing": {"warmup_launches": WARMUP_MIN, "regions": min(max(1, args.regions), 3), "launches_per_region": min(max(1, args.region_launches), 40)},
+            "stream_ceiling": stream_ceilings(workload, received, assignments, capacity, min(max(1, args.regions), 3),
+                                              min(max(1, args.region_launches), 40))}
+
+
 def measure(workload, args, device, detailed):
     """All figures of one workload.  `detailed` adds the layout, seven-tensor-handle and --steps
     figures (the headline workload)."""
@@ -484,25 +505,26 @@ def measure(workload, args, device, detailed):
                 samples.append(time.perf_counter() - t0)
             return statistics.median(samples[WARMUP_MIN:]) * 1e6
 
+        everything = args.series == "all"
         step_wall, step_gpu = series(step)
         _, dispatch_gpu = series(do_dispatch)
         _, combine_gpu = series(do_combine)
-        _, hot_gpu = series(do_dispatch_hot)
+        _, hot_gpu = series(do_dispatch_hot) if everything else (None, dispatch_gpu)
         # the same two dispatch series with the walk's window-wise source prefetch forced on and off
         # (the library turns it on by itself for rows of two chunks only, where it costs nothing with
         # cache-resident sources; elsewhere it trades the one for the other and is the caller's switch)
         prefetch_gpu = {}
-        if workload.expand:
+        if workload.expand and everything:
             for setting in (0, 1):
                 library.nanoep_set_tuning(b"DISPATCH_PREFETCH", setting)
                 prefetch_gpu[setting] = (series(do_dispatch)[1], series(do_dispatch_hot)[1])
             library.nanoep_set_tuning(b"DISPATCH_PREFETCH", -1)
-        cached_latency = call_to_complete(do_dispatch)
-        combine_latency = call_to_complete(do_combine)
-        layout_us = layout_gpu_us(workload, idx) if detailed else None
+        cached_latency = call_to_complete(do_dispatch) if everything else 0.0
+        combine_latency = call_to_complete(do_combine) if everything else 0.0
+        layout_us = layout_gpu_us(workload, idx) if detailed and everything else 0.0
 
         seven = None
-        if detailed and workload.expand:
+        if detailed and workload.expand and everything:
             # A caller that keeps more handles alive than the runtime remembers, and only the seven
             # tensors of each: four more fresh dispatches (other routings) make `handle` the fifth
             # oldest, and its replays go through a copy without the private tensors.  The first replay
@@ -542,7 +564,7 @@ def measure(workload, args, device, detailed):
                    "gpu_us_per_step": round(cli_gpu / max(1, args.steps) * 1e6, 2)}
 
         side = None
-        if asynchronous:
+        if asynchronous and everything:
             # the caller on a stream of its own: every call makes the communication stream wait for the
             # caller's stream and the caller's stream wait for the call's completion event
             with torch.cuda.stream(torch.cuda.Stream(device=device)):
@@ -554,7 +576,7 @@ def measure(workload, args, device, detailed):
                     "timed": "HIP events on the caller's stream around back-to-back dispatch -> event.current_stream_wait() calls: two "
                              "cross-stream waits per call on top of the kernel"}
 
-        ceilings = stream_ceilings(workload, n_recv, assignments, capacity, min(regions, 3), min(launches, 40)) if args.calibration else None
+        ceilings = stream_ceilings(workload, n_recv, assignments, capacity, min(regions, 3), min(launches, 40)) if args.calibration and everything else None
 
     wall_us, wall_us_min = summarize(step_wall, launches)
     gpu_step_us, gpu_step_us_min = summarize(step_gpu, launches)
@@ -665,6 +687,9 @@ def main():
     device = torch.device("cuda", 0)
     torch.cuda.set_device(device)
 
+    if args.series == "streams":
+        print(json.dumps({name: measure_streams(workloads.WORKLOADS[name], args, device) for name in names}), flush=True)
+        return 0
     workload = workloads.WORKLOADS[names[0]]
     measured = measure(workload, args, device, detailed=True)
     cli = measured["cli_region"]

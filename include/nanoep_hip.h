@@ -136,8 +136,12 @@ int nanoep_layout(const int64_t* topk_idx, int64_t num_tokens, int num_topk, int
 
 /*
  * nanoep_layout without the workspace arguments, for callers that cannot allocate device memory
- * (code under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc).  It has
- * no counterpart in the reference.  The kernels' workspace is a file-scope device array of
+ * (tight serving loops, harnesses that forbid hipMalloc, code that records its launches into a HIP
+ * graph).  It has no counterpart in the reference.  A caller that captures it must know two things:
+ * the first call on a device resolves the array's address through the runtime and belongs outside
+ * the capture, and the -1 this call stores into host_counts[0] is a host store made when the call
+ * is made, not part of the graph: before every launch of the graph the caller stores -1 there
+ * itself, or nanoep_wait_counts answers with the previous launch's counts.  The kernels' workspace is a file-scope device array of
  * NANOEP_STATIC_SCRATCH_BYTES that each GPU holds until the process ends; the call allocates
  * and frees nothing (its first call on a device looks the array's address up once).  Inputs, outputs
  * and results are those of nanoep_layout.  A geometry whose workspace

@@ -15,7 +15,9 @@ def test_every_declared_symbol_is_exported():
     declared = cabi.declared_symbols()
     assert {"nanoep_layout", "nanoep_dispatch", "nanoep_combine", "nanoep_wait_counts", "nanoep_window_layout",
             "nanoep_layout_workspace_bytes", "nanoep_copy_bytes", "nanoep_abi_version",
-            "nanoep_slot_order_entries", "nanoep_layout_block_tokens"} <= set(declared)
+            "nanoep_slot_order_entries", "nanoep_layout_block_tokens", "nanoep_layout_static", "nanoep_rebuild_order",
+            "nanoep_rebuild_workspace_bytes", "nanoep_rebuild_window_tokens", "nanoep_stream_probe", "nanoep_set_tuning",
+            "nanoep_get_tuning", "nanoep_reset_tuning", "nanoep_device_topology"} <= set(declared)
     library = cabi.lib()
     for name in declared:
         assert hasattr(library, name), f"{name} is declared in include/nanoep_hip.h but not exported"
@@ -89,6 +91,79 @@ def test_argument_checks_come_before_any_device_work():
     assert library.nanoep_layout_block_tokens(4096, 256, -1) == 0
     out = (ctypes.c_int64 * 4)()
     assert library.nanoep_wait_counts(null, null, 0.0, out) == 1
+
+
+def test_tuning_switches_are_set_through_the_abi_and_read_from_the_environment_once(monkeypatch):
+    """The switches are parsed from NANOEP_<NAME> once; afterwards only nanoep_set_tuning changes
+    them (an environment variable set later is not seen until nanoep_reset_tuning reads it)."""
+    library = cabi.lib()
+    assert cabi.get_tuning("WINDOW_TOKENS") == 0 and cabi.get_tuning("DISPATCH_ORDER") == -1 and cabi.get_tuning("XCDS") == 0
+    value = ctypes.c_int(0)
+    assert library.nanoep_get_tuning(b"NO_SUCH_SWITCH", ctypes.byref(value)) == 1
+    assert library.nanoep_set_tuning(b"NO_SUCH_SWITCH", 3) == 1 and library.nanoep_set_tuning(None, 3) == 1
+    try:
+        assert library.nanoep_set_tuning(b"WINDOW_TOKENS", 128) == 0
+        assert cabi.get_tuning("WINDOW_TOKENS") == 128
+        assert library.nanoep_layout_block_tokens(4096, 256, 7168) == 128  # the forced window shows in the plan
+        monkeypatch.setenv("NANOEP_WINDOW_TOKENS", "192")
+        assert library.nanoep_layout_block_tokens(4096, 256, 7168) == 128  # the environment is not read again by a call
+        with cabi.forced_tuning({"WINDOW_TOKENS": 64, "DISPATCH_SPAN": None}):
+            assert cabi.get_tuning("WINDOW_TOKENS") == 64
+        assert cabi.get_tuning("WINDOW_TOKENS") == 128
+        library.nanoep_reset_tuning()
+        assert cabi.get_tuning("WINDOW_TOKENS") == 192
+    finally:
+        monkeypatch.delenv("NANOEP_WINDOW_TOKENS", raising=False)
+        library.nanoep_reset_tuning()
+    assert cabi.get_tuning("WINDOW_TOKENS") == 0 and library.nanoep_layout_block_tokens(4096, 256, 7168) == 256
+
+
+def test_topology_defaults_and_overrides_size_the_windows():
+    """Without a device the plans assume the MI355X's 256 CUs, 8 XCDs and 4 MiB of L2 per XCD; the
+    XCDS and L2_BYTES switches stand in for other parts: the window follows the L2, the number of
+    windows a batch is cut into follows the XCD count."""
+    library = cabi.lib()
+    assert cabi.device_topology() == (256, 8, 4 << 20)
+    try:
+        library.nanoep_set_tuning(b"L2_BYTES", 8 << 20)
+        assert cabi.device_topology() == (256, 8, 8 << 20)
+        assert [library.nanoep_layout_block_tokens(100000, 256, h) for h in (2048, 4096, 8192, 16384)] == [1024, 512, 512, 256]
+        library.nanoep_set_tuning(b"L2_BYTES", 2 << 20)
+        assert [library.nanoep_layout_block_tokens(100000, 256, h) for h in (4096, 8192, 16384)] == [256, 128, 64]
+        library.nanoep_set_tuning(b"L2_BYTES", 0)
+        library.nanoep_set_tuning(b"XCDS", 4)
+        assert cabi.device_topology() == (256, 4, 4 << 20)
+        # 1024 tokens of 7168 elements: eight windows of 128 tokens for 8 XCDs, four of 256 for 4
+        assert library.nanoep_layout_block_tokens(1024, 256, 7168) == 256
+        library.nanoep_set_tuning(b"XCDS", 0)
+        assert library.nanoep_layout_block_tokens(1024, 256, 7168) == 128
+    finally:
+        library.nanoep_reset_tuning()
+
+
+def test_rebuild_and_stream_probe_argument_checks():
+    library = cabi.lib()
+    null = None
+    assert library.nanoep_rebuild_workspace_bytes(4096, 8) >= (4096 // 32) * 4 and library.nanoep_rebuild_workspace_bytes(-1, 8) == 0
+    assert library.nanoep_rebuild_workspace_bytes(16, 0) == 0 and library.nanoep_rebuild_workspace_bytes(16, 33) == 0
+    # the layout's window, halved until a window's T * K entries fit the sort (4096)
+    assert library.nanoep_rebuild_window_tokens(4096, 8, 7168) == 256 and library.nanoep_rebuild_window_tokens(8192, 8, 2048) == 512
+    assert library.nanoep_rebuild_window_tokens(32768, 8, 512) == 512 and library.nanoep_rebuild_window_tokens(4096, 32, 7168) == 128
+    assert library.nanoep_rebuild_window_tokens(4096, 0, 7168) == 0
+    # no tokens, missing pointers, a tag with low bits, a negative tag, too many (token, k) pairs
+    assert library.nanoep_rebuild_order(8, 8, 0, 0, 0, 2, 4, 256, 8, 8, 8, 1024, null, 0, null) == 1
+    assert library.nanoep_rebuild_order(8, null, 1, 4, 4, 2, 4, 256, 8, 8, 8, 1024, null, 0, null) == 1
+    assert library.nanoep_rebuild_order(8, 8, 1, 4, 4, 2, 4, 256, 8, 8, 8, 1024, null, 5, null) == 1
+    assert library.nanoep_rebuild_order(8, 8, 1, 4, 4, 2, 4, 256, 8, 8, 8, 1024, null, -(1 << 32), null) == 1
+    assert library.nanoep_rebuild_order(8, 8, 1, 4, 1 << 30, 8, 4, 256, 8, 8, 8, 1 << 30, null, 0, null) == 1
+    assert library.nanoep_rebuild_order(8, 8, 5, 4, 4, 2, 4, 256, 8, 8, 8, 1024, null, 0, null) == 1  # more rows than tokens
+    assert library.nanoep_rebuild_order(8, 8, 1, 4, 4, 2, 4, 256, 8, 8, 8, 16, null, 0, null) == 3  # workspace too small
+    library.nanoep_stream_probe.argtypes = [ctypes.c_int, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int64, ctypes.c_int, ctypes.c_int,
+                                            ctypes.c_int64, ctypes.c_int, ctypes.c_void_p]
+    for bad in ((4, 16, 16, 64, 256, 1, 1, 0), (2, 16, 16, 64, 250, 1, 1, 0), (2, 16, 16, 64, 16384, 1, 1, 0), (2, 16, 16, 64, 256, 3, 1, 0),
+                (2, 16, 16, 64, 256, 2, 64, 0), (3, 16, 16, 60, 256, 2, 64, 0), (2, 16, 16, 64, 256, 2, 1, 17), (2, null, 16, 64, 256, 2, 1, 0),
+                (1, null, null, 64, 256, 1, 1, 0), (0, 16, 24, 64, 256, 1, 1, 0)):
+        assert library.nanoep_stream_probe(*bad, null) == 1, bad
 
 
 def test_wait_counts_reads_a_mailbox_the_host_wrote():

@@ -397,6 +397,20 @@ def test_forced_window_sizes(device, tuning, window, tokens, experts):
     run_dispatch_combine(device, idx, 512, experts, 8, True, True, True, seed=5)
 
 
+@pytest.mark.parametrize("xcds", [1, 2, 3, 4, 8, 16])
+@pytest.mark.parametrize("tokens,experts,topk,hidden,alignment", [(3000, 40, 8, 5120, 16), (5000, 16, 2, 1024, 1), (900, 8, 4, 256, 4)])
+def test_any_xcd_count_gives_the_same_bytes(device, tuning, xcds, tokens, experts, topk, hidden, alignment):
+    """The kernels take the XCD count as an argument (the device's; the XCDS switch stands in for a
+    partitioned or another part).  The block remap is a bijection for any count, so every count gives
+    the oracle's bytes through every walk; what the count changes is locality, which is not tested."""
+    tuning("XCDS", xcds)
+    assert cabi.device_topology()[1] == xcds
+    idx = cases.routing("dropout", tokens, experts, topk, seed=xcds)
+    run_dispatch_combine(device, idx, hidden, experts, alignment, True, True, True, seed=xcds)
+    if xcds in (1, 3):
+        run_dispatch_combine(device, idx, hidden, experts, alignment, False, False, True, seed=xcds)
+
+
 @pytest.mark.parametrize(
     "tokens,experts,topk,hidden,alignment",
     [
