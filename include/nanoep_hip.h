@@ -69,6 +69,7 @@ int nanoep_device_topology(int* out_cus, int* out_xcds, int64_t* out_l2_bytes);
  *   DISPATCH_SPAN (0: by size; 1 | 2 chunks a wavefront of the slot-order walk)
  *   DISPATCH_SIDE (-1; 0 | 1: weights of that walk in workgroups of their own)
  *   DISPATCH_WHOLE_ROWS (-1; 0 | 1: one workgroup a list entry)
+ *   DISPATCH_PREFETCH (-1: by row length; 0 | 1: window-wise source prefetch of that walk)
  *   LAYOUT_LAUNCHES (0; 2 | 3: layout plan)     WINDOW_TOKENS (0; window of the slot-order list)
  *   RECALL_ORDER, FRESH_OUTPUTS, REBUILD_ORDER (-1; 0 | 1: host-extension policies)
  *   XCDS, L2_BYTES (0: ask the device)
@@ -206,10 +207,15 @@ int nanoep_wait_counts(int64_t* host_counts, void* stream, double timeout_second
  * A from the buffer's last word: -1 sizes the launch for the most entries the list can hold (T * K),
  * -g (g > 1) for about g entries, which is cheaper when many choices are masked and correct whatever
  * A turns out to be (workgroups then take several turns).
+ * The slot-order walk can read every window's source rows front to back just ahead of the window's
+ * copies (the DISPATCH_PREFETCH switch; on by itself for rows of 513 to 1024 elements): the same
+ * bytes from HBM, as one sequential burst per window instead of one row at a time among the stores.
  * x / recv_x are bf16, 16-byte aligned, H % 8 == 0.  weights / recv_weights / recv_topk_idx may be
  * NULL (recv_topk_idx must be NULL when expanded).  num_cus is the reference's SM budget
  * (0 = whole device): it is range-checked against the device's compute-unit count and otherwise
- * ignored, because these kernels are sized by the work, not by a cooperative grid.
+ * ignored here, because these kernels are sized by the work, not by a cooperative grid; a caller
+ * that wants the kernels confined to fewer compute units passes a stream created with a CU mask
+ * (hipExtStreamCreateWithCUMask), as the host extension does.
  */
 int nanoep_dispatch(const void* x, const float* weights, const int32_t* recv_metadata, const int64_t* dst_slots,
                     const int32_t* token_slots, const int64_t* slot_order, int64_t slot_order_entries,

@@ -22,7 +22,8 @@
 //                          (list entry, row chunk), token block by token block and expert-major
 //                          inside a block, so a block's source rows stay in one XCD's L2 and every
 //                          expert receives runs of consecutive rows; one 128-bit load and one
-//                          nontemporal 128-bit store per lane.
+//                          nontemporal 128-bit store per lane.  Optionally a few workgroups ahead
+//                          of every window read its source rows front to back (prefetch).
 //   dispatch_rows_kernel : the same work item walked in source-token order (small batches, handles
 //                          without the list); extra work items zero-fill the alignment gaps.
 //   dispatch_compact_kernel / combine_compact_kernel : compact layouts are row copies with holes;
@@ -30,6 +31,10 @@
 //   combine_rows_kernel  : one wavefront per (source token, row chunk): gathers the token's rows in
 //                          ascending k, fp32 accumulate, one round-to-nearest-even bf16 store.
 //   combine_few_rows_kernel : the same for K <= 4 with the slot table, without the bookkeeping.
+//   rebuild_table_kernel + rebuild_order_kernel : the slot table and the slot-order list of a handle
+//                          rebuilt from its recv_metadata and dst_slots alone (an LDS bitonic sort
+//                          of every window's (slot, source) pairs).
+//   stream_probe_kernel  : plain streams in the shape of the row kernels (measured ceilings).
 //
 // Every byte moved is HBM-bound integer/byte work; there is no contraction, hence no MFMA.
 #ifndef NANOEP_DEVICE_H_
