@@ -64,12 +64,12 @@ int nanoep_device_topology(int* out_cus, int* out_xcds, int64_t* out_l2_bytes);
  * (first use of the library); afterwards only these calls change it, so no entry point touches the
  * environment on its way to a launch.  Meant for tests and sweeps: the defaults are the measured
  * best.  No counterpart in the reference.
- *   CHUNKS_PER_BLOCK, ROWS_PER_BLOCK (0: by shape)  workgroup shape of the row kernels
+ *   CHUNKS_PER_BLOCK, ROWS_PER_BLOCK (0: by shape)  workgroup shape of the row kernels (the slot-order
+ *                     walk takes ROWS_PER_BLOCK list entries a workgroup for rows of up to 4 KiB)
  *   DISPATCH_ORDER (-1; 0: token-order walk even when the handle has a slot-order list)
- *   DISPATCH_SPAN (0: by size; 1 | 2 chunks a wavefront of the slot-order walk)
- *   DISPATCH_SIDE (-1; 0 | 1: weights of that walk in workgroups of their own)
- *   DISPATCH_WHOLE_ROWS (-1; 0 | 1: one workgroup a list entry)
- *   DISPATCH_PREFETCH (-1: by row length; 0 | 1: window-wise source prefetch of that walk)
+ *   DISPATCH_SPAN (0: by size; 1 | 2 | 4 chunks a wavefront of the slot-order walk)
+ *   DISPATCH_PREFETCH (-1: on; 0: no window-wise source prefetch in that walk, for sources that are
+ *                     known to sit in the last-level cache)
  *   LAYOUT_LAUNCHES (0; 2 | 3: layout plan)     WINDOW_TOKENS (0; window of the slot-order list)
  *   RECALL_ORDER, FRESH_OUTPUTS, REBUILD_ORDER (-1; 0 | 1: host-extension policies)
  *   XCDS, L2_BYTES (0: ask the device)
@@ -207,9 +207,10 @@ int nanoep_wait_counts(int64_t* host_counts, void* stream, double timeout_second
  * A from the buffer's last word: -1 sizes the launch for the most entries the list can hold (T * K),
  * -g (g > 1) for about g entries, which is cheaper when many choices are masked and correct whatever
  * A turns out to be (workgroups then take several turns).
- * The slot-order walk can read every window's source rows front to back just ahead of the window's
- * copies (the DISPATCH_PREFETCH switch; on by itself for rows of 513 to 1024 elements): the same
- * bytes from HBM, as one sequential burst per window instead of one row at a time among the stores.
+ * The slot-order walk reads every window's source rows front to back just ahead of the window's
+ * copies (unless the DISPATCH_PREFETCH switch is 0): the same bytes from HBM, as one sequential burst
+ * per window instead of one row at a time among the stores.  It serves lists of fewer than 2^29
+ * entries and rows of up to 64 KiB; beyond either the work is walked in source-token order.
  * x / recv_x are bf16, 16-byte aligned, H % 8 == 0.  weights / recv_weights / recv_topk_idx may be
  * NULL (recv_topk_idx must be NULL when expanded).  num_cus is the reference's SM budget
  * (0 = whole device): it is range-checked against the device's compute-unit count and otherwise

@@ -22,7 +22,6 @@ struct SwitchSlot {
 constexpr SwitchSlot kSwitches[] = {
     {"CHUNKS_PER_BLOCK", &Tuning::chunks_per_block}, {"ROWS_PER_BLOCK", &Tuning::rows_per_block},
     {"DISPATCH_ORDER", &Tuning::dispatch_order},     {"DISPATCH_SPAN", &Tuning::dispatch_span},
-    {"DISPATCH_SIDE", &Tuning::dispatch_side},       {"DISPATCH_WHOLE_ROWS", &Tuning::dispatch_whole_rows},
     {"LAYOUT_LAUNCHES", &Tuning::layout_launches},   {"WINDOW_TOKENS", &Tuning::window_tokens},
     {"RECALL_ORDER", &Tuning::recall_order},         {"FRESH_OUTPUTS", &Tuning::fresh_outputs},
     {"REBUILD_ORDER", &Tuning::rebuild_order},       {"XCDS", &Tuning::xcds},

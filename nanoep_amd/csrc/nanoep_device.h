@@ -83,10 +83,8 @@ struct Tuning {
     int chunks_per_block = 0;       // CHUNKS_PER_BLOCK: wavefronts along a row in a workgroup, 0 = by shape
     int rows_per_block = 0;         // ROWS_PER_BLOCK: rows a workgroup, 0 = by shape
     int dispatch_order = -1;        // DISPATCH_ORDER: 0 forces the token-order walk
-    int dispatch_span = 0;          // DISPATCH_SPAN: 1 | 2 chunks a wavefront of the slot-order walk, 0 = by size
-    int dispatch_side = -1;         // DISPATCH_SIDE: 0 | 1 weights of that walk in workgroups of their own
-    int dispatch_whole_rows = -1;   // DISPATCH_WHOLE_ROWS: 0 | 1 the kernel variant for one workgroup a list entry
-    int dispatch_prefetch = -1;     // DISPATCH_PREFETCH: 0 | 1 window-wise source prefetch in the slot-order walk
+    int dispatch_span = 0;          // DISPATCH_SPAN: 1 | 2 | 4 chunks a wavefront of the slot-order walk, 0 = by size
+    int dispatch_prefetch = -1;     // DISPATCH_PREFETCH: 0 = no window-wise source prefetch in the slot-order walk
     int layout_launches = 0;        // LAYOUT_LAUNCHES: 2 | 3 forces the layout plan
     int window_tokens = 0;          // WINDOW_TOKENS: forces the window of the slot-order list
     int recall_order = -1;          // RECALL_ORDER: 0 = seven-tensor handles never get private tensors back (host extension)
@@ -144,6 +142,15 @@ __device__ __forceinline__ void store_vec(u32x4* p, u32x4 v) {
 template <class T>
 __device__ __forceinline__ T uniform_load(const T* p) {
     return *(const __attribute__((address_space(4))) T*)(p);
+}
+
+// Element `index` of such an array, addressed with a 32-bit byte offset (index * sizeof(T) < 2^32):
+// the offset then rides in the load instruction instead of a 64-bit address computation.
+template <class T>
+__device__ __forceinline__ T uniform_load_at(const T* base, uint32_t index) {
+    typedef const __attribute__((address_space(4))) char* ConstantBytes;
+    typedef const __attribute__((address_space(4))) T* ConstantElement;
+    return *(ConstantElement)((ConstantBytes)(base) + index * static_cast<uint32_t>(sizeof(T)));
 }
 
 // n / d for n < 2^31 as one 64-bit multiply and shift: magic = ceil(2^shift / d), shift = 31 + ceil(log2 d).
@@ -204,28 +211,14 @@ struct RowBlocking {
 
 enum WalkShape {
     kTokenOrderWalk,  // two-wavefront workgroups: best or within noise of best for the expanded token-order walks
-    kSlotOrderWalk,   // one workgroup a row up to 16 wavefronts, an even split beyond
     kRowCopyWalk,     // compact layouts (plain row copies): single-wavefront workgroups
 };
 
 inline RowBlocking pick_row_blocking(int chunks, WalkShape shape, const Tuning& tuning) {
     RowBlocking blocking{};
     int per_block = tuning.chunks_per_block;
-    if (per_block < 1 || per_block > kMaxWavesPerBlock) {
-        per_block = kDefaultChunksPerBlock;
-        if (shape == kSlotOrderWalk) {
-            // measured on long timed regions: one 14-wavefront workgroup a row against two of 7:
-            // 4096 x 7168: 83.7 -> 81.7 us, 8192 x 6144: 145.7 -> 139.7 us (2-wavefront workgroups: 91 us).
-            // The same holds for a fresh dispatch, whose grid is sized for every choice being valid
-            // (host-visible, cold sources, 4096 x 7168: 125.0 -> 118.6 us; no difference with
-            // alignment 128 or with cache-resident sources).
-            const int most = kMaxWavesPerBlock;
-            const int pieces = (chunks + most - 1) / most;
-            per_block = (chunks + pieces - 1) / pieces;
-        } else if (shape == kRowCopyWalk) {
-            per_block = 1;
-        }
-    }
+    if (per_block < 1 || per_block > kMaxWavesPerBlock)
+        per_block = shape == kRowCopyWalk ? 1 : kDefaultChunksPerBlock;
     if (per_block > chunks)
         per_block = chunks;
     blocking.chunks_per_block = static_cast<unsigned>(per_block);
@@ -238,6 +231,12 @@ inline RowBlocking pick_row_blocking(int chunks, WalkShape shape, const Tuning& 
     }
     blocking.rows_per_block = static_cast<unsigned>(rows);
     return blocking;
+}
+
+// List entries a workgroup of the slot-order walk takes when a row has up to four pieces (longer
+// rows take a workgroup each, one wavefront a piece).
+inline int default_walk_rows(int pieces) {
+    return pieces >= 4 ? 1 : 4 / pieces;
 }
 
 inline int validate_cu_budget(int num_cus, const Topology& topology) {

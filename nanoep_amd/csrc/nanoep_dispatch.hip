@@ -150,202 +150,206 @@ __global__ void __launch_bounds__(1024) dispatch_rows_kernel(const u32x4* __rest
     }
 }
 
-// The slot-order walk, stripped to what its wavefronts need: a wavefront lives about a microsecond,
-// most of it waiting in a chain of scalar work -> list entry -> source load -> store, so every
-// scalar instruction and branch ahead of the source load is throughput (ten more scalar
-// instructions and three taken branches there measured +6 % on the whole kernel).  kZeroFill is
-// false when the launch has no gap rows to clear: the copy path then carries none of that
-// bookkeeping.  kWholeRows is the launch with one workgroup a list entry and one wavefront a piece
-// of the row (rows of 5 to 16 pieces, no side workgroups): block index and wavefront index are
-// the entry and the piece, with no division and no taken branch on the way to the load.
-// kSpan is the number of consecutive 1 KiB chunks a wavefront moves (loads issued back to back,
-// then the stores).  One is best while the source fits the last-level cache; beyond that size the
-// single-chunk walk loses a quarter of its rate and two chunks a wavefront win it back.
-// kPrefetch: the list is cut into segments of about one window's entries, and the copy workgroups of
-// every segment are preceded by a few workgroups that read the window's source rows front to back
-// (kPrefetchLoads KiB a wavefront, the data dropped).  The window's first touches then reach HBM as
-// one sequential burst ahead of the segment's stores instead of one row at a time among them, and
-// the copy wavefronts find their rows in the XCD's L2.  No bytes are read twice from HBM; what it
-// costs is one more L2 read per source row.
+// Arguments of dispatch_walk_kernel.  The first words are what every copy wavefront needs on its
+// way to the source load: they sit together so that they arrive in one batch of scalar loads.
+struct WalkArgs {
+    const u32x4* x;             // [T][row_bytes / 16]
+    u32x4* recv_x;              // [C][row_bytes / 16]
+    const int64_t* slot_order;  // [entries]
+    uint32_t entries;
+    uint32_t source_limit;  // T*K
+    uint32_t out_rows;
+    uint32_t copy_per_xcd;  // workgroups of the walk one XCD takes
+    uint32_t row_bytes;
+    uint32_t topk_magic;  // fast divisor by K
+    uint32_t topk_shift;
+    uint32_t xcd_count;
+    uint32_t xcd_magic;  // fast divisor by the XCD count
+    uint32_t xcd_shift;
+    uint32_t rows_per_block;  // list entries a workgroup (rows of up to four pieces)
+    uint32_t weight_lane;     // 0: the first lane of a row moves the entry's weight; ~0: there are no weights
+    const float* weights;     // [T][K] or null
+    float* recv_weights;      // [C] or null
+    // window-wise prefetch
+    uint32_t segment_blocks;   // prefetch + copy workgroups of a segment
+    uint32_t segment_magic;    // fast divisor by segment_blocks
+    uint32_t segment_shift;
+    uint32_t prefetch_blocks;  // prefetch workgroups at the head of a segment
+    uint32_t window_vectors;   // 16-byte vectors of one window's source rows
+    uint32_t source_vectors;   // ... of all source rows
+    // entry count on the device
+    uint32_t share_magic;  // fast divisor by the copy workgroups of a segment
+    uint32_t share_shift;
+    uint32_t rows_magic;  // fast divisor by rows_per_block
+    uint32_t rows_shift;
+    const int64_t* live_count;
+    // gap rows
+    const int64_t* expert_counts;
+    const int64_t* expert_offsets;
+    uint32_t pad_blocks;
+    uint32_t pad_per_xcd;
+    uint32_t pad_per_expert;
+    uint32_t pad_groups_per_expert;
+    uint32_t row_vectors;
+};
+
+// What a workgroup of the walk's grid does when it has no copy work: every XCD's copy workgroups are
+// followed by its share of the workgroups that clear the alignment gaps, each wavefront one whole
+// gap row (and its weight): workgroup (e, g) owns gap candidates j = g * waves .. of expert e, row
+// offsets[e] + counts[e] + j while that is below offsets[e+1].
+__device__ __forceinline__ void walk_gap_rows(const WalkArgs& a, uint32_t xcd, uint32_t pad_index) {
+    const uint32_t pad_block = xcd * a.pad_per_xcd + pad_index;
+    if (pad_index >= a.pad_per_xcd || pad_block >= a.pad_blocks)
+        return;
+    const uint32_t waves = blockDim.x / kWave;
+    const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
+    const uint32_t lane = threadIdx.x % kWave;
+    const uint32_t expert = pad_block / a.pad_groups_per_expert;
+    const uint32_t group = pad_block - expert * a.pad_groups_per_expert;
+    const uint32_t j = group * waves + wave;
+    if (j >= a.pad_per_expert)
+        return;
+    const int64_t out_row = uniform_load(a.expert_offsets + expert) + uniform_load(a.expert_counts + expert) + j;
+    if (out_row < 0 || out_row >= uniform_load(a.expert_offsets + expert + 1) || out_row >= static_cast<int64_t>(a.out_rows))
+        return;
+    const u32x4 zero = {0u, 0u, 0u, 0u};
+    u32x4* dst = a.recv_x + out_row * a.row_vectors;
+    for (uint32_t vector = lane; vector < a.row_vectors; vector += kWave)
+        store_vec<true>(dst + vector, zero);
+    if (lane == 0 && a.recv_weights != nullptr)
+        a.recv_weights[out_row] = 0.0f;
+}
+
+// Window-wise source prefetch: the list is cut into segments of about one window's entries, and the
+// copy workgroups of every segment are preceded by a few workgroups that read the window's source
+// rows front to back (kPrefetchLoads KiB a wavefront, the data dropped).  The window's first touches
+// then reach HBM as one sequential burst ahead of the segment's stores instead of one row at a time
+// among them, and the copy wavefronts find their rows in the XCD's L2.  No bytes are read twice from
+// HBM; what it costs is one more L2 read per source row.
 constexpr int kPrefetchLoads = 4;
 
-template <bool kDeviceCount, bool kZeroFill, int kSpan, bool kWholeRows, bool kPrefetch>
-__global__ void __launch_bounds__(1024) dispatch_ordered_kernel(const u32x4* __restrict__ x,              // [T][vectors]
-                                                                const float* __restrict__ weights,       // [T][K] or null
-                                                                const int64_t* __restrict__ slot_order,  // [entries]
-                                                                const int64_t* __restrict__ live_count,  // device entry count (kDeviceCount)
-                                                                const int64_t* __restrict__ expert_counts,
-                                                                const int64_t* __restrict__ expert_offsets,
-                                                                u32x4* __restrict__ recv_x,        // [C][vectors]
-                                                                float* __restrict__ recv_weights,  // [C] or null
-                                                                uint32_t entries,
-                                                                uint32_t source_limit,  // T*K
-                                                                uint32_t out_rows,
-                                                                uint32_t copy_blocks,
-                                                                uint32_t copy_per_xcd,
-                                                                uint32_t pad_blocks,
-                                                                uint32_t pad_per_xcd,
-                                                                uint32_t pad_per_expert,
-                                                                uint32_t pad_groups_per_expert,
-                                                                uint32_t parts,
-                                                                uint32_t parts_magic,
-                                                                uint32_t parts_shift,
-                                                                uint32_t chunks_per_block,  // == blockDim.y
-                                                                uint32_t rows_per_block,    // == blockDim.z
-                                                                uint32_t vectors,
-                                                                uint32_t chunks,      // pieces of kSpan chunks in a row
-                                                                uint32_t topk_magic,  // fast divisor by K
-                                                                uint32_t topk_shift,
-                                                                uint32_t rows_magic,  // fast divisor by rows_per_block
-                                                                uint32_t rows_shift,
-                                                                uint32_t payload_blocks,  // blocks behind them, if any, move the weights
-                                                                uint32_t segment_blocks,     // kPrefetch: prefetch + copy workgroups of a segment
-                                                                uint32_t segment_magic,      // fast divisor by segment_blocks
-                                                                uint32_t segment_shift,
-                                                                uint32_t prefetch_blocks,    // prefetch workgroups at the head of a segment
-                                                                uint32_t share_magic,        // fast divisor by the copy workgroups of a segment
-                                                                uint32_t share_shift,
-                                                                uint32_t window_vectors,     // 16-byte vectors of one window's source rows
-                                                                uint32_t source_vectors,     // ... of all source rows
-                                                                XcdMap xcds) {
-    NANOEP_FETCH_ARGS_4(x, weights, recv_x, recv_weights);
-    NANOEP_FETCH_ARGS_4(slot_order, entries, source_limit, out_rows);
-    NANOEP_FETCH_ARGS_4(copy_blocks, copy_per_xcd, parts, parts_magic);
-    NANOEP_FETCH_ARGS_4(parts_shift, chunks_per_block, rows_per_block, vectors);
-    NANOEP_FETCH_ARGS_4(chunks, topk_magic, topk_shift, live_count);
-    NANOEP_FETCH_ARGS_4(xcds.count, xcds.magic, xcds.shift, payload_blocks);
-    // workgroups per XCD the grid holds for the copy work: with the entry count on the device the live
-    // list may be shorter (the rest of the grid leaves at once) or longer (workgroups then take more
-    // than one turn, `grid_copy_per_xcd` list positions apart) than what the grid was sized for
-    const uint32_t grid_copy_per_xcd = copy_per_xcd;
-    if (kDeviceCount) {
-        // The list length was not known when the grid was sized: the walk covers the entries in use,
-        // so that the per-XCD ranges split the real work and not an unused tail.
-        // A word that cannot be a count (the layout did not run) walks nothing.
-        const int64_t live = uniform_load(live_count);
-        entries = live >= 0 && live <= static_cast<int64_t>(source_limit) ? static_cast<uint32_t>(live) : 0u;
-        // (one workgroup a list entry: no division by a runtime number on every wavefront's way to its load)
-        if (kWholeRows)
-            copy_blocks = entries;
-        else
-            copy_blocks = fast_divide(entries + rows_per_block - 1, rows_magic, rows_shift) * parts;
-        // with prefetch: whole segments of the size the host chose (from the count it expected), each
-        // with its prefetch workgroups in front
-        const uint32_t walk_blocks =
-            kPrefetch ? fast_divide(copy_blocks + (segment_blocks - prefetch_blocks) - 1, share_magic, share_shift) * segment_blocks
-                      : copy_blocks;
-        copy_per_xcd = fast_divide(walk_blocks + xcds.count - 1, xcds.magic, xcds.shift);
-    }
-    if (!kWholeRows && blockIdx.x >= payload_blocks) {
-        // The weights of the assignments, one lane per list entry, in workgroups of their own at the
-        // end of the grid.  The host asks for them when a row is one or two chunks: hung onto the
-        // row's first payload wavefront the weight is a second round trip in every (second) wavefront
-        // (131072 x 512 top-8: 77.5 -> 74.5 us).  With longer rows the first wavefronts are few and
-        // carry it at no measurable cost, while these extra workgroups cost 0.1 ns per assignment
-        // (4096 x 7168: +1 us, 32768 x 7168: +25 us of 700).
-        const uint32_t wave = threadIdx.z * chunks_per_block + threadIdx.y;
-        const uint32_t lanes = (gridDim.x - payload_blocks) * (chunks_per_block * rows_per_block) * kWave;
-        for (uint32_t flat = ((blockIdx.x - payload_blocks) * (chunks_per_block * rows_per_block) + wave) * kWave + threadIdx.x;
-             flat < entries; flat += lanes) {
-            const int64_t entry = slot_order[flat];
-            const uint32_t source = static_cast<uint32_t>(entry);
-            const uint32_t out_row = static_cast<uint32_t>(static_cast<uint64_t>(entry) >> 32);
-            if (entry >= 0 && source < source_limit && out_row < out_rows)
-                recv_weights[out_row] = weights[source];
-        }
-        return;
-    }
-    const uint32_t index_in_xcd = fast_divide(blockIdx.x, xcds.magic, xcds.shift);
-    const uint32_t xcd = blockIdx.x - index_in_xcd * xcds.count;
-    // the XCD's workgroups up to `copy_turns` copy, the ones behind them clear gap rows
-    const uint32_t copy_turns = kDeviceCount && copy_per_xcd > grid_copy_per_xcd ? grid_copy_per_xcd : copy_per_xcd;
-    if (kZeroFill && index_in_xcd >= copy_turns) {
-        const uint32_t pad_index = index_in_xcd - copy_turns;
-        const uint32_t pad_block = xcd * pad_per_xcd + pad_index;
-        if (pad_index < pad_per_xcd && pad_block < pad_blocks)
-            zero_fill_gap_rows(pad_block, pad_per_expert, pad_groups_per_expert, chunks_per_block, rows_per_block,
-                               expert_counts, expert_offsets, recv_x, recv_weights, out_rows, static_cast<int>(vectors));
-        return;
-    }
-    if (index_in_xcd >= copy_turns)
-        return;
-    // one turn, except where a device-side count found more entries than the grid was sized for
-    for (uint32_t at = index_in_xcd; at < copy_per_xcd; at += grid_copy_per_xcd) {
-        uint32_t block = xcd * copy_per_xcd + at;
-        if (kPrefetch) {
-            const uint32_t segment = fast_divide(block, segment_magic, segment_shift);
-            const uint32_t within = block - segment * segment_blocks;
-            if (within < prefetch_blocks) {
-                const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.z * chunks_per_block + threadIdx.y);
-                const uint32_t waves = chunks_per_block * rows_per_block;
-                const uint64_t window_first = static_cast<uint64_t>(segment) * window_vectors;
-                uint64_t window_end = window_first + window_vectors;
-                if (window_end > source_vectors)
-                    window_end = source_vectors;
-                const uint64_t first = window_first + static_cast<uint64_t>(within * waves + wave) * (kPrefetchLoads * kWave);
-                if (first < window_end) {
-                    u32x4 fetched[kPrefetchLoads];
+// One workgroup's turn at the slot-order walk: `block` is its position in the walk (with prefetch:
+// among the prefetch and copy workgroups of all segments).
+template <int kPieces, int kSpan, bool kPrefetch>
+__device__ __forceinline__ void walk_copy(const WalkArgs& a, uint32_t entries, uint32_t block) {
+    if (kPrefetch) {
+        const uint32_t segment = fast_divide(block, a.segment_magic, a.segment_shift);
+        const uint32_t within = block - segment * a.segment_blocks;
+        if (within < a.prefetch_blocks) {
+            const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
+            const uint32_t waves = blockDim.x / kWave;
+            const uint64_t window_first = static_cast<uint64_t>(segment) * a.window_vectors;
+            uint64_t window_end = window_first + a.window_vectors;
+            if (window_end > a.source_vectors)
+                window_end = a.source_vectors;
+            const uint64_t first = window_first + static_cast<uint64_t>(within * waves + wave) * (kPrefetchLoads * kWave);
+            if (first < window_end) {
+                u32x4 fetched[kPrefetchLoads];
 #pragma unroll
-                    for (int u = 0; u < kPrefetchLoads; ++u) {
-                        const uint64_t from = first + u * kWave + threadIdx.x;
-                        fetched[u] = x[from < window_end ? from : window_first];
-                    }
-#pragma unroll
-                    for (int u = 0; u < kPrefetchLoads; ++u)
-                        asm volatile("" ::"v"(fetched[u].x), "v"(fetched[u].y), "v"(fetched[u].z), "v"(fetched[u].w));
+                for (int u = 0; u < kPrefetchLoads; ++u) {
+                    const uint64_t from = first + u * kWave + threadIdx.x % kWave;
+                    fetched[u] = a.x[from < window_end ? from : window_first];
                 }
-                if (!kDeviceCount)
-                    break;
-                continue;
+#pragma unroll
+                for (int u = 0; u < kPrefetchLoads; ++u)
+                    asm volatile("" ::"v"(fetched[u].x), "v"(fetched[u].y), "v"(fetched[u].z), "v"(fetched[u].w));
             }
-            block = segment * (segment_blocks - prefetch_blocks) + (within - prefetch_blocks);
+            return;
         }
-        uint32_t candidate, chunk;
-        if (kWholeRows) {
-            // one workgroup a row, as many wavefronts as the row has pieces: the block is the list entry
-            if (block >= entries)
-                break;
-            candidate = block;
-            chunk = __builtin_amdgcn_readfirstlane(threadIdx.y);
-        } else {
-            if (block >= copy_blocks)
-                break;
-            const uint32_t group = fast_divide(block, parts_magic, parts_shift);
-            const uint32_t part = block - group * parts;
-            candidate = group * rows_per_block + __builtin_amdgcn_readfirstlane(threadIdx.z);
-            chunk = part * chunks_per_block + __builtin_amdgcn_readfirstlane(threadIdx.y);
-        }
-        if (kWholeRows || (candidate < entries && chunk < chunks)) {
-            const int64_t entry = uniform_load(slot_order + candidate);
-            const uint32_t source = static_cast<uint32_t>(entry);
-            const uint32_t out_row = static_cast<uint32_t>(static_cast<uint64_t>(entry) >> 32);
-            if (entry >= 0 && source < source_limit && out_row < out_rows) {
-                const uint32_t token = fast_divide(source, topk_magic, topk_shift);
-                const uint32_t vector = chunk * (kSpan * kWave) + threadIdx.x;
-                // no workgroups behind the payload: the row's first wavefront moves its weight, fetched through
-                // the scalar path while the payload load is in flight
-                const bool carries_weight = chunk == 0 && recv_weights != nullptr && (kWholeRows || payload_blocks == gridDim.x);
-                float weight = 0.0f;
-                if (carries_weight)
-                    weight = uniform_load(weights + source);
-                u32x4 data[kSpan];
+        block = segment * (a.segment_blocks - a.prefetch_blocks) + (within - a.prefetch_blocks);
+    }
+    // the list entry of this wavefront and the first 16-byte vector of the row its lanes move
+    uint32_t candidate, lane_vector;
+    if (kPieces == 0) {
+        candidate = block;
+        lane_vector = kSpan == 1 ? threadIdx.x : (threadIdx.x / kWave) * (kSpan * kWave) + threadIdx.x % kWave;
+    } else {
+        const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
+        const uint32_t row = wave / kPieces;
+        candidate = block * a.rows_per_block + row;
+        lane_vector = kSpan == 1 ? threadIdx.x - row * (kPieces * kWave)
+                                 : (wave - row * kPieces) * (kSpan * kWave) + threadIdx.x % kWave;
+    }
+    if (candidate >= entries)
+        return;
+    const int64_t entry = uniform_load_at(a.slot_order, candidate);
+    const uint32_t source = static_cast<uint32_t>(entry);
+    const uint32_t out_row = static_cast<uint32_t>(static_cast<uint64_t>(entry) >> 32);
+    // (a negative entry has an impossible row; the empty statement keeps the two tests two
+    // compare-and-branch pairs: merged into one condition they cost three more scalar instructions)
+    if (out_row >= a.out_rows)
+        return;
+    asm volatile("");
+    if (source >= a.source_limit)
+        return;
+    const uint32_t token = fast_divide(source, a.topk_magic, a.topk_shift);
+    const char* from = reinterpret_cast<const char*>(a.x) + static_cast<uint64_t>(token) * a.row_bytes;
+    char* to = reinterpret_cast<char*>(a.recv_x) + static_cast<uint64_t>(out_row) * a.row_bytes;
+    const uint32_t lane_bytes = lane_vector * 16u;
+    u32x4 data[kSpan];
 #pragma unroll
-                for (int s = 0; s < kSpan; ++s) {
-                    const uint32_t from = vector + s * kWave;
-                    data[s] = x[static_cast<uint64_t>(token) * vectors + (from < vectors ? from : 0u)];
-                }
+    for (int s = 0; s < kSpan; ++s) {
+        const uint32_t at_bytes = lane_bytes + s * (kWave * 16u);
+        // lanes past the end of the row re-read its start instead of branching around the load
+        data[s] = *reinterpret_cast<const u32x4*>(from + (at_bytes < a.row_bytes ? at_bytes : 0u));
+    }
+    // the entry's weight rides with the first lane of its row while the payload is in flight
+    // (weight_lane is no lane at all when there are no weights to move here)
+    if (lane_vector == a.weight_lane)
+        a.recv_weights[out_row] = a.weights[source];
 #pragma unroll
-                for (int s = 0; s < kSpan; ++s) {
-                    const uint32_t to = vector + s * kWave;
-                    if (to < vectors)
-                        store_vec<true>(recv_x + static_cast<uint64_t>(out_row) * vectors + to, data[s]);
-                }
-                if (carries_weight && threadIdx.x == 0)
-                    recv_weights[out_row] = weight;
-            }
+    for (int s = 0; s < kSpan; ++s) {
+        const uint32_t at_bytes = lane_bytes + s * (kWave * 16u);
+        if (at_bytes < a.row_bytes)
+            store_vec<true>(reinterpret_cast<u32x4*>(to + at_bytes), data[s]);
+    }
+}
+
+// The slot-order walk.  Its wavefronts are short (a list entry, a source load, a store) and there are
+// hundreds of thousands of them, so the scalar instructions each one spends on finding its work are a
+// throughput limit of their own (a compute unit issues one a cycle): everything on the way to the
+// load is kept to the minimum, and the gap rows live behind the one test that ends a wavefront with
+// no copy work.
+//   kPieces 0 : one workgroup a list entry, one wavefront a piece of the row (rows of 5 to 16 pieces)
+//   kPieces 1..4 : rows of that many pieces, rows_per_block entries a workgroup
+//   kSpan   : 1 KiB chunks a wavefront moves (a piece)
+template <int kPieces, int kSpan, bool kDeviceCount, bool kPrefetch>
+__global__ void __launch_bounds__(1024) dispatch_walk_kernel(const WalkArgs a) {
+    NANOEP_FETCH_ARGS_4(a.x, a.recv_x, a.slot_order, a.entries);
+    NANOEP_FETCH_ARGS_4(a.source_limit, a.out_rows, a.copy_per_xcd, a.row_bytes);
+    NANOEP_FETCH_ARGS_4(a.topk_magic, a.topk_shift, a.xcd_count, a.xcd_magic);
+    NANOEP_FETCH_ARGS_4(a.xcd_shift, a.rows_per_block, a.weight_lane, a.weights);
+    NANOEP_FETCH_ARGS_2(a.recv_weights, a.weights);
+    if (kPrefetch)
+        NANOEP_FETCH_ARGS_4(a.segment_blocks, a.segment_magic, a.segment_shift, a.prefetch_blocks);
+    const uint32_t index_in_xcd = fast_divide(blockIdx.x, a.xcd_magic, a.xcd_shift);
+    const uint32_t xcd = blockIdx.x - index_in_xcd * a.xcd_count;
+    if (!kDeviceCount) {
+        if (index_in_xcd >= a.copy_per_xcd) {
+            walk_gap_rows(a, xcd, index_in_xcd - a.copy_per_xcd);
+            __builtin_amdgcn_endpgm();
         }
-        if (!kDeviceCount)
-            break;
+        walk_copy<kPieces, kSpan, kPrefetch>(a, a.entries, xcd * a.copy_per_xcd + index_in_xcd);
+        return;
+    }
+    // The entry count is on the device: the live list may be shorter than what the grid was sized for
+    // (the rest of the grid leaves at once) or longer (workgroups then take more than one turn, a
+    // grid's worth of list positions apart).  A word that cannot be a count (the layout did not run)
+    // walks nothing.
+    const int64_t live = uniform_load(a.live_count);
+    const uint32_t entries = live >= 0 && live <= static_cast<int64_t>(a.source_limit) ? static_cast<uint32_t>(live) : 0u;
+    const uint32_t copy_blocks = kPieces == 0 ? entries : fast_divide(entries + a.rows_per_block - 1, a.rows_magic, a.rows_shift);
+    // with prefetch: whole segments of the size the host chose (from the count it expected)
+    const uint32_t walk_blocks =
+        kPrefetch ? fast_divide(copy_blocks + (a.segment_blocks - a.prefetch_blocks) - 1, a.share_magic, a.share_shift) * a.segment_blocks
+                  : copy_blocks;
+    const uint32_t copy_per_xcd = fast_divide(walk_blocks + a.xcd_count - 1, a.xcd_magic, a.xcd_shift);
+    const uint32_t copy_turns = copy_per_xcd > a.copy_per_xcd ? a.copy_per_xcd : copy_per_xcd;
+    if (index_in_xcd < copy_turns) {
+        for (uint32_t at = index_in_xcd; at < copy_per_xcd; at += a.copy_per_xcd)
+            walk_copy<kPieces, kSpan, kPrefetch>(a, entries, xcd * copy_per_xcd + at);
+    } else {
+        walk_gap_rows(a, xcd, index_in_xcd - copy_turns);
     }
 }
 
@@ -455,152 +459,181 @@ int nanoep_dispatch(const void* x, const float* weights, const int32_t* recv_met
 
     // full list length without its trailing count word
     const int64_t order_bound = nanoep_slot_order_entries(num_tokens, num_topk, num_local_experts) - 1;
-    // The walk is used whenever the handle carries the list.  With cache-resident sources and fewer
-    // than eight token blocks the token-order walk is up to 15 % faster, but with cold sources it is
-    // 25-60 % slower at every size, so the list decides.
-    const int order_switch = tuning.dispatch_order;  // 0 forces the token-order walk
-    const bool ordered = expand && slot_order != nullptr && order_bound > 0 && order_switch != 0;
-    if (ordered && (slot_order_entries > order_bound || num_tokens * num_topk >= (int64_t{1} << 31)))
-        return NANOEP_ERR_INVALID_ARGUMENT;
-    // A negative entry count defers to the count word the layout stored behind the list.  -1 sizes the
-    // grid for the most entries the list can hold (T * K), -g for about g of them: workgroups beyond
-    // the live count leave at once, and where the live count is above g workgroups take several turns.
-    const int64_t* live_count = ordered && slot_order_entries < 0 ? slot_order + order_bound : nullptr;
-    if (live_count != nullptr) {
-        const int64_t most = num_tokens * num_topk;
-        const int64_t expected = slot_order_entries == -1 ? most : -slot_order_entries;
-        slot_order_entries = expected < most ? expected : most;
-    }
-
     const int vectors = hidden / 8;
-    int chunks = (vectors + kWave - 1) / kWave;
-    // Chunks per wavefront of the slot-order walk: two once the source outgrows the last-level cache,
-    // and for rows of two chunks, which then take one wavefront (16384 x 1024 top-4: 39.8 -> 35.6 us;
-    // at four chunks the gain is within +3 / -1 %).  NANOEP_DISPATCH_SPAN=1|2 overrides.  `chunks`
-    // then counts pieces of that many chunks.
-    const int row_chunks = chunks;
-    int span = 1;
-    if (ordered) {
-        const bool short_rows = chunks == 2;
-        span = short_rows || static_cast<int64_t>(num_tokens) * hidden * 2 > kLastLevelCacheBytes ? 2 : 1;
-        const int forced_span = tuning.dispatch_span;
-        if (forced_span == 1 || forced_span == 2)
-            span = forced_span;
-        chunks = (chunks + span - 1) / span;
-    }
-    const WalkShape walk = ordered ? kSlotOrderWalk : expand ? kTokenOrderWalk : kRowCopyWalk;
-    const RowBlocking blocking = pick_row_blocking(chunks, walk, tuning);
-    const int64_t waves = static_cast<int64_t>(blocking.chunks_per_block) * blocking.rows_per_block;
-    const int64_t copy_candidates = ordered ? slot_order_entries : expand ? num_tokens * num_topk : num_tokens;
-    const int64_t copy_blocks = (copy_candidates + blocking.rows_per_block - 1) / blocking.rows_per_block * blocking.parts;
+    const int row_chunks = (vectors + kWave - 1) / kWave;
+    // The slot-order walk is used whenever the handle carries the list.  With cache-resident sources and
+    // fewer than eight token blocks the token-order walk is up to 15 % faster, but with cold sources
+    // it is 25-60 % slower at every size, so the list decides.  A wavefront moves one 1 KiB chunk; two
+    // once the source outgrows the last-level cache (the single-chunk walk then loses a quarter of
+    // its rate) and as many as it takes for a row to fit the 16 wavefronts of a workgroup
+    // (NANOEP_DISPATCH_SPAN=1|2|4 asks for a number).  The walk addresses the list with 32-bit byte
+    // offsets: lists of 2^29 entries and more, and rows beyond 64 KiB, take the token-order walk.
+    int span = static_cast<int64_t>(num_tokens) * hidden * 2 > kLastLevelCacheBytes ? 2 : 1;
+    if (tuning.dispatch_span == 1 || tuning.dispatch_span == 2 || tuning.dispatch_span == 4)
+        span = tuning.dispatch_span;
+    while (span < 4 && (row_chunks + span - 1) / span > kMaxWavesPerBlock)
+        span *= 2;
+    const int pieces = (row_chunks + span - 1) / span;
+    const bool ordered = expand && slot_order != nullptr && order_bound > 0 && tuning.dispatch_order != 0 &&
+                         pieces <= kMaxWavesPerBlock && num_tokens * num_topk < (int64_t{1} << 29);
+    if (ordered && slot_order_entries > order_bound)
+        return NANOEP_ERR_INVALID_ARGUMENT;
+    if (num_tokens * num_topk >= (int64_t{1} << 31) || static_cast<int64_t>(num_tokens) * vectors >= (int64_t{1} << 32))
+        return NANOEP_ERR_INVALID_ARGUMENT;
+    auto stream = static_cast<hipStream_t>(stream_handle);
     // No expert's gap exceeds alignment-1 rows, and all gaps together stay below C.
     const int64_t pad_per_expert = !pad ? 0 : (alignment - 1 < expanded_capacity ? alignment - 1 : expanded_capacity);
+
+    if (ordered) {
+        // A negative entry count defers to the count word the layout stored behind the list.  -1 sizes the
+        // grid for the most entries the list can hold (T * K), -g for about g of them: workgroups beyond
+        // the live count leave at once, and where the live count is above g workgroups take several turns.
+        const int64_t* live_count = slot_order_entries < 0 ? slot_order + order_bound : nullptr;
+        if (live_count != nullptr) {
+            const int64_t most = num_tokens * num_topk;
+            const int64_t expected = slot_order_entries == -1 ? most : -slot_order_entries;
+            slot_order_entries = expected < most ? expected : most;
+        }
+        // Rows of up to four pieces share a workgroup (kPieces of the kernel); longer rows take one each.
+        const int kernel_pieces = pieces <= 4 ? pieces : 0;
+        int rows_per_block = 1;
+        if (kernel_pieces != 0) {
+            rows_per_block = tuning.rows_per_block;
+            if (rows_per_block < 1 || rows_per_block * pieces > kMaxWavesPerBlock)
+                rows_per_block = default_walk_rows(pieces);
+        }
+        const int64_t waves = static_cast<int64_t>(pieces) * rows_per_block;
+        const int64_t copy_blocks = (slot_order_entries + rows_per_block - 1) / rows_per_block;
+        const int64_t pad_groups_per_expert = (pad_per_expert + waves - 1) / waves;
+        const int64_t pad_blocks = num_local_experts * pad_groups_per_expert;
+        // Prefetch workgroups ahead of every window's share of the list.  The list's windows hold
+        // nearly the same number of entries each, so equal shares of the list follow them closely.
+        // With sources that come from HBM it gains 5 to 22 % (rows of 512 elements most, 7168 least),
+        // with sources that sit in the last-level cache it costs 0 to 4 %: on unless
+        // NANOEP_DISPATCH_PREFETCH=0.
+        const int window_tokens = nanoep_layout_block_tokens(num_tokens, num_local_experts, hidden);
+        const bool prefetch = window_tokens > 0 && copy_blocks > 0 && tuning.dispatch_prefetch != 0;
+        int64_t segment_copy_blocks = 0, segment_prefetch_blocks = 0, segments = 0;
+        if (prefetch) {
+            const int64_t windows = (num_tokens + window_tokens - 1) / window_tokens;
+            const int64_t segment_entries = (slot_order_entries + windows - 1) / windows;
+            segment_copy_blocks = (segment_entries + rows_per_block - 1) / rows_per_block;
+            segments = (copy_blocks + segment_copy_blocks - 1) / segment_copy_blocks;
+            const int64_t window_kib = (static_cast<int64_t>(window_tokens) * vectors + kWave - 1) / kWave;
+            segment_prefetch_blocks = (window_kib + waves * kPrefetchLoads - 1) / (waves * kPrefetchLoads);
+        }
+        const int64_t walk_blocks = prefetch ? segments * (segment_copy_blocks + segment_prefetch_blocks) : copy_blocks;
+        if (walk_blocks + pad_blocks >= (int64_t{1} << 31) - 2 * int64_t{xcds.count})
+            return NANOEP_ERR_INVALID_ARGUMENT;
+        const uint32_t copy_per_xcd = static_cast<uint32_t>((walk_blocks + xcds.count - 1) / xcds.count);
+        const uint32_t pad_per_xcd = static_cast<uint32_t>((pad_blocks + xcds.count - 1) / xcds.count);
+        const FastDivisor topk_divisor = make_fast_divisor(static_cast<uint32_t>(num_topk));
+        const FastDivisor rows_divisor = make_fast_divisor(static_cast<uint32_t>(rows_per_block));
+        const FastDivisor share_divisor = make_fast_divisor(static_cast<uint32_t>(prefetch ? segment_copy_blocks : 1));
+        const FastDivisor segment_divisor =
+            make_fast_divisor(static_cast<uint32_t>(prefetch ? segment_copy_blocks + segment_prefetch_blocks : 1));
+        WalkArgs a{};
+        a.x = static_cast<const u32x4*>(x);
+        a.recv_x = static_cast<u32x4*>(recv_x);
+        a.slot_order = slot_order;
+        a.entries = static_cast<uint32_t>(slot_order_entries);
+        a.source_limit = static_cast<uint32_t>(num_tokens * num_topk);
+        a.out_rows = static_cast<uint32_t>(out_rows);
+        a.copy_per_xcd = copy_per_xcd;
+        a.row_bytes = static_cast<uint32_t>(vectors) * 16u;
+        a.topk_magic = topk_divisor.magic;
+        a.topk_shift = topk_divisor.shift;
+        a.xcd_count = xcds.count;
+        a.xcd_magic = xcds.magic;
+        a.xcd_shift = xcds.shift;
+        a.rows_per_block = static_cast<uint32_t>(rows_per_block);
+        a.weight_lane = recv_weights == nullptr ? 0xffffffffu : 0u;
+        a.weights = weights;
+        a.recv_weights = recv_weights;
+        a.segment_blocks = static_cast<uint32_t>(segment_copy_blocks + segment_prefetch_blocks);
+        a.segment_magic = segment_divisor.magic;
+        a.segment_shift = segment_divisor.shift;
+        a.prefetch_blocks = static_cast<uint32_t>(segment_prefetch_blocks);
+        a.window_vectors = static_cast<uint32_t>(static_cast<int64_t>(window_tokens) * vectors);
+        a.source_vectors = static_cast<uint32_t>(num_tokens * vectors);
+        a.share_magic = share_divisor.magic;
+        a.share_shift = share_divisor.shift;
+        a.rows_magic = rows_divisor.magic;
+        a.rows_shift = rows_divisor.shift;
+        a.live_count = live_count;
+        a.expert_counts = expert_counts;
+        a.expert_offsets = expert_offsets;
+        a.pad_blocks = static_cast<uint32_t>(pad_blocks);
+        a.pad_per_xcd = pad_per_xcd;
+        a.pad_per_expert = static_cast<uint32_t>(pad_per_expert);
+        a.pad_groups_per_expert = static_cast<uint32_t>(pad_groups_per_expert > 0 ? pad_groups_per_expert : 1);
+        a.row_vectors = static_cast<uint32_t>(vectors);
+        const dim3 grid(static_cast<unsigned>((int64_t{copy_per_xcd} + pad_per_xcd) * xcds.count));
+        const dim3 threads(static_cast<unsigned>(waves * kWave));
+        const bool device_count = live_count != nullptr;
+#define NANOEP_LAUNCH_WALK(PIECES, SPAN)                                                       \
+    do {                                                                                       \
+        if (device_count && prefetch)                                                          \
+            dispatch_walk_kernel<PIECES, SPAN, true, true><<<grid, threads, 0, stream>>>(a);   \
+        else if (device_count)                                                                 \
+            dispatch_walk_kernel<PIECES, SPAN, true, false><<<grid, threads, 0, stream>>>(a);  \
+        else if (prefetch)                                                                     \
+            dispatch_walk_kernel<PIECES, SPAN, false, true><<<grid, threads, 0, stream>>>(a);  \
+        else                                                                                   \
+            dispatch_walk_kernel<PIECES, SPAN, false, false><<<grid, threads, 0, stream>>>(a); \
+    } while (0)
+#define NANOEP_LAUNCH_WALK_PIECES(PIECES)  \
+    do {                                   \
+        if (span == 4)                     \
+            NANOEP_LAUNCH_WALK(PIECES, 4); \
+        else if (span == 2)                \
+            NANOEP_LAUNCH_WALK(PIECES, 2); \
+        else                               \
+            NANOEP_LAUNCH_WALK(PIECES, 1); \
+    } while (0)
+        switch (kernel_pieces) {
+            case 1:
+                NANOEP_LAUNCH_WALK_PIECES(1);
+                break;
+            case 2:
+                NANOEP_LAUNCH_WALK_PIECES(2);
+                break;
+            case 3:
+                NANOEP_LAUNCH_WALK_PIECES(3);
+                break;
+            case 4:
+                NANOEP_LAUNCH_WALK_PIECES(4);
+                break;
+            default:
+                NANOEP_LAUNCH_WALK_PIECES(0);
+                break;
+        }
+#undef NANOEP_LAUNCH_WALK_PIECES
+#undef NANOEP_LAUNCH_WALK
+        NANOEP_HIP_TRY(hipGetLastError());
+        return NANOEP_OK;
+    }
+
+    // token-order walks and the compact row copy: workgroups of (64, chunks, rows)
+    const int chunks = row_chunks;
+    const RowBlocking blocking = pick_row_blocking(chunks, expand ? kTokenOrderWalk : kRowCopyWalk, tuning);
+    const int64_t waves = static_cast<int64_t>(blocking.chunks_per_block) * blocking.rows_per_block;
+    const int64_t copy_candidates = expand ? num_tokens * num_topk : num_tokens;
+    const int64_t copy_blocks = (copy_candidates + blocking.rows_per_block - 1) / blocking.rows_per_block * blocking.parts;
     const int64_t pad_groups_per_expert = (pad_per_expert + waves - 1) / waves;
     const int64_t pad_blocks = num_local_experts * pad_groups_per_expert;
-    if (copy_candidates >= (int64_t{1} << 31) || copy_blocks + pad_blocks >= (int64_t{1} << 31) - 2 * int64_t{xcds.count})
+    if (copy_blocks + pad_blocks >= (int64_t{1} << 31) - 2 * int64_t{xcds.count})
         return NANOEP_ERR_INVALID_ARGUMENT;
-    // Prefetch workgroups ahead of every window's share of the list.  The list's windows hold nearly the same number of entries each, so equal shares
-    // of the list follow them closely.
-    const int window_tokens = ordered ? nanoep_layout_block_tokens(num_tokens, num_local_experts, hidden) : 0;
-    // On by default for rows of two chunks (513 to 1024 elements), where it gains 7 to 19 % with sources
-    // that come from HBM and costs nothing with cache-resident ones.  For other row lengths it trades:
-    // rows of one chunk +21 % against -14 %, the 4096 x 4096 top-2 batch +7 % against -9 %, rows of 7168
-    // elements +0 to 2 % against -10 %; there it is the caller's choice (the DISPATCH_PREFETCH switch).
-    const bool prefetch = ordered && window_tokens > 0 && copy_blocks > 0 &&
-                          (tuning.dispatch_prefetch < 0 ? row_chunks == 2 : tuning.dispatch_prefetch > 0);
-    int64_t segment_copy_blocks = 0, segment_prefetch_blocks = 0, segments = 0;
-    if (prefetch) {
-        const int64_t windows = (num_tokens + window_tokens - 1) / window_tokens;
-        const int64_t segment_entries = (copy_candidates + windows - 1) / windows;
-        segment_copy_blocks = (segment_entries + blocking.rows_per_block - 1) / blocking.rows_per_block * blocking.parts;
-        segments = (copy_blocks + segment_copy_blocks - 1) / segment_copy_blocks;
-        const int64_t window_kib = (static_cast<int64_t>(window_tokens) * vectors + kWave - 1) / kWave;
-        segment_prefetch_blocks = (window_kib + waves * kPrefetchLoads - 1) / (waves * kPrefetchLoads);
-    }
-    const int64_t walk_blocks = prefetch ? segments * (segment_copy_blocks + segment_prefetch_blocks) : copy_blocks;
-    if (walk_blocks >= (int64_t{1} << 31) - 2 * int64_t{xcds.count} - pad_blocks ||
-        static_cast<int64_t>(num_tokens) * vectors >= (int64_t{1} << 32))
-        return NANOEP_ERR_INVALID_ARGUMENT;
-    const uint32_t copy_per_xcd = static_cast<uint32_t>((walk_blocks + xcds.count - 1) / xcds.count);
+    const uint32_t copy_per_xcd = static_cast<uint32_t>((copy_blocks + xcds.count - 1) / xcds.count);
     const uint32_t pad_per_xcd = static_cast<uint32_t>((pad_blocks + xcds.count - 1) / xcds.count);
     int topk_shift = -1;
     if ((num_topk & (num_topk - 1)) == 0)
         for (topk_shift = 0; (1 << topk_shift) < num_topk; ++topk_shift) {
         }
-
-    // slot-order walk over rows of one or two chunks: one lane per list entry moves the weights, in
-    // workgroups at the end of the grid (+3-4 %); longer rows carry the weight on their first wavefront
-    // (8192 x 2048 top-8 with alignment 128: 56.0 against 57.0 us).  NANOEP_DISPATCH_SIDE=0|1 overrides.
-    const int side_switch = tuning.dispatch_side;
-    const bool side_weights = ordered && recv_weights != nullptr && (side_switch < 0 ? row_chunks <= 2 : side_switch != 0);
-    const int64_t side_lanes = side_weights ? copy_candidates : 0;
-    const int64_t side_blocks = (side_lanes + kWave * waves - 1) / (kWave * waves);
-    const int64_t payload_blocks = (int64_t{copy_per_xcd} + pad_per_xcd) * xcds.count;
-    if (payload_blocks + side_blocks >= (int64_t{1} << 31))
-        return NANOEP_ERR_INVALID_ARGUMENT;
-    const dim3 grid(static_cast<unsigned>(payload_blocks + side_blocks));
+    const dim3 grid(static_cast<unsigned>((int64_t{copy_per_xcd} + pad_per_xcd) * xcds.count));
     const dim3 block(kWave, blocking.chunks_per_block, blocking.rows_per_block);
     const FastDivisor parts_divisor = make_fast_divisor(blocking.parts);
-    auto stream = static_cast<hipStream_t>(stream_handle);
-    if (ordered) {
-        const FastDivisor topk_divisor = make_fast_divisor(static_cast<uint32_t>(num_topk));
-        const FastDivisor rows_divisor = make_fast_divisor(blocking.rows_per_block);
-        const FastDivisor share_divisor = make_fast_divisor(static_cast<uint32_t>(prefetch ? segment_copy_blocks : 1));
-        const FastDivisor segment_divisor = make_fast_divisor(static_cast<uint32_t>(prefetch ? segment_copy_blocks + segment_prefetch_blocks : 1));
-#define NANOEP_LAUNCH_ORDERED_ROWS(DEVICE_COUNT, ZERO_FILL, SPAN, WHOLE_ROWS, PREFETCH)                               \
-    dispatch_ordered_kernel<DEVICE_COUNT, ZERO_FILL, SPAN, WHOLE_ROWS, PREFETCH><<<grid, block, 0, stream>>>(        \
-        static_cast<const u32x4*>(x), weights, slot_order, live_count, expert_counts, expert_offsets,                \
-        static_cast<u32x4*>(recv_x), recv_weights, static_cast<uint32_t>(copy_candidates),                           \
-        static_cast<uint32_t>(num_tokens * num_topk), static_cast<uint32_t>(out_rows),                               \
-        static_cast<uint32_t>(copy_blocks), copy_per_xcd, static_cast<uint32_t>(pad_blocks), pad_per_xcd,            \
-        static_cast<uint32_t>(pad_per_expert),                                                                       \
-        static_cast<uint32_t>(pad_groups_per_expert > 0 ? pad_groups_per_expert : 1), blocking.parts,                \
-        parts_divisor.magic, parts_divisor.shift, blocking.chunks_per_block, blocking.rows_per_block,                \
-        static_cast<uint32_t>(vectors), static_cast<uint32_t>(chunks), topk_divisor.magic, topk_divisor.shift,       \
-        rows_divisor.magic, rows_divisor.shift, static_cast<uint32_t>(payload_blocks),                               \
-        static_cast<uint32_t>(segment_copy_blocks + segment_prefetch_blocks), segment_divisor.magic,                 \
-        segment_divisor.shift, static_cast<uint32_t>(segment_prefetch_blocks),                                       \
-        share_divisor.magic, share_divisor.shift,                                                                    \
-        static_cast<uint32_t>(static_cast<int64_t>(window_tokens) * vectors),                                        \
-        static_cast<uint32_t>(num_tokens * vectors), xcds)
-#define NANOEP_LAUNCH_ORDERED_SPAN(DEVICE_COUNT, ZERO_FILL, SPAN)                                 \
-    do {                                                                                          \
-        if (whole_rows && prefetch)                                                               \
-            NANOEP_LAUNCH_ORDERED_ROWS(DEVICE_COUNT, ZERO_FILL, SPAN, true, true);                \
-        else if (whole_rows)                                                                      \
-            NANOEP_LAUNCH_ORDERED_ROWS(DEVICE_COUNT, ZERO_FILL, SPAN, true, false);               \
-        else if (prefetch)                                                                        \
-            NANOEP_LAUNCH_ORDERED_ROWS(DEVICE_COUNT, ZERO_FILL, SPAN, false, true);               \
-        else                                                                                      \
-            NANOEP_LAUNCH_ORDERED_ROWS(DEVICE_COUNT, ZERO_FILL, SPAN, false, false);              \
-    } while (0)
-#define NANOEP_LAUNCH_ORDERED(DEVICE_COUNT, ZERO_FILL)             \
-    do {                                                           \
-        if (span == 2)                                             \
-            NANOEP_LAUNCH_ORDERED_SPAN(DEVICE_COUNT, ZERO_FILL, 2); \
-        else                                                       \
-            NANOEP_LAUNCH_ORDERED_SPAN(DEVICE_COUNT, ZERO_FILL, 1); \
-    } while (0)
-        // a workgroup per list entry with a wavefront per piece of the row: the kernel then needs no
-        // division to find its entry and piece (4096 x 7168: 81.5 -> 80.4 us, with alignment 128
-        // 100.6 -> 96.9 us, 8192 x 5120: 123.1 -> 120.3 us).  Rows of four pieces are better off
-        // with the general path (8192 x 2048 with cache-resident sources: 37.6 against 38.3 us).
-        const int whole_rows_switch = tuning.dispatch_whole_rows;
-        const bool whole_rows = blocking.parts == 1 && blocking.rows_per_block == 1 &&
-                                blocking.chunks_per_block == static_cast<unsigned>(chunks) && side_blocks == 0 &&
-                                (whole_rows_switch < 0 ? chunks >= 5 : whole_rows_switch != 0);
-        if (live_count != nullptr && pad_blocks > 0)
-            NANOEP_LAUNCH_ORDERED(true, true);
-        else if (live_count != nullptr)
-            NANOEP_LAUNCH_ORDERED(true, false);
-        else if (pad_blocks > 0)
-            NANOEP_LAUNCH_ORDERED(false, true);
-        else
-            NANOEP_LAUNCH_ORDERED(false, false);
-#undef NANOEP_LAUNCH_ORDERED
-#undef NANOEP_LAUNCH_ORDERED_SPAN
-#undef NANOEP_LAUNCH_ORDERED_ROWS
-    } else if (!expand) {
+    if (!expand) {
         const int64_t blocks = (num_tokens + blocking.rows_per_block - 1) / blocking.rows_per_block * blocking.parts;
         // one lane per (token, k) for the ids and weights, when the caller wants either
         const int64_t row_side_lanes = recv_topk_idx != nullptr || recv_weights != nullptr ? num_tokens * num_topk : 0;

@@ -194,15 +194,15 @@ def slot_order_of(metadata, use_order=True):
 
 
 def dispatch(x, weights, metadata, counts, num_local_experts, alignment, expand, zero_padding, *, num_cus=0, poison=None,
-             use_table=True, use_order=True, order_count="exact", walk="forced", span=None, whole_rows=None, prefetch=None):
+             use_table=True, use_order=True, order_count="exact", walk="forced", span=None, rows=None, prefetch=None):
     """Returns (recv_x, recv_topk_idx | None, recv_weights | None) through nanoep_dispatch.
 
     walk="forced" sets the library's switch for the slot-order walk explicitly, walk="auto" leaves
-    the switch alone (the library then walks the list whenever it is given one).  span=1|2
+    the switch alone (the library then walks the list whenever it is given one).  span=1|2|4
     forces the number of chunks a wavefront of that walk moves (the library picks it by source size).
-    whole_rows=0|1 forces or forbids that walk's kernel variant for one workgroup a list entry (the
-    library takes it for rows of five pieces and more whose workgroup covers the row).  prefetch=0|1
-    forbids or asks for that walk's window-wise source prefetch.
+    rows=n asks for n list entries a workgroup of that walk (honoured for rows of up to four pieces while
+    the workgroup stays within 16 wavefronts).  prefetch=0|1 forbids or asks for that walk's window-wise
+    source prefetch.
     """
     recv_metadata, expert_counts, expert_offsets, dst_slots = metadata[0], metadata[1], metadata[2], metadata[3]
     received, capacity = counts[0], counts[1]
@@ -230,7 +230,7 @@ def dispatch(x, weights, metadata, counts, num_local_experts, alignment, expand,
     else:
         order_entries = -1 if order_count == "device" else -int(order_count[1])
     switches = {"DISPATCH_ORDER": 1 if walk == "forced" else None, "DISPATCH_SPAN": span,
-                "DISPATCH_WHOLE_ROWS": None if whole_rows is None else int(whole_rows),
+                "ROWS_PER_BLOCK": rows,
                 "DISPATCH_PREFETCH": None if prefetch is None else int(prefetch)}
     with forced_tuning(switches):
         status = lib().nanoep_dispatch(

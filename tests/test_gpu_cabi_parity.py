@@ -100,23 +100,23 @@ def run_dispatch_combine(device, idx, hidden, experts, alignment, expand, zero_p
             )
             assert torch.equal(wide_x.view(torch.int16), got_x.view(torch.int16))
             assert wide_w is None or torch.equal(wide_w.view(torch.int32), got_w.view(torch.int32))
-        # ... so must both kernel variants of that walk (one workgroup a list entry without any
-        # division, and the general one), with either entry count and either width
-        for whole_rows in (0, 1):
-            for order_count, span in (("exact", 1), ("device", 1), ("exact", 2)):
+        # ... so must that walk with other numbers of list entries a workgroup and of chunks a wavefront
+        # (rows of up to four pieces share workgroups, longer ones take one each), with either entry count
+        for rows in (1, 2, 4, 16):
+            for order_count, span in (("exact", 1), ("device", 1), ("exact", 2), ("device", 4)):
                 rows_x, _, rows_w = cabi.dispatch(
                     x.to(device), None if w is None else w.to(device), metadata, counts, experts, alignment, expand, zero_padding,
-                    num_cus=num_cus, poison=POISON, order_count=order_count, span=span, whole_rows=whole_rows,
+                    num_cus=num_cus, poison=POISON, order_count=order_count, span=span, rows=rows,
                 )
                 assert torch.equal(rows_x.view(torch.int16), got_x.view(torch.int16))
                 assert rows_w is None or torch.equal(rows_w.view(torch.int32), got_w.view(torch.int32))
-        # ... so must the walk with and without its window-wise source prefetch, in both kernel variants
+        # ... so must the walk with and without its window-wise source prefetch
         for prefetch in (0, 1):
-            for whole_rows in (0, 1):
+            for rows in (None, 3):
                 for order_count in ("exact", "device"):
                     fetched_x, _, fetched_w = cabi.dispatch(
                         x.to(device), None if w is None else w.to(device), metadata, counts, experts, alignment, expand, zero_padding,
-                        num_cus=num_cus, poison=POISON, prefetch=prefetch, whole_rows=whole_rows, order_count=order_count,
+                        num_cus=num_cus, poison=POISON, prefetch=prefetch, rows=rows, order_count=order_count,
                     )
                     assert torch.equal(fetched_x.view(torch.int16), got_x.view(torch.int16))
                     assert fetched_w is None or torch.equal(fetched_w.view(torch.int32), got_w.view(torch.int32))
