@@ -522,9 +522,8 @@ def measure(workload, args, device, detailed):
         _, dispatch_gpu = series(do_dispatch)
         _, combine_gpu = series(do_combine)
         _, hot_gpu = series(do_dispatch_hot) if everything else (None, dispatch_gpu)
-        # the same two dispatch series with the walk's window-wise source prefetch forced on and off
-        # (the library turns it on by itself for rows of two chunks only, where it costs nothing with
-        # cache-resident sources; elsewhere it trades the one for the other and is the caller's switch)
+        # the same two dispatch series with the walk's window-wise source prefetch forced off and on
+        # (on is the library's default; off is for callers whose sources sit in the last-level cache)
         prefetch_gpu = {}
         if workload.expand and everything:
             for setting in (0, 1):
@@ -588,7 +587,7 @@ def measure(workload, args, device, detailed):
     hot_us, hot_us_min = summarize(hot_gpu, launches)
     value = (d_bytes + c_bytes) / wall_us / 1e3
     # the kernels the library routes this workload to (names as a kernel trace shows them)
-    dispatch_kernel = "dispatch_ordered_kernel" if workload.expand else "dispatch_compact_kernel"
+    dispatch_kernel = "dispatch_walk_kernel" if workload.expand else "dispatch_compact_kernel"
     if not workload.expand:
         combine_kernel = "combine_compact_kernel"
     else:
@@ -650,7 +649,7 @@ def measure(workload, args, device, detailed):
                    "frac": round(d_bytes / summarize(cold, launches)[0] / 1e3 / HBM_PEAK_GBS, 4)}
             for name, (cold, hot) in (("off", prefetch_gpu[0]), ("on", prefetch_gpu[1]))
         }
-        result["dispatch_prefetch_switch"]["default"] = "on" if 512 < workload.hidden <= 1024 else "off"
+        result["dispatch_prefetch_switch"]["default"] = "on"
     if side is not None:
         result["side_stream_consumer"] = side
     if ceilings is not None:

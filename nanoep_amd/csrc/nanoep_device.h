@@ -236,7 +236,7 @@ inline RowBlocking pick_row_blocking(int chunks, WalkShape shape, const Tuning& 
 // List entries a workgroup of the slot-order walk takes when a row has up to four pieces (longer
 // rows take a workgroup each, one wavefront a piece).
 inline int default_walk_rows(int pieces) {
-    return pieces >= 4 ? 1 : 4 / pieces;
+    return pieces == 3 ? 1 : pieces == 1 ? 4 : 2;
 }
 
 inline int validate_cu_budget(int num_cus, const Topology& topology) {

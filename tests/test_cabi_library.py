@@ -82,7 +82,7 @@ def test_argument_checks_come_before_any_device_work():
     # rows of up to 4096 elements: windows of 512 tokens (two layout blocks) once there are eight of them
     assert [library.nanoep_layout_block_tokens(t, 256, 2048) for t in sizes] == [256, 256, 64, 64, 128, 128, 128, 256, 256, 512, 512, 512]
     # a window's rows fit an XCD's 4 MiB L2
-    assert [library.nanoep_layout_block_tokens(100000, 256, h) for h in (8, 1024, 1032, 4096, 4104, 8192, 8200, 16384, 16392, 1 << 20)] == [1024, 1024, 512, 512, 256, 256, 128, 128, 64, 64]
+    assert [library.nanoep_layout_block_tokens(100000, 256, h) for h in (8, 1024, 1032, 3840, 3848, 7680, 7688, 15360, 15368, 1 << 20)] == [1024, 1024, 512, 512, 256, 256, 128, 128, 64, 64]
     # windows of 1024 tokens (rows of up to 1024 elements) once there are sixteen of them
     assert [library.nanoep_layout_block_tokens(t, 256, 1024) for t in (4096, 15360, 15361, 16384)] == [512, 512, 1024, 1024]
     assert library.nanoep_layout_block_tokens(100000, 1400, 2048) == 512  # four layout blocks of 128 tokens (1401 LDS rows)
@@ -127,9 +127,9 @@ def test_topology_defaults_and_overrides_size_the_windows():
     try:
         library.nanoep_set_tuning(b"L2_BYTES", 8 << 20)
         assert cabi.device_topology() == (256, 8, 8 << 20)
-        assert [library.nanoep_layout_block_tokens(100000, 256, h) for h in (2048, 4096, 8192, 16384)] == [1024, 512, 512, 256]
+        assert [library.nanoep_layout_block_tokens(100000, 256, h) for h in (2048, 4096, 8192, 16384)] == [1024, 512, 256, 128]
         library.nanoep_set_tuning(b"L2_BYTES", 2 << 20)
-        assert [library.nanoep_layout_block_tokens(100000, 256, h) for h in (4096, 8192, 16384)] == [256, 128, 64]
+        assert [library.nanoep_layout_block_tokens(100000, 256, h) for h in (3840, 7680, 16384)] == [256, 128, 64]
         library.nanoep_set_tuning(b"L2_BYTES", 0)
         library.nanoep_set_tuning(b"XCDS", 4)
         assert cabi.device_topology() == (256, 4, 4 << 20)
