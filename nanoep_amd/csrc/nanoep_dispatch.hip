@@ -177,9 +177,12 @@ struct WalkArgs {
     uint32_t prefetch_blocks;  // prefetch workgroups at the head of a segment
     uint32_t window_vectors;   // 16-byte vectors of one window's source rows
     uint32_t source_vectors;   // ... of all source rows
+    uint32_t segment_entries;       // list entries of a segment: ceil(entries / windows)
+    uint32_t segment_copy_entries;  // list entries the copy workgroups of a segment cover in one turn
     // entry count on the device
-    uint32_t share_magic;  // fast divisor by the copy workgroups of a segment
-    uint32_t share_shift;
+    uint32_t windows;  // segments of the walk
+    uint32_t windows_magic;  // fast divisor by it
+    uint32_t windows_shift;
     uint32_t rows_magic;  // fast divisor by rows_per_block
     uint32_t rows_shift;
     const int64_t* live_count;
@@ -228,48 +231,10 @@ __device__ __forceinline__ void walk_gap_rows(const WalkArgs& a, uint32_t xcd, u
 // HBM; what it costs is one more L2 read per source row.
 constexpr int kPrefetchLoads = 4;
 
-// One workgroup's turn at the slot-order walk: `block` is its position in the walk (with prefetch:
-// among the prefetch and copy workgroups of all segments).
-template <int kPieces, int kSpan, bool kPrefetch>
-__device__ __forceinline__ void walk_copy(const WalkArgs& a, uint32_t entries, uint32_t block) {
-    if (kPrefetch) {
-        const uint32_t segment = fast_divide(block, a.segment_magic, a.segment_shift);
-        const uint32_t within = block - segment * a.segment_blocks;
-        if (within < a.prefetch_blocks) {
-            const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
-            const uint32_t waves = blockDim.x / kWave;
-            const uint64_t window_first = static_cast<uint64_t>(segment) * a.window_vectors;
-            uint64_t window_end = window_first + a.window_vectors;
-            if (window_end > a.source_vectors)
-                window_end = a.source_vectors;
-            const uint64_t first = window_first + static_cast<uint64_t>(within * waves + wave) * (kPrefetchLoads * kWave);
-            if (first < window_end) {
-                u32x4 fetched[kPrefetchLoads];
-#pragma unroll
-                for (int u = 0; u < kPrefetchLoads; ++u) {
-                    const uint64_t from = first + u * kWave + threadIdx.x % kWave;
-                    fetched[u] = a.x[from < window_end ? from : window_first];
-                }
-#pragma unroll
-                for (int u = 0; u < kPrefetchLoads; ++u)
-                    asm volatile("" ::"v"(fetched[u].x), "v"(fetched[u].y), "v"(fetched[u].z), "v"(fetched[u].w));
-            }
-            return;
-        }
-        block = segment * (a.segment_blocks - a.prefetch_blocks) + (within - a.prefetch_blocks);
-    }
-    // the list entry of this wavefront and the first 16-byte vector of the row its lanes move
-    uint32_t candidate, lane_vector;
-    if (kPieces == 0) {
-        candidate = block;
-        lane_vector = kSpan == 1 ? threadIdx.x : (threadIdx.x / kWave) * (kSpan * kWave) + threadIdx.x % kWave;
-    } else {
-        const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
-        const uint32_t row = wave / kPieces;
-        candidate = block * a.rows_per_block + row;
-        lane_vector = kSpan == 1 ? threadIdx.x - row * (kPieces * kWave)
-                                 : (wave - row * kPieces) * (kSpan * kWave) + threadIdx.x % kWave;
-    }
+// One wavefront's copy: list entry `candidate`, the piece of its row that starts at 16-byte vector
+// `lane_vector` of this lane.
+template <int kSpan>
+__device__ __forceinline__ void walk_copy_entry(const WalkArgs& a, uint32_t entries, uint32_t candidate, uint32_t lane_vector) {
     if (candidate >= entries)
         return;
     const int64_t entry = uniform_load_at(a.slot_order, candidate);
@@ -294,7 +259,7 @@ __device__ __forceinline__ void walk_copy(const WalkArgs& a, uint32_t entries, u
         data[s] = *reinterpret_cast<const u32x4*>(from + (at_bytes < a.row_bytes ? at_bytes : 0u));
     }
     // the entry's weight rides with the first lane of its row while the payload is in flight
-    // (weight_lane is no lane at all when there are no weights to move here)
+    // (weight_lane is no lane at all when there are no weights to move)
     if (lane_vector == a.weight_lane)
         a.recv_weights[out_row] = a.weights[source];
 #pragma unroll
@@ -303,6 +268,66 @@ __device__ __forceinline__ void walk_copy(const WalkArgs& a, uint32_t entries, u
         if (at_bytes < a.row_bytes)
             store_vec<true>(reinterpret_cast<u32x4*>(to + at_bytes), data[s]);
     }
+}
+
+// One workgroup's turn at the slot-order walk; `block` is its position in the walk.
+// Without prefetch the walk is the list front to back, rows_per_block entries a workgroup.
+// With prefetch the walk is cut into one segment per window of the list: `prefetch_blocks`
+// workgroups that read the window's source rows, then `segment_copy_entries / rows_per_block`
+// workgroups that copy the segment's share of the list, entries [s * segment_entries, (s + 1) *
+// segment_entries) of it.  The windows hold nearly the same number of entries each, so equal shares
+// follow them closely (a skewed mask only costs locality).  With the entry count on the device the
+// host sizes the segments' workgroups for the count it expects and the share follows the live count:
+// workgroups beyond it leave at once, and where it is larger they take more than one turn.
+template <int kPieces, int kSpan, bool kDeviceCount, bool kPrefetch>
+__device__ __forceinline__ void walk_copy(const WalkArgs& a, uint32_t entries, uint32_t segment_entries, uint32_t block) {
+    // the entry of this wavefront within its workgroup and the first 16-byte vector of the row its lanes move
+    uint32_t row = 0, lane_vector;
+    if (kPieces == 0) {
+        lane_vector = kSpan == 1 ? threadIdx.x : (threadIdx.x / kWave) * (kSpan * kWave) + threadIdx.x % kWave;
+    } else {
+        const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
+        row = wave / kPieces;
+        lane_vector = kSpan == 1 ? threadIdx.x - row * (kPieces * kWave)
+                                 : (wave - row * kPieces) * (kSpan * kWave) + threadIdx.x % kWave;
+    }
+    if (!kPrefetch) {
+        walk_copy_entry<kSpan>(a, entries, kPieces == 0 ? block : block * a.rows_per_block + row, lane_vector);
+        return;
+    }
+    const uint32_t segment = fast_divide(block, a.segment_magic, a.segment_shift);
+    const uint32_t within = block - segment * a.segment_blocks;
+    if (within < a.prefetch_blocks) {
+        const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
+        const uint32_t waves = blockDim.x / kWave;
+        const uint64_t window_first = static_cast<uint64_t>(segment) * a.window_vectors;
+        uint64_t window_end = window_first + a.window_vectors;
+        if (window_end > a.source_vectors)
+            window_end = a.source_vectors;
+        const uint64_t first = window_first + static_cast<uint64_t>(within * waves + wave) * (kPrefetchLoads * kWave);
+        if (first < window_end) {
+            u32x4 fetched[kPrefetchLoads];
+#pragma unroll
+            for (int u = 0; u < kPrefetchLoads; ++u) {
+                const uint64_t from = first + u * kWave + threadIdx.x % kWave;
+                fetched[u] = a.x[from < window_end ? from : window_first];
+            }
+#pragma unroll
+            for (int u = 0; u < kPrefetchLoads; ++u)
+                asm volatile("" ::"v"(fetched[u].x), "v"(fetched[u].y), "v"(fetched[u].z), "v"(fetched[u].w));
+        }
+        return;
+    }
+    const uint32_t copy_block = within - a.prefetch_blocks;
+    uint32_t in_segment = kPieces == 0 ? copy_block : copy_block * a.rows_per_block + row;
+    const uint32_t segment_first = segment * segment_entries;
+    if (!kDeviceCount) {
+        if (in_segment < segment_entries)
+            walk_copy_entry<kSpan>(a, entries, segment_first + in_segment, lane_vector);
+        return;
+    }
+    for (; in_segment < segment_entries; in_segment += a.segment_copy_entries)
+        walk_copy_entry<kSpan>(a, entries, segment_first + in_segment, lane_vector);
 }
 
 // The slot-order walk.  Its wavefronts are short (a list entry, a source load, a store) and there are
@@ -324,30 +349,34 @@ __global__ void __launch_bounds__(1024) dispatch_walk_kernel(const WalkArgs a) {
         NANOEP_FETCH_ARGS_4(a.segment_blocks, a.segment_magic, a.segment_shift, a.prefetch_blocks);
     const uint32_t index_in_xcd = fast_divide(blockIdx.x, a.xcd_magic, a.xcd_shift);
     const uint32_t xcd = blockIdx.x - index_in_xcd * a.xcd_count;
-    if (!kDeviceCount) {
+    if (!kDeviceCount || kPrefetch) {
+        // the grid's shape is the host's: with prefetch the segments are the windows of the batch
         if (index_in_xcd >= a.copy_per_xcd) {
             walk_gap_rows(a, xcd, index_in_xcd - a.copy_per_xcd);
             __builtin_amdgcn_endpgm();
         }
-        walk_copy<kPieces, kSpan, kPrefetch>(a, a.entries, xcd * a.copy_per_xcd + index_in_xcd);
+        uint32_t entries = a.entries, segment_entries = a.segment_entries;
+        if (kDeviceCount) {
+            // a word that cannot be a count (the layout did not run) walks nothing
+            const int64_t live = uniform_load(a.live_count);
+            entries = live >= 0 && live <= static_cast<int64_t>(a.source_limit) ? static_cast<uint32_t>(live) : 0u;
+            segment_entries = fast_divide(entries + a.windows - 1, a.windows_magic, a.windows_shift);
+        }
+        walk_copy<kPieces, kSpan, kDeviceCount, kPrefetch>(a, entries, segment_entries, xcd * a.copy_per_xcd + index_in_xcd);
         return;
     }
-    // The entry count is on the device: the live list may be shorter than what the grid was sized for
-    // (the rest of the grid leaves at once) or longer (workgroups then take more than one turn, a
-    // grid's worth of list positions apart).  A word that cannot be a count (the layout did not run)
-    // walks nothing.
+    // The entry count is on the device and the walk is the plain list: the live list may be shorter
+    // than what the grid was sized for (the rest of the grid leaves at once) or longer (workgroups
+    // then take more than one turn, a grid's worth of list positions apart).  A word that cannot be a
+    // count (the layout did not run) walks nothing.
     const int64_t live = uniform_load(a.live_count);
     const uint32_t entries = live >= 0 && live <= static_cast<int64_t>(a.source_limit) ? static_cast<uint32_t>(live) : 0u;
     const uint32_t copy_blocks = kPieces == 0 ? entries : fast_divide(entries + a.rows_per_block - 1, a.rows_magic, a.rows_shift);
-    // with prefetch: whole segments of the size the host chose (from the count it expected)
-    const uint32_t walk_blocks =
-        kPrefetch ? fast_divide(copy_blocks + (a.segment_blocks - a.prefetch_blocks) - 1, a.share_magic, a.share_shift) * a.segment_blocks
-                  : copy_blocks;
-    const uint32_t copy_per_xcd = fast_divide(walk_blocks + a.xcd_count - 1, a.xcd_magic, a.xcd_shift);
+    const uint32_t copy_per_xcd = fast_divide(copy_blocks + a.xcd_count - 1, a.xcd_magic, a.xcd_shift);
     const uint32_t copy_turns = copy_per_xcd > a.copy_per_xcd ? a.copy_per_xcd : copy_per_xcd;
     if (index_in_xcd < copy_turns) {
         for (uint32_t at = index_in_xcd; at < copy_per_xcd; at += a.copy_per_xcd)
-            walk_copy<kPieces, kSpan, kPrefetch>(a, entries, xcd * copy_per_xcd + at);
+            walk_copy<kPieces, kSpan, kDeviceCount, kPrefetch>(a, entries, 0u, xcd * copy_per_xcd + at);
     } else {
         walk_gap_rows(a, xcd, index_in_xcd - copy_turns);
     }
@@ -513,23 +542,24 @@ int nanoep_dispatch(const void* x, const float* weights, const int32_t* recv_met
         // NANOEP_DISPATCH_PREFETCH=0.
         const int window_tokens = nanoep_layout_block_tokens(num_tokens, num_local_experts, hidden);
         const bool prefetch = window_tokens > 0 && copy_blocks > 0 && tuning.dispatch_prefetch != 0;
-        int64_t segment_copy_blocks = 0, segment_prefetch_blocks = 0, segments = 0;
+        // Segments are the windows of the batch; each takes the workgroups that copy its share of the
+        // entries the host expects, behind the ones that read the window's rows.
+        int64_t segment_entries = 0, segment_copy_blocks = 0, segment_prefetch_blocks = 0, windows = 1;
         if (prefetch) {
-            const int64_t windows = (num_tokens + window_tokens - 1) / window_tokens;
-            const int64_t segment_entries = (slot_order_entries + windows - 1) / windows;
+            windows = (num_tokens + window_tokens - 1) / window_tokens;
+            segment_entries = (slot_order_entries + windows - 1) / windows;
             segment_copy_blocks = (segment_entries + rows_per_block - 1) / rows_per_block;
-            segments = (copy_blocks + segment_copy_blocks - 1) / segment_copy_blocks;
             const int64_t window_kib = (static_cast<int64_t>(window_tokens) * vectors + kWave - 1) / kWave;
             segment_prefetch_blocks = (window_kib + waves * kPrefetchLoads - 1) / (waves * kPrefetchLoads);
         }
-        const int64_t walk_blocks = prefetch ? segments * (segment_copy_blocks + segment_prefetch_blocks) : copy_blocks;
+        const int64_t walk_blocks = prefetch ? windows * (segment_copy_blocks + segment_prefetch_blocks) : copy_blocks;
         if (walk_blocks + pad_blocks >= (int64_t{1} << 31) - 2 * int64_t{xcds.count})
             return NANOEP_ERR_INVALID_ARGUMENT;
         const uint32_t copy_per_xcd = static_cast<uint32_t>((walk_blocks + xcds.count - 1) / xcds.count);
         const uint32_t pad_per_xcd = static_cast<uint32_t>((pad_blocks + xcds.count - 1) / xcds.count);
         const FastDivisor topk_divisor = make_fast_divisor(static_cast<uint32_t>(num_topk));
         const FastDivisor rows_divisor = make_fast_divisor(static_cast<uint32_t>(rows_per_block));
-        const FastDivisor share_divisor = make_fast_divisor(static_cast<uint32_t>(prefetch ? segment_copy_blocks : 1));
+        const FastDivisor windows_divisor = make_fast_divisor(static_cast<uint32_t>(windows));
         const FastDivisor segment_divisor =
             make_fast_divisor(static_cast<uint32_t>(prefetch ? segment_copy_blocks + segment_prefetch_blocks : 1));
         WalkArgs a{};
@@ -556,8 +586,11 @@ int nanoep_dispatch(const void* x, const float* weights, const int32_t* recv_met
         a.prefetch_blocks = static_cast<uint32_t>(segment_prefetch_blocks);
         a.window_vectors = static_cast<uint32_t>(static_cast<int64_t>(window_tokens) * vectors);
         a.source_vectors = static_cast<uint32_t>(num_tokens * vectors);
-        a.share_magic = share_divisor.magic;
-        a.share_shift = share_divisor.shift;
+        a.segment_entries = static_cast<uint32_t>(segment_entries);
+        a.segment_copy_entries = static_cast<uint32_t>(segment_copy_blocks * rows_per_block);
+        a.windows = static_cast<uint32_t>(windows);
+        a.windows_magic = windows_divisor.magic;
+        a.windows_shift = windows_divisor.shift;
         a.rows_magic = rows_divisor.magic;
         a.rows_shift = rows_divisor.shift;
         a.live_count = live_count;
