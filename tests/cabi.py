@@ -243,8 +243,10 @@ def dispatch(x, weights, metadata, counts, num_local_experts, alignment, expand,
     return recv_x, recv_idx, recv_w
 
 
-def combine(y, weights, bias, metadata, counts, expand, *, multiple_reduction=False, num_cus=0, poison=None, use_table=True):
-    """Returns (out_x [T,H], out_weights [T,K] | None) through nanoep_combine."""
+def combine(y, weights, bias, metadata, counts, expand, *, multiple_reduction=False, num_cus=0, poison=None, use_table=True,
+            stores=None):
+    """Returns (out_x [T,H], out_weights [T,K] | None) through nanoep_combine.  stores=0|1 asks for
+    nontemporal / agent-scope stores of the output rows (the library picks by output size)."""
     recv_metadata, dst_slots = metadata[0], metadata[3]
     tokens = dst_slots.shape[0]
     topk = recv_metadata.shape[1] - 2
@@ -256,11 +258,12 @@ def combine(y, weights, bias, metadata, counts, expand, *, multiple_reduction=Fa
         for tensor in (out_x, out_w):
             if tensor is not None and tensor.numel():
                 tensor.view(torch.uint8).fill_(poison)
-    check(
-        lib().nanoep_combine(
-            ptr(y), ptr(weights), ptr(bias), ptr(recv_metadata), ptr(dst_slots), ptr(token_slots_of(metadata, use_table)), counts[0],
-            y.shape[0], tokens,
-            hidden, topk, int(expand), int(multiple_reduction), ptr(out_x), ptr(out_w), num_cus, stream_handle(),
+    with forced_tuning({"COMBINE_STORES": stores}):
+        check(
+            lib().nanoep_combine(
+                ptr(y), ptr(weights), ptr(bias), ptr(recv_metadata), ptr(dst_slots), ptr(token_slots_of(metadata, use_table)), counts[0],
+                y.shape[0], tokens,
+                hidden, topk, int(expand), int(multiple_reduction), ptr(out_x), ptr(out_w), num_cus, stream_handle(),
+            )
         )
-    )
     return out_x, out_w

@@ -174,6 +174,16 @@ def run_dispatch_combine(device, idx, hidden, experts, alignment, expand, zero_p
         assert_bits_equal(got_out, want_out, f"combine x multi={multi}")
         if weighted:
             assert_bits_equal(got_ow, want_ow, "combine weights")
+        # either kind of store for the output rows
+        for stores in (0, 1):
+            stored_out, stored_ow = cabi.combine(
+                y.to(device), None if yw is None else yw.to(device), None if bias is None else bias.to(device), metadata,
+                counts, expand, multiple_reduction=multi, num_cus=num_cus, poison=POISON, stores=stores,
+            )
+            torch.cuda.synchronize()
+            assert_bits_equal(stored_out, want_out, f"combine x multi={multi} stores={stores}")
+            if weighted:
+                assert_bits_equal(stored_ow, want_ow, f"combine weights stores={stores}")
         if expand:
             plain_out, plain_ow = cabi.combine(
                 y.to(device), None if yw is None else yw.to(device), None if bias is None else bias.to(device), metadata,
