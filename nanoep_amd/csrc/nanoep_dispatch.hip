@@ -438,7 +438,7 @@ __global__ void __launch_bounds__(1024) dispatch_compact_kernel(const u32x4* __r
     const uint32_t vector = chunk * kWave + threadIdx.x;
     const bool in_row = vector < vectors;
     // the source address depends on the block index alone: its load is in flight during the lookup
-    const u32x4 data = x[static_cast<uint64_t>(token) * vectors + (in_row ? vector : 0u)];
+    const u32x4 data = load_vec<true>(x + static_cast<uint64_t>(token) * vectors + (in_row ? vector : 0u));
     const int64_t row = uniform_load(dst_slots + token);
     if (row < 0 || row >= static_cast<int64_t>(recv_count))
         return;
