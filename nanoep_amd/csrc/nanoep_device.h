@@ -18,12 +18,13 @@
 //   layout_single_block_kernel : (one block) count and assignment passes in a single launch.
 //   layout_scan_kernel + layout_assign_kernel<no scan> : (many blocks) the same in two launches, one
 //                          workgroup doing the scans: slot = offset[e] + block_base[b][e] + rank.
-//   dispatch_ordered_kernel : expanded layouts with the layout's slot-order list: one wavefront per
-//                          (list entry, row chunk), token block by token block and expert-major
-//                          inside a block, so a block's source rows stay in one XCD's L2 and every
+//   dispatch_walk_kernel : expanded layouts with the layout's slot-order list: one wavefront per
+//                          (list entry, row chunk), window of tokens by window and expert-major
+//                          inside a window, so a window's source rows stay in one XCD's L2 and every
 //                          expert receives runs of consecutive rows; one 128-bit load and one
-//                          nontemporal 128-bit store per lane.  Optionally a few workgroups ahead
-//                          of every window read its source rows front to back (prefetch).
+//                          nontemporal 128-bit store per lane, as few scalar instructions ahead of
+//                          the load as the work allows.  A few workgroups ahead of every window read
+//                          its source rows front to back (prefetch).
 //   dispatch_rows_kernel : the same work item walked in source-token order (small batches, handles
 //                          without the list); extra work items zero-fill the alignment gaps.
 //   dispatch_compact_kernel / combine_compact_kernel : compact layouts are row copies with holes;

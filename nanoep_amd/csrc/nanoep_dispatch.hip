@@ -9,14 +9,16 @@ namespace {
 // one 128-bit load and one nontemporal 128-bit store per lane: on this part a wavefront that issues
 // a single store and retires sustains more HBM write bandwidth than one that issues several.
 //
-// A workgroup is (64, chunks_per_block, rows_per_block): threadIdx.y is the chunk, threadIdx.z the
-// destination candidate, so no per-wave division by the chunk count is needed.  In the token-order
-// walk of the expanded layout (dispatch_rows_kernel) candidates are ordered (source token, k): the K destinations of a token are handled by consecutive workgroups
-// behind one XCD's L2, so only the first read of a source row goes to HBM, and every destination
-// row is written as one contiguous run by the wavefronts of one workgroup.  The source address
-// depends only on the block index, so its load is in flight while the wave-uniform lookups
-// (token_slots[t][k], or dst_slots[t] -> recv_metadata[row][2+k] for a handle without that table)
-// resolve the destination row.
+// The token-order walks and the compact row copy use workgroups of (64, chunks_per_block,
+// rows_per_block): threadIdx.y is the chunk, threadIdx.z the destination candidate, so no per-wave
+// division by the chunk count is needed.  In the token-order walk of the expanded layout
+// (dispatch_rows_kernel) candidates are ordered (source token, k): the K destinations of a token are
+// handled by consecutive workgroups behind one XCD's L2, so only the first read of a source row goes
+// to HBM, and every destination row is written as one contiguous run by the wavefronts of one
+// workgroup.  The source address depends only on the block index, so its load is in flight while the
+// wave-uniform lookups (token_slots[t][k], or dst_slots[t] -> recv_metadata[row][2+k] for a handle
+// without that table) resolve the destination row.  The slot-order walk (dispatch_walk_kernel, further
+// down) has one-dimensional workgroups and its own, leaner bookkeeping.
 //
 // Zero-fill workgroups clear the alignment gaps: workgroup (e, g) owns gap candidates
 // j = g * waves .. of expert e, row offsets[e] + counts[e] + j while that is below offsets[e+1].
