@@ -516,6 +516,19 @@ def test_randomized_shapes(device, seed):
     run_dispatch_combine(device, idx, hidden, experts, alignment, expand, zero_padding, weighted, seed=seed)
 
 
+@pytest.mark.parametrize(
+    "hidden,tokens",
+    [(8200, 300), (16384, 257), (16392, 300), (32768, 260), (32776, 120), (65544, 70)],
+    ids=["17-chunks", "32-chunks", "33-chunks", "64-chunks", "65-chunks-token-order", "129-chunks-token-order"],
+)
+def test_rows_wider_than_a_workgroup_of_single_chunks(device, hidden, tokens):
+    """Rows of more than 16 KiB: the slot-order walk moves two or four chunks a wavefront so that 16
+    wavefronts still cover a row; rows beyond 64 KiB take the token-order walk.  Bit for bit against
+    the oracle either way, with every forced width that still fits."""
+    idx = cases.routing("dropout", tokens, 9, 3, seed=hidden)
+    run_dispatch_combine(device, idx, hidden, 9, 4, True, True, True, seed=tokens)
+
+
 @pytest.mark.parametrize("seed", range(10))
 def test_randomized_multi_block_shapes(device, seed):
     """Seeded batches of a thousand to nine thousand tokens (many layout blocks, token counts that
