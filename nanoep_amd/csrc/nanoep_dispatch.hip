@@ -229,8 +229,9 @@ __device__ __forceinline__ void walk_gap_rows(const WalkArgs& a, uint32_t xcd, u
 // copy workgroups of every segment are preceded by a few workgroups that read the window's source
 // rows front to back (kPrefetchLoads KiB a wavefront, the data dropped).  The window's first touches
 // then reach HBM as one sequential burst ahead of the segment's stores instead of one row at a time
-// among them, and the copy wavefronts find their rows in the XCD's L2.  No bytes are read twice from
-// HBM; what it costs is one more L2 read per source row.
+// among them, and the copy wavefronts find their rows in the XCD's L2 (unless the write stream has
+// pushed a row out again before its last use: a window close to the size of the L2 re-reads part of
+// itself).  What it costs otherwise is one more L2 read per source row.
 constexpr int kPrefetchLoads = 4;
 
 // One wavefront's copy: list entry `candidate`, the piece of its row that starts at 16-byte vector
@@ -498,7 +499,7 @@ int nanoep_dispatch(const void* x, const float* weights, const int32_t* recv_met
     // once the source outgrows the last-level cache (the single-chunk walk then loses a quarter of
     // its rate) and as many as it takes for a row to fit the 16 wavefronts of a workgroup
     // (NANOEP_DISPATCH_SPAN=1|2|4 asks for a number).  The walk addresses the list with 32-bit byte
-    // offsets: lists of 2^29 entries and more, and rows beyond 64 KiB, take the token-order walk.
+    // offsets: list buffers of 2^29 entries and more, and rows beyond 64 KiB, take the token-order walk.
     int span = static_cast<int64_t>(num_tokens) * hidden * 2 > kLastLevelCacheBytes ? 2 : 1;
     if (tuning.dispatch_span == 1 || tuning.dispatch_span == 2 || tuning.dispatch_span == 4)
         span = tuning.dispatch_span;
@@ -506,7 +507,7 @@ int nanoep_dispatch(const void* x, const float* weights, const int32_t* recv_met
         span *= 2;
     const int pieces = (row_chunks + span - 1) / span;
     const bool ordered = expand && slot_order != nullptr && order_bound > 0 && tuning.dispatch_order != 0 &&
-                         pieces <= kMaxWavesPerBlock && num_tokens * num_topk < (int64_t{1} << 29);
+                         pieces <= kMaxWavesPerBlock && order_bound < (int64_t{1} << 29);
     if (ordered && slot_order_entries > order_bound)
         return NANOEP_ERR_INVALID_ARGUMENT;
     if (num_tokens * num_topk >= (int64_t{1} << 31) || static_cast<int64_t>(num_tokens) * vectors >= (int64_t{1} << 32))
