@@ -86,6 +86,7 @@ struct Tuning {
     int dispatch_order = -1;        // DISPATCH_ORDER: 0 forces the token-order walk
     int dispatch_span = 0;          // DISPATCH_SPAN: 1 | 2 | 4 chunks a wavefront of the slot-order walk, 0 = by size
     int dispatch_prefetch = -1;     // DISPATCH_PREFETCH: 0 = no window-wise source prefetch in the slot-order walk
+    int dispatch_pack = 0;          // DISPATCH_PACK: 1 = one list entry a wavefront of the slot-order walk whatever the row length
     int combine_stores = -1;        // COMBINE_STORES: 0 | 1 nontemporal / agent-scope stores for the combine's output, -1 = by size
     int layout_launches = 0;        // LAYOUT_LAUNCHES: 2 | 3 forces the layout plan
     int window_tokens = 0;          // WINDOW_TOKENS: forces the window of the slot-order list

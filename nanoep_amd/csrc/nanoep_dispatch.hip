@@ -168,7 +168,7 @@ struct WalkArgs {
     uint32_t xcd_count;
     uint32_t xcd_magic;  // fast divisor by the XCD count
     uint32_t xcd_shift;
-    uint32_t rows_per_block;  // list entries a workgroup (rows of up to four pieces)
+    uint32_t rows_per_block;  // list entries a workgroup (rows of up to four pieces; with packed rows: wavefronts x entries a wavefront)
     uint32_t weight_lane;     // 0: the first lane of a row moves the entry's weight; ~0: there are no weights
     const float* weights;     // [T][K] or null
     float* recv_weights;      // [C] or null
@@ -273,6 +273,27 @@ __device__ __forceinline__ void walk_copy_entry(const WalkArgs& a, uint32_t entr
     }
 }
 
+// The same for rows of at most 512 bytes: a wavefront moves kPack list entries at once, its lanes
+// split into kPack groups of 64 / kPack, so that no half of it idles.  Entry, range checks and
+// addresses are per lane here (the groups of a wavefront differ in them); `candidate` is the lane's
+// list entry and `vector` its 16-byte vector of the row.
+template <int kPack>
+__device__ __forceinline__ void walk_copy_packed(const WalkArgs& a, uint32_t entries, uint32_t candidate, uint32_t vector) {
+    if (candidate >= entries)
+        return;
+    const int64_t entry = a.slot_order[candidate];
+    const uint32_t source = static_cast<uint32_t>(entry);
+    const uint32_t out_row = static_cast<uint32_t>(static_cast<uint64_t>(entry) >> 32);
+    // (a negative entry has an impossible row)
+    if (out_row >= a.out_rows || source >= a.source_limit || vector * 16u >= a.row_bytes)
+        return;
+    const uint32_t token = fast_divide(source, a.topk_magic, a.topk_shift);
+    const u32x4 data = *reinterpret_cast<const u32x4*>(reinterpret_cast<const char*>(a.x) + static_cast<uint64_t>(token) * a.row_bytes + vector * 16u);
+    if (vector == a.weight_lane)
+        a.recv_weights[out_row] = a.weights[source];
+    store_vec<true>(reinterpret_cast<u32x4*>(reinterpret_cast<char*>(a.recv_x) + static_cast<uint64_t>(out_row) * a.row_bytes + vector * 16u), data);
+}
+
 // One workgroup's turn at the slot-order walk; `block` is its position in the walk.
 // Without prefetch the walk is the list front to back, rows_per_block entries a workgroup.
 // With prefetch the walk is cut into one segment per window of the list: `prefetch_blocks`
@@ -284,18 +305,29 @@ __device__ __forceinline__ void walk_copy_entry(const WalkArgs& a, uint32_t entr
 // workgroups beyond it leave at once, and where it is larger they take more than one turn.
 template <int kPieces, int kSpan, bool kDeviceCount, bool kPrefetch>
 __device__ __forceinline__ void walk_copy(const WalkArgs& a, uint32_t entries, uint32_t segment_entries, uint32_t block) {
-    // the entry of this wavefront within its workgroup and the first 16-byte vector of the row its lanes move
-    uint32_t row = 0, lane_vector;
+    // kPieces -2 / -4: rows of one piece that fill half / a quarter of a wavefront, two / four entries a wavefront
+    constexpr int kPack = kPieces < 0 ? -kPieces : 1;
+    constexpr int kRowPieces = kPieces < 0 ? 1 : kPieces;
+    static_assert(kPack == 1 || kSpan == 1, "packed rows are single chunks");
+    // the entry of this lane within its workgroup and the first 16-byte vector of the row it moves
+    uint32_t in_block = 0, lane_vector;
     if (kPieces == 0) {
         lane_vector = kSpan == 1 ? threadIdx.x : (threadIdx.x / kWave) * (kSpan * kWave) + threadIdx.x % kWave;
-    } else {
+    } else if (kPack == 1) {
         const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
-        row = wave / kPieces;
-        lane_vector = kSpan == 1 ? threadIdx.x - row * (kPieces * kWave)
-                                 : (wave - row * kPieces) * (kSpan * kWave) + threadIdx.x % kWave;
+        in_block = wave / kRowPieces;
+        lane_vector = kSpan == 1 ? threadIdx.x - in_block * (kRowPieces * kWave)
+                                 : (wave - in_block * kRowPieces) * (kSpan * kWave) + threadIdx.x % kWave;
+    } else {
+        in_block = threadIdx.x / (kWave / kPack);
+        lane_vector = threadIdx.x % (kWave / kPack);
     }
     if (!kPrefetch) {
-        walk_copy_entry<kSpan>(a, entries, kPieces == 0 ? block : block * a.rows_per_block + row, lane_vector);
+        const uint32_t candidate = kPieces == 0 ? block : block * a.rows_per_block + in_block;
+        if (kPack == 1)
+            walk_copy_entry<kSpan>(a, entries, candidate, lane_vector);
+        else
+            walk_copy_packed<kPack>(a, entries, candidate, lane_vector);
         return;
     }
     const uint32_t segment = fast_divide(block, a.segment_magic, a.segment_shift);
@@ -322,15 +354,23 @@ __device__ __forceinline__ void walk_copy(const WalkArgs& a, uint32_t entries, u
         return;
     }
     const uint32_t copy_block = within - a.prefetch_blocks;
-    uint32_t in_segment = kPieces == 0 ? copy_block : copy_block * a.rows_per_block + row;
+    uint32_t in_segment = kPieces == 0 ? copy_block : copy_block * a.rows_per_block + in_block;
     const uint32_t segment_first = segment * segment_entries;
     if (!kDeviceCount) {
-        if (in_segment < segment_entries)
-            walk_copy_entry<kSpan>(a, entries, segment_first + in_segment, lane_vector);
+        if (in_segment < segment_entries) {
+            if (kPack == 1)
+                walk_copy_entry<kSpan>(a, entries, segment_first + in_segment, lane_vector);
+            else
+                walk_copy_packed<kPack>(a, entries, segment_first + in_segment, lane_vector);
+        }
         return;
     }
-    for (; in_segment < segment_entries; in_segment += a.segment_copy_entries)
-        walk_copy_entry<kSpan>(a, entries, segment_first + in_segment, lane_vector);
+    for (; in_segment < segment_entries; in_segment += a.segment_copy_entries) {
+        if (kPack == 1)
+            walk_copy_entry<kSpan>(a, entries, segment_first + in_segment, lane_vector);
+        else
+            walk_copy_packed<kPack>(a, entries, segment_first + in_segment, lane_vector);
+    }
 }
 
 // The slot-order walk.  Its wavefronts are short (a list entry, a source load, a store) and there are
@@ -340,6 +380,7 @@ __device__ __forceinline__ void walk_copy(const WalkArgs& a, uint32_t entries, u
 // no copy work.
 //   kPieces 0 : one workgroup a list entry, one wavefront a piece of the row (rows of 5 to 16 pieces)
 //   kPieces 1..4 : rows of that many pieces, rows_per_block entries a workgroup
+//   kPieces -2, -4 : rows of up to 512 / 256 bytes, two / four entries a wavefront
 //   kSpan   : 1 KiB chunks a wavefront moves (a piece)
 template <int kPieces, int kSpan, bool kDeviceCount, bool kPrefetch>
 __global__ void __launch_bounds__(1024) dispatch_walk_kernel(const WalkArgs a) {
@@ -535,7 +576,12 @@ int nanoep_dispatch(const void* x, const float* weights, const int32_t* recv_met
                 rows_per_block = default_walk_rows(pieces);
         }
         const int64_t waves = static_cast<int64_t>(pieces) * rows_per_block;
-        const int64_t copy_blocks = (slot_order_entries + rows_per_block - 1) / rows_per_block;
+        // Rows of at most 512 / 256 bytes fill half / a quarter of a wavefront: two / four list entries a
+        // wavefront then (65536 x 256 top-8: 75.1 -> 64.1 us with sources from HBM, 61.3 -> 45.4 with cache-resident
+        // ones; 65536 x 128: 57.6 -> 36.7 / 51.8 -> 24.2).  NANOEP_DISPATCH_PACK=1 keeps one entry a wavefront.
+        const int pack = pieces != 1 || span != 1 || tuning.dispatch_pack == 1 ? 1 : vectors <= kWave / 4 ? 4 : vectors <= kWave / 2 ? 2 : 1;
+        const int64_t entries_per_block = static_cast<int64_t>(rows_per_block) * pack;
+        const int64_t copy_blocks = (slot_order_entries + entries_per_block - 1) / entries_per_block;
         const int64_t pad_groups_per_expert = (pad_per_expert + waves - 1) / waves;
         const int64_t pad_blocks = num_local_experts * pad_groups_per_expert;
         // Prefetch workgroups ahead of every window's share of the list.  The list's windows hold
@@ -551,7 +597,7 @@ int nanoep_dispatch(const void* x, const float* weights, const int32_t* recv_met
         if (prefetch) {
             windows = (num_tokens + window_tokens - 1) / window_tokens;
             segment_entries = (slot_order_entries + windows - 1) / windows;
-            segment_copy_blocks = (segment_entries + rows_per_block - 1) / rows_per_block;
+            segment_copy_blocks = (segment_entries + entries_per_block - 1) / entries_per_block;
             const int64_t window_kib = (static_cast<int64_t>(window_tokens) * vectors + kWave - 1) / kWave;
             segment_prefetch_blocks = (window_kib + waves * kPrefetchLoads - 1) / (waves * kPrefetchLoads);
         }
@@ -561,7 +607,7 @@ int nanoep_dispatch(const void* x, const float* weights, const int32_t* recv_met
         const uint32_t copy_per_xcd = static_cast<uint32_t>((walk_blocks + xcds.count - 1) / xcds.count);
         const uint32_t pad_per_xcd = static_cast<uint32_t>((pad_blocks + xcds.count - 1) / xcds.count);
         const FastDivisor topk_divisor = make_fast_divisor(static_cast<uint32_t>(num_topk));
-        const FastDivisor rows_divisor = make_fast_divisor(static_cast<uint32_t>(rows_per_block));
+        const FastDivisor rows_divisor = make_fast_divisor(static_cast<uint32_t>(entries_per_block));
         const FastDivisor windows_divisor = make_fast_divisor(static_cast<uint32_t>(windows));
         const FastDivisor segment_divisor =
             make_fast_divisor(static_cast<uint32_t>(prefetch ? segment_copy_blocks + segment_prefetch_blocks : 1));
@@ -579,7 +625,7 @@ int nanoep_dispatch(const void* x, const float* weights, const int32_t* recv_met
         a.xcd_count = xcds.count;
         a.xcd_magic = xcds.magic;
         a.xcd_shift = xcds.shift;
-        a.rows_per_block = static_cast<uint32_t>(rows_per_block);
+        a.rows_per_block = static_cast<uint32_t>(entries_per_block);
         a.weight_lane = recv_weights == nullptr ? 0xffffffffu : 0u;
         a.weights = weights;
         a.recv_weights = recv_weights;
@@ -590,7 +636,7 @@ int nanoep_dispatch(const void* x, const float* weights, const int32_t* recv_met
         a.window_vectors = static_cast<uint32_t>(static_cast<int64_t>(window_tokens) * vectors);
         a.source_vectors = static_cast<uint32_t>(num_tokens * vectors);
         a.segment_entries = static_cast<uint32_t>(segment_entries);
-        a.segment_copy_entries = static_cast<uint32_t>(segment_copy_blocks * rows_per_block);
+        a.segment_copy_entries = static_cast<uint32_t>(segment_copy_blocks * entries_per_block);
         a.windows = static_cast<uint32_t>(windows);
         a.windows_magic = windows_divisor.magic;
         a.windows_shift = windows_divisor.shift;
@@ -627,7 +673,13 @@ int nanoep_dispatch(const void* x, const float* weights, const int32_t* recv_met
         else                               \
             NANOEP_LAUNCH_WALK(PIECES, 1); \
     } while (0)
-        switch (kernel_pieces) {
+        switch (pack > 1 ? -pack : kernel_pieces) {
+            case -4:
+                NANOEP_LAUNCH_WALK(-4, 1);
+                break;
+            case -2:
+                NANOEP_LAUNCH_WALK(-2, 1);
+                break;
             case 1:
                 NANOEP_LAUNCH_WALK_PIECES(1);
                 break;

@@ -194,7 +194,7 @@ def slot_order_of(metadata, use_order=True):
 
 
 def dispatch(x, weights, metadata, counts, num_local_experts, alignment, expand, zero_padding, *, num_cus=0, poison=None,
-             use_table=True, use_order=True, order_count="exact", walk="forced", span=None, rows=None, prefetch=None):
+             use_table=True, use_order=True, order_count="exact", walk="forced", span=None, rows=None, prefetch=None, pack=None):
     """Returns (recv_x, recv_topk_idx | None, recv_weights | None) through nanoep_dispatch.
 
     walk="forced" sets the library's switch for the slot-order walk explicitly, walk="auto" leaves
@@ -202,7 +202,8 @@ def dispatch(x, weights, metadata, counts, num_local_experts, alignment, expand,
     forces the number of chunks a wavefront of that walk moves (the library picks it by source size).
     rows=n asks for n list entries a workgroup of that walk (honoured for rows of up to four pieces while
     the workgroup stays within 16 wavefronts).  prefetch=0|1 forbids or asks for that walk's window-wise
-    source prefetch.
+    source prefetch.  pack=1 keeps one list entry a wavefront for rows of at most 512 bytes (the library
+    packs two or four).
     """
     recv_metadata, expert_counts, expert_offsets, dst_slots = metadata[0], metadata[1], metadata[2], metadata[3]
     received, capacity = counts[0], counts[1]
@@ -230,7 +231,7 @@ def dispatch(x, weights, metadata, counts, num_local_experts, alignment, expand,
     else:
         order_entries = -1 if order_count == "device" else -int(order_count[1])
     switches = {"DISPATCH_ORDER": 1 if walk == "forced" else None, "DISPATCH_SPAN": span,
-                "ROWS_PER_BLOCK": rows,
+                "ROWS_PER_BLOCK": rows, "DISPATCH_PACK": pack,
                 "DISPATCH_PREFETCH": None if prefetch is None else int(prefetch)}
     with forced_tuning(switches):
         status = lib().nanoep_dispatch(

@@ -120,6 +120,16 @@ def run_dispatch_combine(device, idx, hidden, experts, alignment, expand, zero_p
                     )
                     assert torch.equal(fetched_x.view(torch.int16), got_x.view(torch.int16))
                     assert fetched_w is None or torch.equal(fetched_w.view(torch.int32), got_w.view(torch.int32))
+        # ... so must rows of at most 512 bytes with one list entry a wavefront instead of two or four
+        if hidden <= 256:
+            for order_count in ("exact", "device"):
+                for rows in (None, 3):
+                    single_x, _, single_w = cabi.dispatch(
+                        x.to(device), None if w is None else w.to(device), metadata, counts, experts, alignment, expand, zero_padding,
+                        num_cus=num_cus, poison=POISON, pack=1, rows=rows, order_count=order_count,
+                    )
+                    assert torch.equal(single_x.view(torch.int16), got_x.view(torch.int16))
+                    assert single_w is None or torch.equal(single_w.view(torch.int32), got_w.view(torch.int32))
         # ... so must the same call with the library's switches left alone
         auto_x, _, auto_w = cabi.dispatch(
             x.to(device), None if w is None else w.to(device), metadata, counts, experts, alignment, expand, zero_padding,
