@@ -68,8 +68,8 @@ int nanoep_device_topology(int* out_cus, int* out_xcds, int64_t* out_l2_bytes);
  *                     walk takes ROWS_PER_BLOCK list entries a workgroup for rows of up to 4 KiB)
  *   DISPATCH_ORDER (-1; 0: token-order walk even when the handle has a slot-order list)
  *   DISPATCH_SPAN (0: by size; 1 | 2 | 4 chunks a wavefront of the slot-order walk)
- *   DISPATCH_PACK (0: rows of at most 512 / 256 bytes go two / four list entries a wavefront in that
- *                     walk; 1: one entry a wavefront whatever the row length)
+ *   DISPATCH_PACK (0: rows of at most 512 / 256 bytes go four / eight list entries a wavefront in
+ *                     that walk; 1: one entry a wavefront whatever the row length)
  *   DISPATCH_PREFETCH (-1: on; 0: no window-wise source prefetch in that walk, for sources that are
  *                     known to sit in the last-level cache)
  *   COMBINE_STORES (-1: by output size; 0 | 1: nontemporal / agent-scope stores for the combine's output)

@@ -274,10 +274,11 @@ __device__ __forceinline__ void walk_copy_entry(const WalkArgs& a, uint32_t entr
 }
 
 // The same for rows of at most 512 bytes: a wavefront moves kPack list entries at once, its lanes
-// split into kPack groups of 64 / kPack, so that no half of it idles.  Entry, range checks and
-// addresses are per lane here (the groups of a wavefront differ in them); `candidate` is the lane's
-// list entry and `vector` its 16-byte vector of the row.
-template <int kPack>
+// split into kPack groups of 64 / kPack that move kLaneVectors 16-byte vectors a lane, so that no
+// half of it idles and there are fewer wavefronts to start.  Entry, range checks and addresses are
+// per lane here (the groups of a wavefront differ in them); `candidate` is the lane's list entry
+// and `vector` the first 16-byte vector of the row it moves.
+template <int kPack, int kLaneVectors>
 __device__ __forceinline__ void walk_copy_packed(const WalkArgs& a, uint32_t entries, uint32_t candidate, uint32_t vector) {
     if (candidate >= entries)
         return;
@@ -288,10 +289,23 @@ __device__ __forceinline__ void walk_copy_packed(const WalkArgs& a, uint32_t ent
     if (out_row >= a.out_rows || source >= a.source_limit || vector * 16u >= a.row_bytes)
         return;
     const uint32_t token = fast_divide(source, a.topk_magic, a.topk_shift);
-    const u32x4 data = *reinterpret_cast<const u32x4*>(reinterpret_cast<const char*>(a.x) + static_cast<uint64_t>(token) * a.row_bytes + vector * 16u);
+    const char* from = reinterpret_cast<const char*>(a.x) + static_cast<uint64_t>(token) * a.row_bytes;
+    char* to = reinterpret_cast<char*>(a.recv_x) + static_cast<uint64_t>(out_row) * a.row_bytes;
+    constexpr uint32_t kStride = (kWave / kPack) * 16u;
+    u32x4 data[kLaneVectors];
+#pragma unroll
+    for (int s = 0; s < kLaneVectors; ++s) {
+        const uint32_t at_bytes = vector * 16u + s * kStride;
+        data[s] = *reinterpret_cast<const u32x4*>(from + (at_bytes < a.row_bytes ? at_bytes : 0u));
+    }
     if (vector == a.weight_lane)
         a.recv_weights[out_row] = a.weights[source];
-    store_vec<true>(reinterpret_cast<u32x4*>(reinterpret_cast<char*>(a.recv_x) + static_cast<uint64_t>(out_row) * a.row_bytes + vector * 16u), data);
+#pragma unroll
+    for (int s = 0; s < kLaneVectors; ++s) {
+        const uint32_t at_bytes = vector * 16u + s * kStride;
+        if (at_bytes < a.row_bytes)
+            store_vec<true>(reinterpret_cast<u32x4*>(to + at_bytes), data[s]);
+    }
 }
 
 // One workgroup's turn at the slot-order walk; `block` is its position in the walk.
@@ -305,10 +319,9 @@ __device__ __forceinline__ void walk_copy_packed(const WalkArgs& a, uint32_t ent
 // workgroups beyond it leave at once, and where it is larger they take more than one turn.
 template <int kPieces, int kSpan, bool kDeviceCount, bool kPrefetch>
 __device__ __forceinline__ void walk_copy(const WalkArgs& a, uint32_t entries, uint32_t segment_entries, uint32_t block) {
-    // kPieces -2 / -4: rows of one piece that fill half / a quarter of a wavefront, two / four entries a wavefront
+    // kPieces -4 / -8: rows of at most 512 / 256 bytes, four / eight entries a wavefront, kSpan vectors a lane
     constexpr int kPack = kPieces < 0 ? -kPieces : 1;
     constexpr int kRowPieces = kPieces < 0 ? 1 : kPieces;
-    static_assert(kPack == 1 || kSpan == 1, "packed rows are single chunks");
     // the entry of this lane within its workgroup and the first 16-byte vector of the row it moves
     uint32_t in_block = 0, lane_vector;
     if (kPieces == 0) {
@@ -327,7 +340,7 @@ __device__ __forceinline__ void walk_copy(const WalkArgs& a, uint32_t entries, u
         if (kPack == 1)
             walk_copy_entry<kSpan>(a, entries, candidate, lane_vector);
         else
-            walk_copy_packed<kPack>(a, entries, candidate, lane_vector);
+            walk_copy_packed<kPack, kSpan>(a, entries, candidate, lane_vector);
         return;
     }
     const uint32_t segment = fast_divide(block, a.segment_magic, a.segment_shift);
@@ -361,7 +374,7 @@ __device__ __forceinline__ void walk_copy(const WalkArgs& a, uint32_t entries, u
             if (kPack == 1)
                 walk_copy_entry<kSpan>(a, entries, segment_first + in_segment, lane_vector);
             else
-                walk_copy_packed<kPack>(a, entries, segment_first + in_segment, lane_vector);
+                walk_copy_packed<kPack, kSpan>(a, entries, segment_first + in_segment, lane_vector);
         }
         return;
     }
@@ -369,7 +382,7 @@ __device__ __forceinline__ void walk_copy(const WalkArgs& a, uint32_t entries, u
         if (kPack == 1)
             walk_copy_entry<kSpan>(a, entries, segment_first + in_segment, lane_vector);
         else
-            walk_copy_packed<kPack>(a, entries, segment_first + in_segment, lane_vector);
+            walk_copy_packed<kPack, kSpan>(a, entries, segment_first + in_segment, lane_vector);
     }
 }
 
@@ -380,8 +393,8 @@ __device__ __forceinline__ void walk_copy(const WalkArgs& a, uint32_t entries, u
 // no copy work.
 //   kPieces 0 : one workgroup a list entry, one wavefront a piece of the row (rows of 5 to 16 pieces)
 //   kPieces 1..4 : rows of that many pieces, rows_per_block entries a workgroup
-//   kPieces -2, -4 : rows of up to 512 / 256 bytes, two / four entries a wavefront
-//   kSpan   : 1 KiB chunks a wavefront moves (a piece)
+//   kPieces -4, -8 : rows of up to 512 / 256 bytes, four / eight entries a wavefront
+//   kSpan   : 1 KiB chunks a wavefront moves (a piece); with packed rows, 16-byte vectors a lane moves
 template <int kPieces, int kSpan, bool kDeviceCount, bool kPrefetch>
 __global__ void __launch_bounds__(1024) dispatch_walk_kernel(const WalkArgs a) {
     NANOEP_FETCH_ARGS_4(a.x, a.recv_x, a.slot_order, a.entries);
@@ -568,18 +581,28 @@ int nanoep_dispatch(const void* x, const float* weights, const int32_t* recv_met
             slot_order_entries = expected < most ? expected : most;
         }
         // Rows of up to four pieces share a workgroup (kPieces of the kernel); longer rows take one each.
-        const int kernel_pieces = pieces <= 4 ? pieces : 0;
+        // Rows of at most 512 bytes fill half a wavefront or less: the lanes of a wavefront then split
+        // into four or eight groups that move one list entry each, a lane one or two 16-byte vectors of
+        // it (up to 128 bytes: 8 entries x 1 vector; up to 256: 8 x 2; up to 512: 4 x 2).  Sources from
+        // HBM / cache resident, one entry a wavefront -> packed: 65536 x 256 top-8 75.1 -> 58.3 us /
+        // 61.3 -> 46.3; 65536 x 192 66.4 -> 46.5 / 57.6 -> 31.1; 65536 x 128 57.6 -> 33.0 / 51.8 -> 24.5;
+        // 65536 x 64 top-4 31.5 -> 10.6 / 29.9 -> 8.3.  (Two entries of 32 lanes x 1 vector at 512-byte
+        // rows: 64.2 / 45.5; the same split for rows of 1 KiB and more loses 3 to 10 %.)
+        // NANOEP_DISPATCH_PACK=1 keeps one entry a wavefront.
+        int pack = 1, lane_vectors = 1;
+        if (row_chunks == 1 && vectors <= kWave / 2 && tuning.dispatch_pack != 1) {
+            pack = vectors <= kWave / 4 ? 8 : 4;
+            lane_vectors = vectors <= kWave / 8 ? 1 : 2;
+        }
+        const int walk_pieces = pack > 1 ? 1 : pieces;
+        const int kernel_pieces = walk_pieces <= 4 ? walk_pieces : 0;
         int rows_per_block = 1;
         if (kernel_pieces != 0) {
             rows_per_block = tuning.rows_per_block;
-            if (rows_per_block < 1 || rows_per_block * pieces > kMaxWavesPerBlock)
-                rows_per_block = default_walk_rows(pieces);
+            if (rows_per_block < 1 || rows_per_block * walk_pieces > kMaxWavesPerBlock)
+                rows_per_block = default_walk_rows(walk_pieces);
         }
-        const int64_t waves = static_cast<int64_t>(pieces) * rows_per_block;
-        // Rows of at most 512 / 256 bytes fill half / a quarter of a wavefront: two / four list entries a
-        // wavefront then (65536 x 256 top-8: 75.1 -> 64.1 us with sources from HBM, 61.3 -> 45.4 with cache-resident
-        // ones; 65536 x 128: 57.6 -> 36.7 / 51.8 -> 24.2).  NANOEP_DISPATCH_PACK=1 keeps one entry a wavefront.
-        const int pack = pieces != 1 || span != 1 || tuning.dispatch_pack == 1 ? 1 : vectors <= kWave / 4 ? 4 : vectors <= kWave / 2 ? 2 : 1;
+        const int64_t waves = static_cast<int64_t>(walk_pieces) * rows_per_block;
         const int64_t entries_per_block = static_cast<int64_t>(rows_per_block) * pack;
         const int64_t copy_blocks = (slot_order_entries + entries_per_block - 1) / entries_per_block;
         const int64_t pad_groups_per_expert = (pad_per_expert + waves - 1) / waves;
@@ -674,11 +697,14 @@ int nanoep_dispatch(const void* x, const float* weights, const int32_t* recv_met
             NANOEP_LAUNCH_WALK(PIECES, 1); \
     } while (0)
         switch (pack > 1 ? -pack : kernel_pieces) {
-            case -4:
-                NANOEP_LAUNCH_WALK(-4, 1);
+            case -8:
+                if (lane_vectors == 2)
+                    NANOEP_LAUNCH_WALK(-8, 2);
+                else
+                    NANOEP_LAUNCH_WALK(-8, 1);
                 break;
-            case -2:
-                NANOEP_LAUNCH_WALK(-2, 1);
+            case -4:
+                NANOEP_LAUNCH_WALK(-4, 2);
                 break;
             case 1:
                 NANOEP_LAUNCH_WALK_PIECES(1);

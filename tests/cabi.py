@@ -203,7 +203,7 @@ def dispatch(x, weights, metadata, counts, num_local_experts, alignment, expand,
     rows=n asks for n list entries a workgroup of that walk (honoured for rows of up to four pieces while
     the workgroup stays within 16 wavefronts).  prefetch=0|1 forbids or asks for that walk's window-wise
     source prefetch.  pack=1 keeps one list entry a wavefront for rows of at most 512 bytes (the library
-    packs two or four).
+    packs four or eight).
     """
     recv_metadata, expert_counts, expert_offsets, dst_slots = metadata[0], metadata[1], metadata[2], metadata[3]
     received, capacity = counts[0], counts[1]

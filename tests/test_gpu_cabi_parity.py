@@ -120,7 +120,7 @@ def run_dispatch_combine(device, idx, hidden, experts, alignment, expand, zero_p
                     )
                     assert torch.equal(fetched_x.view(torch.int16), got_x.view(torch.int16))
                     assert fetched_w is None or torch.equal(fetched_w.view(torch.int32), got_w.view(torch.int32))
-        # ... so must rows of at most 512 bytes with one list entry a wavefront instead of two or four
+        # ... so must rows of at most 512 bytes with one list entry a wavefront instead of four or eight
         if hidden <= 256:
             for order_count in ("exact", "device"):
                 for rows in (None, 3):
