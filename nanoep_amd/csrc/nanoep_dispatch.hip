@@ -234,6 +234,13 @@ __device__ __forceinline__ void walk_gap_rows(const WalkArgs& a, uint32_t xcd, u
 // itself).  What it costs otherwise is one more L2 read per source row.
 constexpr int kPrefetchLoads = 4;
 
+// A uniform value as the compiler's vector value: what is computed from it runs on the vector unit.
+__device__ __forceinline__ uint32_t vector_copy(uint32_t uniform) {
+    uint32_t value;
+    asm("v_mov_b32 %0, %1" : "=v"(value) : "s"(uniform));
+    return value;
+}
+
 // One wavefront's copy: list entry `candidate`, the piece of its row that starts at 16-byte vector
 // `lane_vector` of this lane.
 template <int kSpan>
@@ -250,10 +257,13 @@ __device__ __forceinline__ void walk_copy_entry(const WalkArgs& a, uint32_t entr
     asm volatile("");
     if (source >= a.source_limit)
         return;
-    const uint32_t token = fast_divide(source, a.topk_magic, a.topk_shift);
-    const char* from = reinterpret_cast<const char*>(a.x) + static_cast<uint64_t>(token) * a.row_bytes;
-    char* to = reinterpret_cast<char*>(a.recv_x) + static_cast<uint64_t>(out_row) * a.row_bytes;
+    // From here on the arithmetic is the vector unit's: the scalar unit is shared by all wavefronts of
+    // a compute unit and is what these short wavefronts queue for.
+    const uint32_t source_v = vector_copy(source), out_row_v = vector_copy(out_row);
+    const uint32_t token = fast_divide(source_v, a.topk_magic, a.topk_shift);
     const uint32_t lane_bytes = lane_vector * 16u;
+    const char* from = reinterpret_cast<const char*>(a.x) + static_cast<uint64_t>(token) * a.row_bytes;
+    char* to = reinterpret_cast<char*>(a.recv_x) + static_cast<uint64_t>(out_row_v) * a.row_bytes;
     u32x4 data[kSpan];
 #pragma unroll
     for (int s = 0; s < kSpan; ++s) {
@@ -264,7 +274,7 @@ __device__ __forceinline__ void walk_copy_entry(const WalkArgs& a, uint32_t entr
     // the entry's weight rides with the first lane of its row while the payload is in flight
     // (weight_lane is no lane at all when there are no weights to move)
     if (lane_vector == a.weight_lane)
-        a.recv_weights[out_row] = a.weights[source];
+        a.recv_weights[out_row_v] = a.weights[source_v];
 #pragma unroll
     for (int s = 0; s < kSpan; ++s) {
         const uint32_t at_bytes = lane_bytes + s * (kWave * 16u);
@@ -364,7 +374,7 @@ __device__ __forceinline__ void walk_copy(const WalkArgs& a, uint32_t entries, u
             for (int u = 0; u < kPrefetchLoads; ++u)
                 asm volatile("" ::"v"(fetched[u].x), "v"(fetched[u].y), "v"(fetched[u].z), "v"(fetched[u].w));
         }
-        return;
+        __builtin_amdgcn_endpgm();
     }
     const uint32_t copy_block = within - a.prefetch_blocks;
     uint32_t in_segment = kPieces == 0 ? copy_block : copy_block * a.rows_per_block + in_block;
@@ -402,8 +412,10 @@ __global__ void __launch_bounds__(1024) dispatch_walk_kernel(const WalkArgs a) {
     NANOEP_FETCH_ARGS_4(a.topk_magic, a.topk_shift, a.xcd_count, a.xcd_magic);
     NANOEP_FETCH_ARGS_4(a.xcd_shift, a.rows_per_block, a.weight_lane, a.weights);
     NANOEP_FETCH_ARGS_2(a.recv_weights, a.weights);
-    if (kPrefetch)
+    if (kPrefetch) {
         NANOEP_FETCH_ARGS_4(a.segment_blocks, a.segment_magic, a.segment_shift, a.prefetch_blocks);
+        NANOEP_FETCH_ARGS_2(a.segment_entries, a.segment_copy_entries);
+    }
     const uint32_t index_in_xcd = fast_divide(blockIdx.x, a.xcd_magic, a.xcd_shift);
     const uint32_t xcd = blockIdx.x - index_in_xcd * a.xcd_count;
     if (!kDeviceCount || kPrefetch) {
@@ -420,7 +432,7 @@ __global__ void __launch_bounds__(1024) dispatch_walk_kernel(const WalkArgs a) {
             segment_entries = fast_divide(entries + a.windows - 1, a.windows_magic, a.windows_shift);
         }
         walk_copy<kPieces, kSpan, kDeviceCount, kPrefetch>(a, entries, segment_entries, xcd * a.copy_per_xcd + index_in_xcd);
-        return;
+        __builtin_amdgcn_endpgm();
     }
     // The entry count is on the device and the walk is the plain list: the live list may be shorter
     // than what the grid was sized for (the rest of the grid leaves at once) or longer (workgroups
