@@ -26,7 +26,7 @@ constexpr SwitchSlot kSwitches[] = {
     {"RECALL_ORDER", &Tuning::recall_order},         {"FRESH_OUTPUTS", &Tuning::fresh_outputs},
     {"REBUILD_ORDER", &Tuning::rebuild_order},       {"XCDS", &Tuning::xcds},
     {"L2_BYTES", &Tuning::l2_bytes},                 {"DISPATCH_PREFETCH", &Tuning::dispatch_prefetch},
-    {"COMBINE_STORES", &Tuning::combine_stores},     {"DISPATCH_PACK", &Tuning::dispatch_pack},
+    {"COMBINE_STORES", &Tuning::combine_stores},     {"DISPATCH_PACK", &Tuning::dispatch_pack}, {"COMBINE_UNITS", &Tuning::combine_units},
 };
 constexpr int kSwitchCount = sizeof(kSwitches) / sizeof(kSwitches[0]);
 

@@ -10,6 +10,10 @@ constexpr int kCombineMultipleReduction = 1;  // round sums of two or more rows 
 constexpr int kCombineAgentStores = 2;        // agent-scope stores for the output instead of nontemporal ones
 // largest output (bytes) that is written with agent-scope stores
 constexpr int64_t kAgentStoreOutputBytes = int64_t{88} << 20;
+// most rows a token of combine_held_kernel, and the wavefronts of one launch it is sized for (the
+// device holds about that many of them at once: 256 compute units x 16)
+constexpr int kHeldRows = 8;
+constexpr int64_t kHeldWavefronts = 4096;
 
 __device__ __forceinline__ float bf16_low(uint32_t packed) { return __uint_as_float(packed << 16); }
 __device__ __forceinline__ float bf16_high(uint32_t packed) { return __uint_as_float(packed & 0xffff0000u); }
@@ -235,6 +239,112 @@ __global__ void __launch_bounds__(1024) combine_few_rows_kernel(const u32x4* __r
     }
 }
 
+// Expanded layout with the slot table at hand and at most eight rows a token: one wavefront (a
+// workgroup of its own) produces the same 1 KiB chunk of the output rows of kUnits consecutive
+// tokens and holds the packed sums back in registers until the last one is done.  The units are
+// sized so that all wavefronts of the launch are resident at once wherever the batch allows it: the
+// whole device then reads first and writes last, and HBM sees the output as one burst behind the
+// gather instead of a write among every eight reads.  A token's eight rows are fetched back to back (a
+// masked k re-reads row 0 so that the loads stay unconditional).
+template <int kUnits>
+__global__ void __launch_bounds__(kWave) combine_held_kernel(const u32x4* __restrict__ y,              // [C][vectors]
+                                                             const float* __restrict__ weights,       // [C] or null
+                                                             const u32x4* __restrict__ bias,          // [T][vectors] or null
+                                                             const int32_t* __restrict__ token_slots,  // [T][K]
+                                                             u32x4* __restrict__ out_x,               // [T][vectors]
+                                                             float* __restrict__ out_weights,         // [T][K] or null
+                                                             uint32_t tokens,
+                                                             uint32_t y_rows,
+                                                             uint32_t chunks,
+                                                             uint32_t chunks_magic,  // fast divisor by chunks
+                                                             uint32_t chunks_shift,
+                                                             uint32_t vectors,
+                                                             uint32_t topk,
+                                                             int flags,  // kCombineMultipleReduction | kCombineAgentStores
+                                                             uint32_t topk_magic,  // fast divisor by K
+                                                             uint32_t topk_shift,
+                                                             uint32_t side_blocks) {
+    NANOEP_FETCH_ARGS_4(y, token_slots, out_x, bias);
+    NANOEP_FETCH_ARGS_4(tokens, y_rows, chunks, chunks_magic);
+    NANOEP_FETCH_ARGS_4(chunks_shift, vectors, topk, flags);
+    const uint32_t lane = threadIdx.x;
+    if (blockIdx.x < side_blocks) {
+        // weights back to their (token, k): one lane each, in workgroups of their own at the front
+        // of the grid (on a payload wavefront they are one more round trip)
+        const uint32_t flat = blockIdx.x * kWave + lane;
+        if (fast_divide(flat, topk_magic, topk_shift) >= tokens)
+            return;
+        const int32_t slot = token_slots[flat];
+        out_weights[flat] = slot >= 0 && static_cast<uint32_t>(slot) < y_rows ? weights[slot] : 0.0f;
+        return;
+    }
+    const uint32_t payload_block = blockIdx.x - side_blocks;
+    const uint32_t group = fast_divide(payload_block, chunks_magic, chunks_shift);
+    const uint32_t chunk = payload_block - group * chunks;
+    const uint32_t vector = chunk * kWave + lane;
+    const bool in_row = vector < vectors;
+    // lanes past the end of a short row re-read vector 0 instead of branching around the loads
+    const uint32_t load_vector = in_row ? vector : 0u;
+    const uint32_t first = group * kUnits;
+    u32x4 packed[kUnits];
+#pragma unroll
+    for (int u = 0; u < kUnits; ++u) {
+        // (a launch's last wavefronts may run past the last token: they sum its row again and drop it)
+        const uint32_t token = first + u < tokens ? first + u : tokens - 1;
+        // lane k fetches the token's k-th slot; the slots are broadcast to scalars below
+        int slot = -1;
+        if (lane < topk)
+            slot = token_slots[static_cast<uint64_t>(token) * topk + lane];
+        const bool valid = slot >= 0 && static_cast<uint32_t>(slot) < y_rows;
+        const uint32_t valid_mask = static_cast<uint32_t>(__ballot(valid));
+        u32x4 bias_data = {0u, 0u, 0u, 0u};
+        if (bias != nullptr)
+            bias_data = load_vec<true>(bias + static_cast<uint64_t>(token) * vectors + load_vector);
+        float acc[8] = {0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f};
+        if (valid_mask != 0) {
+            u32x4 data[kHeldRows];
+#pragma unroll
+            for (int k = 0; k < kHeldRows; ++k) {
+                uint64_t source_row = 0;
+                if ((valid_mask >> k) & 1)
+                    source_row = static_cast<uint32_t>(__builtin_amdgcn_readlane(slot, k));
+                data[k] = load_vec<true>(y + source_row * vectors + load_vector);
+            }
+#pragma unroll
+            for (int k = 0; k < kHeldRows; ++k)
+                if ((valid_mask >> k) & 1)
+                    accumulate(acc, data[k]);
+        }
+        if ((flags & kCombineMultipleReduction) && __popc(valid_mask) >= 2) {
+#pragma unroll
+            for (int j = 0; j < 8; ++j)
+                acc[j] = 0.0f + __uint_as_float(bf16_round(acc[j]) << 16);
+        }
+        if (bias != nullptr)
+            accumulate(acc, bias_data);
+        packed[u].x = bf16_round(acc[0]) | (bf16_round(acc[1]) << 16);
+        packed[u].y = bf16_round(acc[2]) | (bf16_round(acc[3]) << 16);
+        packed[u].z = bf16_round(acc[4]) | (bf16_round(acc[5]) << 16);
+        packed[u].w = bf16_round(acc[6]) | (bf16_round(acc[7]) << 16);
+        // the packed row is pinned here: left to itself the compiler keeps every token's eight fp32 sums
+        // and rounds them all at the end, which doubles the registers held and costs the compute units
+        // a quarter of their resident wavefronts
+        asm volatile("" : "+v"(packed[u].x), "+v"(packed[u].y), "+v"(packed[u].z), "+v"(packed[u].w)::"memory");
+    }
+    if (!in_row)
+        return;
+#pragma unroll
+    for (int u = 0; u < kUnits; ++u) {
+        if (first + u < tokens) {
+            u32x4* to = out_x + static_cast<uint64_t>(first + u) * vectors + vector;
+            if (flags & kCombineAgentStores)
+                store_vec_agent(to, packed[u]);
+            else
+                store_vec<true>(to, packed[u]);
+        }
+    }
+}
+
 // Compact layout: a token has one received row, so the combine is a row copy through fp32
 // (0.0f + x, which turns -0 into +0 and quiets NaNs, then the bias) with holes: tokens that were
 // not sent get 0 (+bias).  Plain launch order, nothing but the copy in the kernel.
@@ -376,6 +486,46 @@ int nanoep_combine(const void* y, const float* weights, const void* bias, const 
             static_cast<uint32_t>(recv_count), blocking.parts, parts_divisor.magic, parts_divisor.shift,
             blocking.chunks_per_block, blocking.rows_per_block, static_cast<uint32_t>(vectors), static_cast<uint32_t>(chunks),
             static_cast<uint32_t>(num_topk), topk_divisor.magic, topk_divisor.shift, static_cast<uint32_t>(side_blocks));
+        NANOEP_HIP_TRY(hipGetLastError());
+        return NANOEP_OK;
+    }
+    // Five to eight rows a token with the slot table at hand: wavefronts that hold the sums of 2, 4, 8
+    // or 16 tokens back and write them at their end, the fewest for which one launch has at most
+    // kHeldWavefronts wavefronts.  Against one (token, chunk) a wavefront, sources from HBM: 4096 x 7168
+    // top-8 78.1 -> 74.7 us (16 tokens a wavefront), 8192 x 2048 49.2 -> 47.1 (8), 2048 x 7168 39.9 ->
+    // 38.1 (8), 4096 x 2048 24.0 -> 22.9 (4), 512 x 7168 12.3 -> 11.4 (2), 16384 x 7168 321 -> 309 (16);
+    // too many tokens a wavefront leave compute units idle (1024 x 7168: 4 tokens 20.4 us, 8 tokens
+    // 22.9, 16 tokens 32.2).  With two to four rows a token the held sums lose to
+    // combine_few_rows_kernel (4096 x 4096 top-2: 17.3 us against 18.1 to 30.5).
+    // NANOEP_COMBINE_UNITS=1 keeps one token a wavefront, 2|4|8|16 asks for that many.
+    int held_units = 0;
+    if (direct && num_topk > 4 && num_topk <= kHeldRows && tuning.combine_units != 1) {
+        const int64_t work = num_tokens * chunks;
+        held_units = work <= 2 * kHeldWavefronts ? 2 : work <= 4 * kHeldWavefronts ? 4 : work <= 8 * kHeldWavefronts ? 8 : 16;
+        if (tuning.combine_units == 2 || tuning.combine_units == 4 || tuning.combine_units == 8 || tuning.combine_units == 16)
+            held_units = tuning.combine_units;
+    }
+    if (held_units > 0) {
+        const FastDivisor chunks_divisor = make_fast_divisor(static_cast<uint32_t>(chunks));
+        const int64_t held_side_blocks = (side_lanes + kWave - 1) / kWave;
+        const int64_t held_blocks = (num_tokens + held_units - 1) / held_units * chunks + held_side_blocks;
+        if (held_blocks >= (int64_t{1} << 31))
+            return NANOEP_ERR_INVALID_ARGUMENT;
+#define NANOEP_LAUNCH_HELD(UNITS)                                                                                      \
+    combine_held_kernel<UNITS><<<dim3(static_cast<unsigned>(held_blocks)), dim3(kWave), 0, stream>>>(                 \
+        static_cast<const u32x4*>(y), weights, static_cast<const u32x4*>(bias), token_slots, static_cast<u32x4*>(out_x), \
+        out_weights, static_cast<uint32_t>(num_tokens), static_cast<uint32_t>(y_rows), static_cast<uint32_t>(chunks),   \
+        chunks_divisor.magic, chunks_divisor.shift, static_cast<uint32_t>(vectors), static_cast<uint32_t>(num_topk), flags, \
+        topk_divisor.magic, topk_divisor.shift, static_cast<uint32_t>(held_side_blocks))
+        if (held_units == 16)
+            NANOEP_LAUNCH_HELD(16);
+        else if (held_units == 8)
+            NANOEP_LAUNCH_HELD(8);
+        else if (held_units == 4)
+            NANOEP_LAUNCH_HELD(4);
+        else
+            NANOEP_LAUNCH_HELD(2);
+#undef NANOEP_LAUNCH_HELD
         NANOEP_HIP_TRY(hipGetLastError());
         return NANOEP_OK;
     }

@@ -245,9 +245,11 @@ def dispatch(x, weights, metadata, counts, num_local_experts, alignment, expand,
 
 
 def combine(y, weights, bias, metadata, counts, expand, *, multiple_reduction=False, num_cus=0, poison=None, use_table=True,
-            stores=None):
+            stores=None, units=None):
     """Returns (out_x [T,H], out_weights [T,K] | None) through nanoep_combine.  stores=0|1 asks for
-    nontemporal / agent-scope stores of the output rows (the library picks by output size)."""
+    nontemporal / agent-scope stores of the output rows (the library picks by output size);
+    units=1|2|4|8|16 for that many tokens a wavefront where the library has a choice (five to eight
+    rows a token with the slot table; it picks by batch size)."""
     recv_metadata, dst_slots = metadata[0], metadata[3]
     tokens = dst_slots.shape[0]
     topk = recv_metadata.shape[1] - 2
@@ -259,7 +261,7 @@ def combine(y, weights, bias, metadata, counts, expand, *, multiple_reduction=Fa
         for tensor in (out_x, out_w):
             if tensor is not None and tensor.numel():
                 tensor.view(torch.uint8).fill_(poison)
-    with forced_tuning({"COMBINE_STORES": stores}):
+    with forced_tuning({"COMBINE_STORES": stores, "COMBINE_UNITS": units}):
         check(
             lib().nanoep_combine(
                 ptr(y), ptr(weights), ptr(bias), ptr(recv_metadata), ptr(dst_slots), ptr(token_slots_of(metadata, use_table)), counts[0],

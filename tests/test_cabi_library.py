@@ -99,7 +99,7 @@ def test_tuning_switches_are_set_through_the_abi_and_read_from_the_environment_o
     library = cabi.lib()
     assert cabi.get_tuning("WINDOW_TOKENS") == 0 and cabi.get_tuning("DISPATCH_ORDER") == -1 and cabi.get_tuning("XCDS") == 0
     assert cabi.get_tuning("DISPATCH_PREFETCH") == -1 and cabi.get_tuning("COMBINE_STORES") == -1 and cabi.get_tuning("DISPATCH_SPAN") == 0
-    assert cabi.get_tuning("DISPATCH_PACK") == 0
+    assert cabi.get_tuning("DISPATCH_PACK") == 0 and cabi.get_tuning("COMBINE_UNITS") == 0
     value = ctypes.c_int(0)
     assert library.nanoep_get_tuning(b"NO_SUCH_SWITCH", ctypes.byref(value)) == 1
     assert library.nanoep_set_tuning(b"NO_SUCH_SWITCH", 3) == 1 and library.nanoep_set_tuning(None, 3) == 1

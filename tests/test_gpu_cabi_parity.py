@@ -194,6 +194,18 @@ def run_dispatch_combine(device, idx, hidden, experts, alignment, expand, zero_p
             assert_bits_equal(stored_out, want_out, f"combine x multi={multi} stores={stores}")
             if weighted:
                 assert_bits_equal(stored_ow, want_ow, f"combine weights stores={stores}")
+        # one, two, four, eight or sixteen tokens a wavefront (a choice only with five to eight rows a
+        # token; the library picks by batch size, and small test batches would all take two)
+        if expand and 4 < topk <= 8:
+            for units in (1, 2, 4, 8, 16):
+                held_out, held_ow = cabi.combine(
+                    y.to(device), None if yw is None else yw.to(device), None if bias is None else bias.to(device), metadata,
+                    counts, expand, multiple_reduction=multi, num_cus=num_cus, poison=POISON, units=units,
+                )
+                torch.cuda.synchronize()
+                assert_bits_equal(held_out, want_out, f"combine x multi={multi} units={units}")
+                if weighted:
+                    assert_bits_equal(held_ow, want_ow, f"combine weights units={units}")
         if expand:
             plain_out, plain_ow = cabi.combine(
                 y.to(device), None if yw is None else yw.to(device), None if bias is None else bias.to(device), metadata,
