@@ -10,10 +10,8 @@ constexpr int kCombineMultipleReduction = 1;  // round sums of two or more rows 
 constexpr int kCombineAgentStores = 2;        // agent-scope stores for the output instead of nontemporal ones
 // largest output (bytes) that is written with agent-scope stores
 constexpr int64_t kAgentStoreOutputBytes = int64_t{88} << 20;
-// most rows a token of combine_held_kernel, and the wavefronts of one launch it is sized for (the
-// device holds about that many of them at once: 256 compute units x 16)
+// most rows a token of combine_held_kernel
 constexpr int kHeldRows = 8;
-constexpr int64_t kHeldWavefronts = 4096;
 
 __device__ __forceinline__ float bf16_low(uint32_t packed) { return __uint_as_float(packed << 16); }
 __device__ __forceinline__ float bf16_high(uint32_t packed) { return __uint_as_float(packed & 0xffff0000u); }
@@ -263,10 +261,12 @@ __global__ void __launch_bounds__(kWave) combine_held_kernel(const u32x4* __rest
                                                              int flags,  // kCombineMultipleReduction | kCombineAgentStores
                                                              uint32_t topk_magic,  // fast divisor by K
                                                              uint32_t topk_shift,
-                                                             uint32_t side_blocks) {
+                                                             uint32_t side_blocks,
+                                                             uint32_t units) {  // tokens a wavefront, at most kUnits
     NANOEP_FETCH_ARGS_4(y, token_slots, out_x, bias);
     NANOEP_FETCH_ARGS_4(tokens, y_rows, chunks, chunks_magic);
     NANOEP_FETCH_ARGS_4(chunks_shift, vectors, topk, flags);
+    NANOEP_FETCH_ARGS_2(side_blocks, units);
     const uint32_t lane = threadIdx.x;
     if (blockIdx.x < side_blocks) {
         // weights back to their (token, k): one lane each, in workgroups of their own at the front
@@ -285,12 +285,15 @@ __global__ void __launch_bounds__(kWave) combine_held_kernel(const u32x4* __rest
     const bool in_row = vector < vectors;
     // lanes past the end of a short row re-read vector 0 instead of branching around the loads
     const uint32_t load_vector = in_row ? vector : 0u;
-    const uint32_t first = group * kUnits;
+    const uint32_t first = group * units;
+    // this wavefront's tokens: first .. first + count - 1
+    const uint32_t count = first + units <= tokens ? units : tokens - first;
     u32x4 packed[kUnits];
 #pragma unroll
     for (int u = 0; u < kUnits; ++u) {
-        // (a launch's last wavefronts may run past the last token: they sum its row again and drop it)
-        const uint32_t token = first + u < tokens ? first + u : tokens - 1;
+        if (static_cast<uint32_t>(u) >= count)
+            continue;
+        const uint32_t token = first + u;
         // lane k fetches the token's k-th slot; the slots are broadcast to scalars below
         int slot = -1;
         if (lane < topk)
@@ -335,7 +338,7 @@ __global__ void __launch_bounds__(kWave) combine_held_kernel(const u32x4* __rest
         return;
 #pragma unroll
     for (int u = 0; u < kUnits; ++u) {
-        if (first + u < tokens) {
+        if (static_cast<uint32_t>(u) < count) {
             u32x4* to = out_x + static_cast<uint64_t>(first + u) * vectors + vector;
             if (flags & kCombineAgentStores)
                 store_vec_agent(to, packed[u]);
@@ -489,20 +492,33 @@ int nanoep_combine(const void* y, const float* weights, const void* bias, const 
         NANOEP_HIP_TRY(hipGetLastError());
         return NANOEP_OK;
     }
-    // Five to eight rows a token with the slot table at hand: wavefronts that hold the sums of 2, 4, 8
-    // or 16 tokens back and write them at their end, the fewest for which one launch has at most
-    // kHeldWavefronts wavefronts.  Against one (token, chunk) a wavefront, sources from HBM: 4096 x 7168
-    // top-8 78.1 -> 74.7 us (16 tokens a wavefront), 8192 x 2048 49.2 -> 47.1 (8), 2048 x 7168 39.9 ->
-    // 38.1 (8), 4096 x 2048 24.0 -> 22.9 (4), 512 x 7168 12.3 -> 11.4 (2), 16384 x 7168 321 -> 309 (16);
-    // too many tokens a wavefront leave compute units idle (1024 x 7168: 4 tokens 20.4 us, 8 tokens
-    // 22.9, 16 tokens 32.2).  With two to four rows a token the held sums lose to
+    // Five to eight rows a token with the slot table at hand: wavefronts that hold the sums of 2 to 16
+    // tokens back and write them at their end; as many tokens a wavefront as it takes for the launch to
+    // fit what the device holds at once with the registers of sixteen held rows (16 wavefronts a
+    // compute unit), or a whole multiple of that when sixteen tokens a wavefront are not enough: a
+    // launch a little larger than what is resident waits for its last few wavefronts with the device
+    // idle (5120 x 7168 top-8 with sixteen tokens a wavefront: 104.7 us against 95.7 with one and 93.1
+    // with nine; 4096 x 7168 with fourteen, six wavefronts too many: 78.8 against 74.1 with fifteen).  Against one
+    // (token, chunk) a wavefront, sources from HBM: 4096 x 7168 top-8 78.2 -> 73.7 us, 8192 x 2048
+    // 49.1 -> 47.6, 2048 x 7168 39.9 -> 37.8, 32768 x 1024 89.0 -> 83.4, 32768 x 512 46.1 -> 44.7,
+    // 8192 x 7168 159.2 -> 155.4.  With two to four rows a token the held sums lose to
     // combine_few_rows_kernel (4096 x 4096 top-2: 17.3 us against 18.1 to 30.5).
-    // NANOEP_COMBINE_UNITS=1 keeps one token a wavefront, 2|4|8|16 asks for that many.
+    // NANOEP_COMBINE_UNITS=1 keeps one token a wavefront, 2..16 asks for that many.
     int held_units = 0;
     if (direct && num_topk > 4 && num_topk <= kHeldRows && tuning.combine_units != 1) {
+        // (16 wavefronts a compute unit, of the compute units this call may use)
+        const Topology topology = current_topology(tuning);
+        const int64_t resident = int64_t{16} * (num_cus > 0 ? num_cus : topology.cus);
         const int64_t work = num_tokens * chunks;
-        held_units = work <= 2 * kHeldWavefronts ? 2 : work <= 4 * kHeldWavefronts ? 4 : work <= 8 * kHeldWavefronts ? 8 : 16;
-        if (tuning.combine_units == 2 || tuning.combine_units == 4 || tuning.combine_units == 8 || tuning.combine_units == 16)
+        int64_t rounds = (work + 16 * resident - 1) / (16 * resident);
+        held_units = 16;
+        for (int units = 2; units <= 16; ++units) {
+            if ((num_tokens + units - 1) / units * chunks <= rounds * resident) {
+                held_units = units;
+                break;
+            }
+        }
+        if (tuning.combine_units >= 2 && tuning.combine_units <= 16)
             held_units = tuning.combine_units;
     }
     if (held_units > 0) {
@@ -516,12 +532,12 @@ int nanoep_combine(const void* y, const float* weights, const void* bias, const 
         static_cast<const u32x4*>(y), weights, static_cast<const u32x4*>(bias), token_slots, static_cast<u32x4*>(out_x), \
         out_weights, static_cast<uint32_t>(num_tokens), static_cast<uint32_t>(y_rows), static_cast<uint32_t>(chunks),   \
         chunks_divisor.magic, chunks_divisor.shift, static_cast<uint32_t>(vectors), static_cast<uint32_t>(num_topk), flags, \
-        topk_divisor.magic, topk_divisor.shift, static_cast<uint32_t>(held_side_blocks))
-        if (held_units == 16)
+        topk_divisor.magic, topk_divisor.shift, static_cast<uint32_t>(held_side_blocks), static_cast<uint32_t>(held_units))
+        if (held_units > 8)
             NANOEP_LAUNCH_HELD(16);
-        else if (held_units == 8)
+        else if (held_units > 4)
             NANOEP_LAUNCH_HELD(8);
-        else if (held_units == 4)
+        else if (held_units > 2)
             NANOEP_LAUNCH_HELD(4);
         else
             NANOEP_LAUNCH_HELD(2);

@@ -89,7 +89,7 @@ struct Tuning {
     int dispatch_order = -1;        // DISPATCH_ORDER: 0 forces the token-order walk
     int dispatch_span = 0;          // DISPATCH_SPAN: 1 | 2 | 4 chunks a wavefront of the slot-order walk, 0 = by size
     int dispatch_prefetch = -1;     // DISPATCH_PREFETCH: 0 = no window-wise source prefetch in the slot-order walk
-    int combine_units = 0;          // COMBINE_UNITS: tokens a wavefront of the gather for 5 to 8 rows a token: 1 | 2 | 4 | 8 | 16, 0 = by size
+    int combine_units = 0;          // COMBINE_UNITS: tokens a wavefront of the gather for 5 to 8 rows a token: 1 .. 16, 0 = by size
     int dispatch_pack = 0;          // DISPATCH_PACK: 1 = one list entry a wavefront of the slot-order walk whatever the row length
     int combine_stores = -1;        // COMBINE_STORES: 0 | 1 nontemporal / agent-scope stores for the combine's output, -1 = by size
     int layout_launches = 0;        // LAYOUT_LAUNCHES: 2 | 3 forces the layout plan
