@@ -168,6 +168,21 @@ __device__ __forceinline__ T uniform_load_at(const T* base, uint32_t index) {
     return *(ConstantElement)((ConstantBytes)(base) + index * static_cast<uint32_t>(sizeof(T)));
 }
 
+// A uniform 64-bit load in two halves: begin issues it, end waits for it.  Between the two the value
+// must not be touched; what the wavefront computes meanwhile hides the load's latency (the compiler
+// on its own moves such a load down to its first use).
+// `anchor` is any scalar the following arithmetic starts from: tied to the statement, it keeps that
+// arithmetic behind the load's issue.
+__device__ __forceinline__ int64_t uniform_load_begin(const int64_t* p, uint32_t& anchor) {
+    int64_t value;
+    asm volatile("s_load_dwordx2 %0, %2, 0x0" : "=s"(value), "+s"(anchor) : "s"(p));
+    return value;
+}
+__device__ __forceinline__ int64_t uniform_load_end(int64_t value) {
+    asm volatile("s_waitcnt lgkmcnt(0)" : "+s"(value));
+    return value;
+}
+
 // n / d for n < 2^31 as one 64-bit multiply and shift: magic = ceil(2^shift / d), shift = 31 + ceil(log2 d).
 struct FastDivisor {
     uint32_t magic;

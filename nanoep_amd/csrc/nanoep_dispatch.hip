@@ -416,8 +416,16 @@ __global__ void __launch_bounds__(1024) dispatch_walk_kernel(const WalkArgs a) {
         NANOEP_FETCH_ARGS_4(a.segment_blocks, a.segment_magic, a.segment_shift, a.prefetch_blocks);
         NANOEP_FETCH_ARGS_2(a.segment_entries, a.segment_copy_entries);
     }
-    const uint32_t index_in_xcd = fast_divide(blockIdx.x, a.xcd_magic, a.xcd_shift);
-    const uint32_t xcd = blockIdx.x - index_in_xcd * a.xcd_count;
+    // the live count's load is on every copy wavefront's way to its list entry: it leaves with the
+    // first batch of arguments and is in flight during the index arithmetic below
+    int64_t live = 0;
+    uint32_t block = blockIdx.x;
+    if (kDeviceCount) {
+        NANOEP_FETCH_ARGS_4(a.windows, a.windows_magic, a.windows_shift, a.live_count);
+        live = uniform_load_begin(a.live_count, block);
+    }
+    const uint32_t index_in_xcd = fast_divide(block, a.xcd_magic, a.xcd_shift);
+    const uint32_t xcd = block - index_in_xcd * a.xcd_count;
     if (!kDeviceCount || kPrefetch) {
         // the grid's shape is the host's: with prefetch the segments are the windows of the batch
         if (index_in_xcd >= a.copy_per_xcd) {
@@ -427,7 +435,7 @@ __global__ void __launch_bounds__(1024) dispatch_walk_kernel(const WalkArgs a) {
         uint32_t entries = a.entries, segment_entries = a.segment_entries;
         if (kDeviceCount) {
             // a word that cannot be a count (the layout did not run) walks nothing
-            const int64_t live = uniform_load(a.live_count);
+            live = uniform_load_end(live);
             entries = live >= 0 && live <= static_cast<int64_t>(a.source_limit) ? static_cast<uint32_t>(live) : 0u;
             segment_entries = fast_divide(entries + a.windows - 1, a.windows_magic, a.windows_shift);
         }
@@ -438,7 +446,7 @@ __global__ void __launch_bounds__(1024) dispatch_walk_kernel(const WalkArgs a) {
     // than what the grid was sized for (the rest of the grid leaves at once) or longer (workgroups
     // then take more than one turn, a grid's worth of list positions apart).  A word that cannot be a
     // count (the layout did not run) walks nothing.
-    const int64_t live = uniform_load(a.live_count);
+    live = uniform_load_end(live);
     const uint32_t entries = live >= 0 && live <= static_cast<int64_t>(a.source_limit) ? static_cast<uint32_t>(live) : 0u;
     const uint32_t copy_blocks = kPieces == 0 ? entries : fast_divide(entries + a.rows_per_block - 1, a.rows_magic, a.rows_shift);
     const uint32_t copy_per_xcd = fast_divide(copy_blocks + a.xcd_count - 1, a.xcd_magic, a.xcd_shift);
