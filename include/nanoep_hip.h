@@ -73,7 +73,7 @@ int nanoep_device_topology(int* out_cus, int* out_xcds, int64_t* out_l2_bytes);
  *   DISPATCH_PREFETCH (-1: on; 0: no window-wise source prefetch in that walk, for sources that are
  *                     known to sit in the last-level cache)
  *   COMBINE_STORES (-1: by output size; 0 | 1: nontemporal / agent-scope stores for the combine's output)
- *   COMBINE_UNITS (0: by size; 1 .. 16 tokens a wavefront of the expanded combine with five to eight
+ *   COMBINE_UNITS (0: by size; 1 .. 16 tokens a wavefront of the expanded combine with five or more
  *                     rows a token and the slot table; 1 = the one-token kernel)
  *   LAYOUT_LAUNCHES (0; 2 | 3: layout plan)     WINDOW_TOKENS (0; window of the slot-order list)
  *   RECALL_ORDER, FRESH_OUTPUTS, REBUILD_ORDER (-1; 0 | 1: host-extension policies)

@@ -10,7 +10,7 @@ constexpr int kCombineMultipleReduction = 1;  // round sums of two or more rows 
 constexpr int kCombineAgentStores = 2;        // agent-scope stores for the output instead of nontemporal ones
 // largest output (bytes) that is written with agent-scope stores
 constexpr int64_t kAgentStoreOutputBytes = int64_t{88} << 20;
-// most rows a token of combine_held_kernel
+// rows of a token that combine_held_kernel fetches at a time
 constexpr int kHeldRows = 8;
 
 __device__ __forceinline__ float bf16_low(uint32_t packed) { return __uint_as_float(packed << 16); }
@@ -237,12 +237,12 @@ __global__ void __launch_bounds__(1024) combine_few_rows_kernel(const u32x4* __r
     }
 }
 
-// Expanded layout with the slot table at hand and at most eight rows a token: one wavefront (a
+// Expanded layout with the slot table at hand and five or more rows a token: one wavefront (a
 // workgroup of its own) produces the same 1 KiB chunk of the output rows of kUnits consecutive
 // tokens and holds the packed sums back in registers until the last one is done.  The units are
 // sized so that all wavefronts of the launch are resident at once wherever the batch allows it: the
 // whole device then reads first and writes last, and HBM sees the output as one burst behind the
-// gather instead of a write among every eight reads.  A token's eight rows are fetched back to back (a
+// gather instead of a write among every eight reads.  A token's rows are fetched eight at a time (a
 // masked k re-reads row 0 so that the loads stay unconditional).
 template <int kUnits>
 __global__ void __launch_bounds__(kWave) combine_held_kernel(const u32x4* __restrict__ y,              // [C][vectors]
@@ -304,18 +304,19 @@ __global__ void __launch_bounds__(kWave) combine_held_kernel(const u32x4* __rest
         if (bias != nullptr)
             bias_data = load_vec<true>(bias + static_cast<uint64_t>(token) * vectors + load_vector);
         float acc[8] = {0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f};
-        if (valid_mask != 0) {
+        // eight rows a pass, in ascending k
+        for (uint32_t base = 0; base < (valid_mask != 0 ? topk : 0u); base += kHeldRows) {
             u32x4 data[kHeldRows];
 #pragma unroll
             for (int k = 0; k < kHeldRows; ++k) {
                 uint64_t source_row = 0;
-                if ((valid_mask >> k) & 1)
-                    source_row = static_cast<uint32_t>(__builtin_amdgcn_readlane(slot, k));
+                if ((valid_mask >> (base + k)) & 1)
+                    source_row = static_cast<uint32_t>(__builtin_amdgcn_readlane(slot, (base + k) & (kWave - 1)));
                 data[k] = load_vec<true>(y + source_row * vectors + load_vector);
             }
 #pragma unroll
             for (int k = 0; k < kHeldRows; ++k)
-                if ((valid_mask >> k) & 1)
+                if ((valid_mask >> (base + k)) & 1)
                     accumulate(acc, data[k]);
         }
         if ((flags & kCombineMultipleReduction) && __popc(valid_mask) >= 2) {
@@ -492,7 +493,7 @@ int nanoep_combine(const void* y, const float* weights, const void* bias, const 
         NANOEP_HIP_TRY(hipGetLastError());
         return NANOEP_OK;
     }
-    // Five to eight rows a token with the slot table at hand: wavefronts that hold the sums of 2 to 16
+    // Five or more rows a token with the slot table at hand: wavefronts that hold the sums of 2 to 16
     // tokens back and write them at their end; as many tokens a wavefront as it takes for the launch to
     // fit what the device holds at once with the registers of sixteen held rows (16 wavefronts a
     // compute unit), or a whole multiple of that when sixteen tokens a wavefront are not enough: a
@@ -501,11 +502,12 @@ int nanoep_combine(const void* y, const float* weights, const void* bias, const 
     // with nine; 4096 x 7168 with fourteen, six wavefronts too many: 78.8 against 74.1 with fifteen).  Against one
     // (token, chunk) a wavefront, sources from HBM: 4096 x 7168 top-8 78.2 -> 73.7 us, 8192 x 2048
     // 49.1 -> 47.6, 2048 x 7168 39.9 -> 37.8, 32768 x 1024 89.0 -> 83.4, 32768 x 512 46.1 -> 44.7,
-    // 8192 x 7168 159.2 -> 155.4.  With two to four rows a token the held sums lose to
+    // 8192 x 7168 159.2 -> 155.4; 4096 x 4096 top-16 82.9 -> 79.7, 2048 x 7168 top-12 57.8 -> 55.3.  With
+    // two to four rows a token the held sums lose to
     // combine_few_rows_kernel (4096 x 4096 top-2: 17.3 us against 18.1 to 30.5).
     // NANOEP_COMBINE_UNITS=1 keeps one token a wavefront, 2..16 asks for that many.
     int held_units = 0;
-    if (direct && num_topk > 4 && num_topk <= kHeldRows && tuning.combine_units != 1) {
+    if (direct && num_topk > 4 && num_topk <= 32 && tuning.combine_units != 1) {
         // (16 wavefronts a compute unit, of the compute units this call may use)
         const Topology topology = current_topology(tuning);
         const int64_t resident = int64_t{16} * (num_cus > 0 ? num_cus : topology.cus);

@@ -32,7 +32,7 @@
 //   combine_rows_kernel  : one wavefront per (source token, row chunk): gathers the token's rows in
 //                          ascending k, fp32 accumulate, one round-to-nearest-even bf16 store.
 //   combine_few_rows_kernel : the same for K <= 4 with the slot table, without the bookkeeping.
-//   combine_held_kernel  : the same for 4 < K <= 8 with the slot table: a wavefront sums its chunk of 2
+//   combine_held_kernel  : the same for K > 4 with the slot table: a wavefront sums its chunk of 2
 //                          to 16 consecutive tokens' rows and writes them all at its end, so that a
 //                          launch whose wavefronts are all resident reads first and writes last.
 //   rebuild_table_kernel + rebuild_order_kernel : the slot table and the slot-order list of a handle
@@ -89,7 +89,7 @@ struct Tuning {
     int dispatch_order = -1;        // DISPATCH_ORDER: 0 forces the token-order walk
     int dispatch_span = 0;          // DISPATCH_SPAN: 1 | 2 | 4 chunks a wavefront of the slot-order walk, 0 = by size
     int dispatch_prefetch = -1;     // DISPATCH_PREFETCH: 0 = no window-wise source prefetch in the slot-order walk
-    int combine_units = 0;          // COMBINE_UNITS: tokens a wavefront of the gather for 5 to 8 rows a token: 1 .. 16, 0 = by size
+    int combine_units = 0;          // COMBINE_UNITS: tokens a wavefront of the gather for five or more rows a token: 1 .. 16, 0 = by size
     int dispatch_pack = 0;          // DISPATCH_PACK: 1 = one list entry a wavefront of the slot-order walk whatever the row length
     int combine_stores = -1;        // COMBINE_STORES: 0 | 1 nontemporal / agent-scope stores for the combine's output, -1 = by size
     int layout_launches = 0;        // LAYOUT_LAUNCHES: 2 | 3 forces the layout plan

@@ -248,7 +248,7 @@ def combine(y, weights, bias, metadata, counts, expand, *, multiple_reduction=Fa
             stores=None, units=None):
     """Returns (out_x [T,H], out_weights [T,K] | None) through nanoep_combine.  stores=0|1 asks for
     nontemporal / agent-scope stores of the output rows (the library picks by output size);
-    units=1..16 for that many tokens a wavefront where the library has a choice (five to eight
+    units=1..16 for that many tokens a wavefront where the library has a choice (five or more
     rows a token with the slot table; it picks by batch size)."""
     recv_metadata, dst_slots = metadata[0], metadata[3]
     tokens = dst_slots.shape[0]

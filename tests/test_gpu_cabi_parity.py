@@ -194,9 +194,9 @@ def run_dispatch_combine(device, idx, hidden, experts, alignment, expand, zero_p
             assert_bits_equal(stored_out, want_out, f"combine x multi={multi} stores={stores}")
             if weighted:
                 assert_bits_equal(stored_ow, want_ow, f"combine weights stores={stores}")
-        # one to sixteen tokens a wavefront (a choice only with five to eight rows a token; the library
+        # one to sixteen tokens a wavefront (a choice only with five or more rows a token; the library
         # picks by batch size, and small test batches would all take two)
-        if expand and 4 < topk <= 8:
+        if expand and topk > 4:
             for units in (1, 2, 3, 4, 7, 8, 9, 13, 16):
                 held_out, held_ow = cabi.combine(
                     y.to(device), None if yw is None else yw.to(device), None if bias is None else bias.to(device), metadata,
