@@ -262,11 +262,13 @@ __global__ void __launch_bounds__(kWave) combine_held_kernel(const u32x4* __rest
                                                              uint32_t topk_magic,  // fast divisor by K
                                                              uint32_t topk_shift,
                                                              uint32_t side_blocks,
-                                                             uint32_t units) {  // tokens a wavefront, at most kUnits
+                                                             uint32_t units,        // tokens a wavefront, at most kUnits
+                                                             uint32_t first_scale,  // first token of a wavefront = group * first_scale
+                                                             uint32_t stride) {     // distance between a wavefront's tokens
     NANOEP_FETCH_ARGS_4(y, token_slots, out_x, bias);
     NANOEP_FETCH_ARGS_4(tokens, y_rows, chunks, chunks_magic);
     NANOEP_FETCH_ARGS_4(chunks_shift, vectors, topk, flags);
-    NANOEP_FETCH_ARGS_2(side_blocks, units);
+    NANOEP_FETCH_ARGS_4(side_blocks, units, first_scale, stride);
     const uint32_t lane = threadIdx.x;
     if (blockIdx.x < side_blocks) {
         // weights back to their (token, k): one lane each, in workgroups of their own at the front
@@ -285,15 +287,17 @@ __global__ void __launch_bounds__(kWave) combine_held_kernel(const u32x4* __rest
     const bool in_row = vector < vectors;
     // lanes past the end of a short row re-read vector 0 instead of branching around the loads
     const uint32_t load_vector = in_row ? vector : 0u;
-    const uint32_t first = group * units;
-    // this wavefront's tokens: first .. first + count - 1
-    const uint32_t count = first + units <= tokens ? units : tokens - first;
+    // this wavefront's tokens: first, first + stride, ... (`units` of them while they are tokens).
+    // Consecutive tokens (first = group * units, stride 1), or, when the whole launch is resident at
+    // once, every groups-th token (first = group, stride = groups): the tokens in flight at any
+    // moment are then neighbours, and so are the rows they read in every expert's segment.
+    const uint32_t first = group * first_scale;
     u32x4 packed[kUnits];
 #pragma unroll
     for (int u = 0; u < kUnits; ++u) {
-        if (static_cast<uint32_t>(u) >= count)
+        const uint32_t token = first + static_cast<uint32_t>(u) * stride;
+        if (static_cast<uint32_t>(u) >= units || token >= tokens)
             continue;
-        const uint32_t token = first + u;
         // lane k fetches the token's k-th slot; the slots are broadcast to scalars below
         int slot = -1;
         if (lane < topk)
@@ -339,8 +343,9 @@ __global__ void __launch_bounds__(kWave) combine_held_kernel(const u32x4* __rest
         return;
 #pragma unroll
     for (int u = 0; u < kUnits; ++u) {
-        if (static_cast<uint32_t>(u) < count) {
-            u32x4* to = out_x + static_cast<uint64_t>(first + u) * vectors + vector;
+        const uint32_t token = first + static_cast<uint32_t>(u) * stride;
+        if (static_cast<uint32_t>(u) < units && token < tokens) {
+            u32x4* to = out_x + static_cast<uint64_t>(token) * vectors + vector;
             if (flags & kCombineAgentStores)
                 store_vec_agent(to, packed[u]);
             else
@@ -507,10 +512,12 @@ int nanoep_combine(const void* y, const float* weights, const void* bias, const 
     // combine_few_rows_kernel (4096 x 4096 top-2: 17.3 us against 18.1 to 30.5).
     // NANOEP_COMBINE_UNITS=1 keeps one token a wavefront, 2..16 asks for that many.
     int held_units = 0;
+    int64_t held_resident = 0;
     if (direct && num_topk > 4 && num_topk <= 32 && tuning.combine_units != 1) {
         // (16 wavefronts a compute unit, of the compute units this call may use)
         const Topology topology = current_topology(tuning);
         const int64_t resident = int64_t{16} * (num_cus > 0 ? num_cus : topology.cus);
+        held_resident = resident;
         const int64_t work = num_tokens * chunks;
         int64_t rounds = (work + 16 * resident - 1) / (16 * resident);
         held_units = 16;
@@ -526,7 +533,13 @@ int nanoep_combine(const void* y, const float* weights, const void* bias, const 
     if (held_units > 0) {
         const FastDivisor chunks_divisor = make_fast_divisor(static_cast<uint32_t>(chunks));
         const int64_t held_side_blocks = (side_lanes + kWave - 1) / kWave;
-        const int64_t held_blocks = (num_tokens + held_units - 1) / held_units * chunks + held_side_blocks;
+        const int64_t held_groups = (num_tokens + held_units - 1) / held_units;
+        const int64_t held_blocks = held_groups * chunks + held_side_blocks;
+        // A launch that is resident as a whole gives a wavefront every held_groups-th token instead of
+        // consecutive ones (4096 x 7168 top-8 74.8 -> 73.6 us, 8192 x 2048 47.4 -> 46.9, 32768 x 512
+        // 44.7 -> 43.5, 32768 x 1024 84.2 -> 83.7; within half a percent at 2048 x 7168, 3000 x 7168,
+        // 4096 x 4096 top-16).  Launches of several rounds lose with it (16384 x 7168: 311 -> 323 us).
+        const bool strided = held_groups * chunks <= held_resident;
         if (held_blocks >= (int64_t{1} << 31))
             return NANOEP_ERR_INVALID_ARGUMENT;
 #define NANOEP_LAUNCH_HELD(UNITS)                                                                                      \
@@ -534,7 +547,8 @@ int nanoep_combine(const void* y, const float* weights, const void* bias, const 
         static_cast<const u32x4*>(y), weights, static_cast<const u32x4*>(bias), token_slots, static_cast<u32x4*>(out_x), \
         out_weights, static_cast<uint32_t>(num_tokens), static_cast<uint32_t>(y_rows), static_cast<uint32_t>(chunks),   \
         chunks_divisor.magic, chunks_divisor.shift, static_cast<uint32_t>(vectors), static_cast<uint32_t>(num_topk), flags, \
-        topk_divisor.magic, topk_divisor.shift, static_cast<uint32_t>(held_side_blocks), static_cast<uint32_t>(held_units))
+        topk_divisor.magic, topk_divisor.shift, static_cast<uint32_t>(held_side_blocks), static_cast<uint32_t>(held_units), \
+        strided ? 1u : static_cast<uint32_t>(held_units), strided ? static_cast<uint32_t>(held_groups) : 1u)
         if (held_units > 8)
             NANOEP_LAUNCH_HELD(16);
         else if (held_units > 4)
