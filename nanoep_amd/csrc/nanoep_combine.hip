@@ -238,8 +238,8 @@ __global__ void __launch_bounds__(1024) combine_few_rows_kernel(const u32x4* __r
 }
 
 // Expanded layout with the slot table at hand and five or more rows a token: one wavefront (a
-// workgroup of its own) produces the same 1 KiB chunk of the output rows of kUnits consecutive
-// tokens and holds the packed sums back in registers until the last one is done.  The units are
+// workgroup of its own) produces the same 1 KiB chunk of the output rows of up to kUnits tokens
+// and holds the packed sums back in registers until the last one is done.  The units are
 // sized so that all wavefronts of the launch are resident at once wherever the batch allows it: the
 // whole device then reads first and writes last, and HBM sees the output as one burst behind the
 // gather instead of a write among every eight reads.  A token's rows are fetched eight at a time (a
