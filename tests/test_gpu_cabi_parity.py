@@ -293,6 +293,22 @@ def test_baseline_shapes(device, name, tokens, hidden, experts, topk, kind, expa
     run_dispatch_combine(device, idx, hidden, experts, alignment, expand, zero_padding, True, seed=6)
 
 
+@pytest.mark.parametrize(
+    "tokens,hidden,experts,topk",
+    [
+        pytest.param(5000, 7168, 64, 6, id="two-rounds-of-wavefronts"),
+        pytest.param(9001, 2048, 128, 8, id="one-round-every-gth-token-with-a-remainder"),
+        pytest.param(3000, 7168, 64, 12, id="one-round-two-passes-of-rows"),
+    ],
+)
+def test_combine_launches_of_one_round_and_of_several(device, tokens, hidden, experts, topk):
+    """The held sums of the combine at the sizes that decide their launch: one round of resident
+    wavefronts (a wavefront then takes every G-th token, here with groups that the last tokens do not
+    fill), several rounds (consecutive tokens), and more than eight rows a token (two passes)."""
+    idx = cases.routing("dropout", tokens, experts, topk, seed=21)
+    run_dispatch_combine(device, idx, hidden, experts, 1, True, False, True, seed=3)
+
+
 def closed_form_slots(idx, experts, alignment):
     """slot[t,k] from the definition, evaluated with torch on the device of idx: experts ascending,
     inside an expert the tokens ascending, every expert's range padded to the alignment."""
