@@ -10,8 +10,10 @@ constexpr int kCombineMultipleReduction = 1;  // round sums of two or more rows 
 constexpr int kCombineAgentStores = 2;        // agent-scope stores for the output instead of nontemporal ones
 // largest output (bytes) that is written with agent-scope stores
 constexpr int64_t kAgentStoreOutputBytes = int64_t{88} << 20;
-// rows of a token that combine_held_kernel fetches at a time
+// rows of a token that combine_held_kernel fetches at a time, and (token, k) pairs whose weights a
+// lane of its side workgroups restores
 constexpr int kHeldRows = 8;
+constexpr int kHeldSideEntries = 8;
 
 __device__ __forceinline__ float bf16_low(uint32_t packed) { return __uint_as_float(packed << 16); }
 __device__ __forceinline__ float bf16_high(uint32_t packed) { return __uint_as_float(packed & 0xffff0000u); }
@@ -259,8 +261,6 @@ __global__ void __launch_bounds__(kWave) combine_held_kernel(const u32x4* __rest
                                                              uint32_t vectors,
                                                              uint32_t topk,
                                                              int flags,  // kCombineMultipleReduction | kCombineAgentStores
-                                                             uint32_t topk_magic,  // fast divisor by K
-                                                             uint32_t topk_shift,
                                                              uint32_t side_blocks,
                                                              uint32_t units,        // tokens a wavefront, at most kUnits
                                                              uint32_t first_scale,  // first token of a wavefront = group * first_scale
@@ -271,13 +271,23 @@ __global__ void __launch_bounds__(kWave) combine_held_kernel(const u32x4* __rest
     NANOEP_FETCH_ARGS_4(side_blocks, units, first_scale, stride);
     const uint32_t lane = threadIdx.x;
     if (blockIdx.x < side_blocks) {
-        // weights back to their (token, k): one lane each, in workgroups of their own at the front
-        // of the grid (on a payload wavefront they are one more round trip)
-        const uint32_t flat = blockIdx.x * kWave + lane;
-        if (fast_divide(flat, topk_magic, topk_shift) >= tokens)
-            return;
-        const int32_t slot = token_slots[flat];
-        out_weights[flat] = slot >= 0 && static_cast<uint32_t>(slot) < y_rows ? weights[slot] : 0.0f;
+        // weights back to their (token, k): kHeldSideEntries consecutive ones a lane, in workgroups
+        // of their own at the front of the grid (on a payload wavefront they are one more round
+        // trip); few enough wavefronts to count little against what the launch is sized for
+        const uint32_t pairs = tokens * topk;
+        const uint32_t flat = (blockIdx.x * kWave + lane) * kHeldSideEntries;
+        int32_t slot[kHeldSideEntries];
+#pragma unroll
+        for (int j = 0; j < kHeldSideEntries; ++j)
+            slot[j] = flat + j < pairs ? token_slots[flat + j] : -1;
+        float restored[kHeldSideEntries];
+#pragma unroll
+        for (int j = 0; j < kHeldSideEntries; ++j)
+            restored[j] = slot[j] >= 0 && static_cast<uint32_t>(slot[j]) < y_rows ? weights[slot[j]] : 0.0f;
+#pragma unroll
+        for (int j = 0; j < kHeldSideEntries; ++j)
+            if (flat + j < pairs)
+                out_weights[flat + j] = restored[j];
         return;
     }
     const uint32_t payload_block = blockIdx.x - side_blocks;
@@ -512,17 +522,22 @@ int nanoep_combine(const void* y, const float* weights, const void* bias, const 
     // combine_few_rows_kernel (4096 x 4096 top-2: 17.3 us against 18.1 to 30.5).
     // NANOEP_COMBINE_UNITS=1 keeps one token a wavefront, 2..16 asks for that many.
     int held_units = 0;
-    int64_t held_resident = 0;
+    int64_t held_resident = 0, held_side = 0;
     if (direct && num_topk > 4 && num_topk <= 32 && tuning.combine_units != 1) {
         // (16 wavefronts a compute unit, of the compute units this call may use)
         const Topology topology = current_topology(tuning);
         const int64_t resident = int64_t{16} * (num_cus > 0 ? num_cus : topology.cus);
         held_resident = resident;
+        // (the side wavefronts that restore the weights are in the launch too)
+        held_side = (side_lanes + kWave * kHeldSideEntries - 1) / (kWave * kHeldSideEntries);
         const int64_t work = num_tokens * chunks;
-        int64_t rounds = (work + 16 * resident - 1) / (16 * resident);
+        const int64_t rounds = (work + held_side + 16 * resident - 1) / (16 * resident);
         held_units = 16;
         for (int units = 2; units <= 16; ++units) {
-            if ((num_tokens + units - 1) / units * chunks <= rounds * resident) {
+            // (with the registers of at most eight / four held rows a compute unit holds 24 / 32 wavefronts)
+            const int64_t room = units > 8 ? resident : units > 4 ? resident + resident / 2 : 2 * resident;
+            const int64_t payload = (num_tokens + units - 1) / units * chunks;
+            if (payload <= rounds * resident && payload + held_side <= rounds * room) {
                 held_units = units;
                 break;
             }
@@ -532,7 +547,7 @@ int nanoep_combine(const void* y, const float* weights, const void* bias, const 
     }
     if (held_units > 0) {
         const FastDivisor chunks_divisor = make_fast_divisor(static_cast<uint32_t>(chunks));
-        const int64_t held_side_blocks = (side_lanes + kWave - 1) / kWave;
+        const int64_t held_side_blocks = held_side;
         const int64_t held_groups = (num_tokens + held_units - 1) / held_units;
         const int64_t held_blocks = held_groups * chunks + held_side_blocks;
         // A launch that is resident as a whole gives a wavefront every held_groups-th token instead of
@@ -547,7 +562,7 @@ int nanoep_combine(const void* y, const float* weights, const void* bias, const 
         static_cast<const u32x4*>(y), weights, static_cast<const u32x4*>(bias), token_slots, static_cast<u32x4*>(out_x), \
         out_weights, static_cast<uint32_t>(num_tokens), static_cast<uint32_t>(y_rows), static_cast<uint32_t>(chunks),   \
         chunks_divisor.magic, chunks_divisor.shift, static_cast<uint32_t>(vectors), static_cast<uint32_t>(num_topk), flags, \
-        topk_divisor.magic, topk_divisor.shift, static_cast<uint32_t>(held_side_blocks), static_cast<uint32_t>(held_units), \
+        static_cast<uint32_t>(held_side_blocks), static_cast<uint32_t>(held_units),                                      \
         strided ? 1u : static_cast<uint32_t>(held_units), strided ? static_cast<uint32_t>(held_groups) : 1u)
         if (held_units > 8)
             NANOEP_LAUNCH_HELD(16);
