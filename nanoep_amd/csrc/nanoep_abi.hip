@@ -84,6 +84,7 @@ Topology current_topology(const Tuning& tuning) {
             // the runtime reports the L2 of one XCD; a part that reports none keeps the default
             if (hipDeviceGetAttribute(&value, hipDeviceAttributeL2CacheSize, device) == hipSuccess && value >= (1 << 20))
                 asked.l2_bytes = value;
+            held_combine_residency(asked.held_wavefronts);
             g_topology[device] = asked;
             g_topology_known[device] = true;
         }

@@ -436,7 +436,32 @@ __global__ void __launch_bounds__(1024) combine_compact_kernel(const u32x4* __re
     }
 }
 
+// Wavefronts of combine_held_kernel<kUnits> that one compute unit holds at once: four SIMDs, each with
+// 512 vector registers a lane shared by its wavefronts (granules of 8), at most 8 wavefronts a SIMD.
+// The register count is the compiler's, so the runtime is asked for it; `fallback` (what this file
+// was written against) is the answer when the runtime gives none.
+template <int kUnits>
+int held_wavefronts_per_cu(int fallback) {
+    hipFuncAttributes attributes{};
+    if (hipFuncGetAttributes(&attributes, reinterpret_cast<const void*>(&combine_held_kernel<kUnits>)) != hipSuccess ||
+        attributes.numRegs <= 0) {
+        (void)hipGetLastError();
+        return fallback;
+    }
+    const int granules = (attributes.numRegs + 7) / 8 * 8;
+    const int per_simd = 512 / granules;
+    return 4 * (per_simd > 8 ? 8 : per_simd < 1 ? 1 : per_simd);
+}
+
 }  // namespace
+
+void held_combine_residency(int out[4]) {
+    out[0] = held_wavefronts_per_cu<2>(out[0]);
+    out[1] = held_wavefronts_per_cu<4>(out[1]);
+    out[2] = held_wavefronts_per_cu<8>(out[2]);
+    out[3] = held_wavefronts_per_cu<16>(out[3]);
+}
+
 }  // namespace nanoep
 
 using namespace nanoep;
@@ -524,9 +549,10 @@ int nanoep_combine(const void* y, const float* weights, const void* bias, const 
     int held_units = 0;
     int64_t held_resident = 0, held_side = 0;
     if (direct && num_topk > 4 && num_topk <= 32 && tuning.combine_units != 1) {
-        // (16 wavefronts a compute unit, of the compute units this call may use)
+        // (the wavefronts of sixteen held rows a compute unit holds, on the compute units this call may use)
         const Topology topology = current_topology(tuning);
-        const int64_t resident = int64_t{16} * (num_cus > 0 ? num_cus : topology.cus);
+        const int64_t cus = num_cus > 0 ? num_cus : topology.cus;
+        const int64_t resident = cus * topology.held_wavefronts[3];
         held_resident = resident;
         // (the side wavefronts that restore the weights are in the launch too)
         held_side = (side_lanes + kWave * kHeldSideEntries - 1) / (kWave * kHeldSideEntries);
@@ -534,8 +560,8 @@ int nanoep_combine(const void* y, const float* weights, const void* bias, const 
         const int64_t rounds = (work + held_side + 16 * resident - 1) / (16 * resident);
         held_units = 16;
         for (int units = 2; units <= 16; ++units) {
-            // (with the registers of at most eight / four held rows a compute unit holds 24 / 32 wavefronts)
-            const int64_t room = units > 8 ? resident : units > 4 ? resident + resident / 2 : 2 * resident;
+            // (with the registers of at most eight / four held rows a compute unit holds more wavefronts)
+            const int64_t room = cus * topology.held_wavefronts[units > 8 ? 3 : units > 4 ? 2 : units > 2 ? 1 : 0];
             const int64_t payload = (num_tokens + units - 1) / units * chunks;
             if (payload <= rounds * resident && payload + held_side <= rounds * room) {
                 held_units = units;

@@ -110,7 +110,12 @@ struct Topology {
     int cus = 256;
     int xcds = 8;
     int64_t l2_bytes = int64_t{4} << 20;
+    // wavefronts of combine_held_kernel<2 | 4 | 8 | 16> that a compute unit holds at once
+    int held_wavefronts[4] = {32, 32, 24, 16};
 };
+
+// Fills Topology::held_wavefronts from the register counts of the built kernels (nanoep_combine.hip).
+void held_combine_residency(int out[4]);
 
 Topology current_topology(const Tuning& tuning);  // defined in nanoep_abi.hip
 
