@@ -318,6 +318,16 @@ __device__ __forceinline__ void walk_copy_packed(const WalkArgs& a, uint32_t ent
     }
 }
 
+// The list's live entry count from the word the layout stored: a word that cannot be a count
+// (negative, or above `limit`) counts as zero.  Two 32-bit scalar tests; the 64-bit comparisons go
+// through the vector unit.
+__device__ __forceinline__ uint32_t live_entries(int64_t word, uint32_t limit) {
+    uint32_t high = static_cast<uint32_t>(static_cast<uint64_t>(word) >> 32);
+    asm volatile("" : "+s"(high));  // (keeps the compiler from fusing the two tests into a 64-bit one)
+    const uint32_t low = high != 0 ? 0xffffffffu : static_cast<uint32_t>(word);
+    return low <= limit ? low : 0u;
+}
+
 // One workgroup's turn at the slot-order walk; `block` is its position in the walk.
 // Without prefetch the walk is the list front to back, rows_per_block entries a workgroup.
 // With prefetch the walk is cut into one segment per window of the list: `prefetch_blocks`
@@ -388,11 +398,23 @@ __device__ __forceinline__ void walk_copy(const WalkArgs& a, uint32_t entries, u
         }
         return;
     }
-    for (; in_segment < segment_entries; in_segment += a.segment_copy_entries) {
-        if (kPack == 1)
-            walk_copy_entry<kSpan>(a, entries, segment_first + in_segment, lane_vector);
-        else
-            walk_copy_packed<kPack, kSpan>(a, entries, segment_first + in_segment, lane_vector);
+    // the first turn stands alone: a second one is the exception (a live count above what the grid
+    // was sized for), and a loop around both makes every wavefront pay for what only a loop needs
+    if (in_segment >= segment_entries)
+        return;
+    if (kPack == 1)
+        walk_copy_entry<kSpan>(a, entries, segment_first + in_segment, lane_vector);
+    else
+        walk_copy_packed<kPack, kSpan>(a, entries, segment_first + in_segment, lane_vector);
+    in_segment += a.segment_copy_entries;
+    if (__builtin_expect(in_segment < segment_entries, 0)) {
+        do {
+            if (kPack == 1)
+                walk_copy_entry<kSpan>(a, entries, segment_first + in_segment, lane_vector);
+            else
+                walk_copy_packed<kPack, kSpan>(a, entries, segment_first + in_segment, lane_vector);
+            in_segment += a.segment_copy_entries;
+        } while (in_segment < segment_entries);
     }
 }
 
@@ -436,7 +458,7 @@ __global__ void __launch_bounds__(1024) dispatch_walk_kernel(const WalkArgs a) {
         if (kDeviceCount) {
             // a word that cannot be a count (the layout did not run) walks nothing
             live = uniform_load_end(live);
-            entries = live >= 0 && live <= static_cast<int64_t>(a.source_limit) ? static_cast<uint32_t>(live) : 0u;
+            entries = live_entries(live, a.source_limit);
             segment_entries = fast_divide(entries + a.windows - 1, a.windows_magic, a.windows_shift);
         }
         walk_copy<kPieces, kSpan, kDeviceCount, kPrefetch>(a, entries, segment_entries, xcd * a.copy_per_xcd + index_in_xcd);
@@ -447,7 +469,7 @@ __global__ void __launch_bounds__(1024) dispatch_walk_kernel(const WalkArgs a) {
     // then take more than one turn, a grid's worth of list positions apart).  A word that cannot be a
     // count (the layout did not run) walks nothing.
     live = uniform_load_end(live);
-    const uint32_t entries = live >= 0 && live <= static_cast<int64_t>(a.source_limit) ? static_cast<uint32_t>(live) : 0u;
+    const uint32_t entries = live_entries(live, a.source_limit);
     const uint32_t copy_blocks = kPieces == 0 ? entries : fast_divide(entries + a.rows_per_block - 1, a.rows_magic, a.rows_shift);
     const uint32_t copy_per_xcd = fast_divide(copy_blocks + a.xcd_count - 1, a.xcd_magic, a.xcd_shift);
     const uint32_t copy_turns = copy_per_xcd > a.copy_per_xcd ? a.copy_per_xcd : copy_per_xcd;
