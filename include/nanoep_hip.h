@@ -240,6 +240,10 @@ int nanoep_dispatch(const void* x, const float* weights, const int32_t* recv_met
  * the final fp32 pass, as the reference's allow_multiple_reduction mode does.
  * out_weights[t,k] = valid ? (expand ? weights[slot] : weights[row,k]) : 0.
  * y_rows is the row count of y (C when expanded, N when compact).
+ * num_cus (0 = whole device) is range-checked like the dispatch's; the expanded combine with five or
+ * more rows a token and the slot table also sizes its launch by it (its wavefronts hold the sums of
+ * several tokens, as many as it takes for the launch to fit the wavefronts that many compute units
+ * hold at once), so a caller that confines the call with a CU-masked stream passes the mask's count.
  */
 int nanoep_combine(const void* y, const float* weights, const void* bias, const int32_t* recv_metadata,
                    const int64_t* dst_slots, const int32_t* token_slots, int64_t recv_count, int64_t y_rows,
