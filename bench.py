@@ -580,6 +580,42 @@ def measure(workload, args, device, detailed):
 
         ceilings = stream_ceilings(workload, n_recv, assignments, capacity, min(regions, 3), min(launches, 40)) if args.calibration and everything else None
 
+        graph_step = None
+        if everything and not asynchronous:
+            # The cached step recorded once into a HIP graph (two kernel nodes, the combine reading the
+            # dispatch's rows) and replayed: one graph launch a step against two API calls a step.
+            # A graph's pointers are fixed, so its source is one tensor (cache resident where it fits);
+            # the eager figure beside it runs the same two calls on the same tensor.
+            try:
+                graph = torch.cuda.CUDAGraph()
+                torch.cuda.synchronize()
+                with torch.cuda.graph(graph):
+                    captured = buffer.dispatch(xs[0], weights=weights, handle=handle, zero_padding=workload.zero_padding)
+                    captured_out = buffer.combine(captured.x, handle, weights=captured.topk_weights if workload.combine_weights else None)
+
+                def eager_same_source(i):
+                    out = buffer.dispatch(xs[0], weights=weights, handle=handle, zero_padding=workload.zero_padding)
+                    return buffer.combine(out.x, handle, weights=out.topk_weights if workload.combine_weights else None)
+
+                graph_gpu = series(lambda i: graph.replay())[1]
+                eager_gpu = series(eager_same_source)[1]
+                graph_latency = call_to_complete(lambda i: graph.replay())
+                eager_latency = call_to_complete(eager_same_source)
+                graph.replay()
+                torch.cuda.synchronize()
+                same = bool(torch.equal(captured_out.x.view(torch.int16).cpu(), gpu_combined.view(torch.int16)))
+                graph_step = {
+                    "gpu_us_per_step": round(summarize(graph_gpu, launches)[0], 2),
+                    "eager_gpu_us_per_step": round(summarize(eager_gpu, launches)[0], 2),
+                    "us_call_to_complete": round(graph_latency, 1),
+                    "eager_us_call_to_complete": round(eager_latency, 1),
+                    "same_bytes_as_eager": same,
+                    "step": "cached-handle dispatch + combine of its rows, one static source tensor; graph: one replay a step, eager: two API calls a step",
+                }
+                del graph, captured, captured_out
+            except RuntimeError as error:  # a capture the runtime refuses is reported, not fatal to the other figures
+                graph_step = {"error": str(error).splitlines()[0][:200]}
+
     wall_us, wall_us_min = summarize(step_wall, launches)
     gpu_step_us, gpu_step_us_min = summarize(step_gpu, launches)
     d_us, d_us_min = summarize(dispatch_gpu, launches)
@@ -656,6 +692,8 @@ def measure(workload, args, device, detailed):
         result["stream_ceiling"] = ceilings
     if seven is not None:
         result.update(seven)
+    if graph_step is not None:
+        result["hip_graph_step"] = graph_step
     if detailed:
         result["cli_region"] = cli
         result["layout_us_gpu_no_host_wait"] = round(layout_us, 2)
@@ -707,7 +745,7 @@ def main():
         others[name] = {key: entry[key] for key in (
             "value", "unit", "ms_per_step", "dispatch_us", "dispatch_us_min", "combine_us", "combine_us_min",
             "dispatch_us_cache_resident_source", "fresh_dispatch_us_host", "cached_dispatch_us_call_to_complete",
-            "combine_us_call_to_complete", "roofline", "roofline_combine", "dispatch_prefetch_switch", "side_stream_consumer", "stream_ceiling",
+            "combine_us_call_to_complete", "roofline", "roofline_combine", "dispatch_prefetch_switch", "side_stream_consumer", "stream_ceiling", "hip_graph_step",
             "cpu_baseline", "bit_exact_vs_oracle") if key in entry}
         others[name]["config"] = {key: entry["config"][key] for key in (
             "tokens", "hidden", "experts", "topk", "layout", "alignment", "zero_padding", "rotating_source_copies", "step")}
