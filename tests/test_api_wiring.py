@@ -352,3 +352,17 @@ def test_reference_import_paths():
         assert getattr(backends, name) is getattr(nanoep_amd, name) is getattr(cuda, name)
     assert nanoep_amd.EPConfig is not None and nanoep_amd.__version__
     assert callable(cuda.check_torch_deterministic)
+
+
+def test_the_benchmark_refuses_more_than_one_gpu():
+    """bench.py measures one rank on one GPU; any other --gpus ends at once with a message and a
+    non-zero status, before anything touches a device."""
+    import pathlib
+    import subprocess
+    import sys
+
+    bench = pathlib.Path(__file__).resolve().parents[1] / "bench.py"
+    done = subprocess.run([sys.executable, str(bench), "--gpus", "2"], capture_output=True, text=True, timeout=120)
+    assert done.returncode != 0
+    assert "ONE GPU" in done.stderr + done.stdout
+    assert not any(line.startswith("{") for line in done.stdout.splitlines())
