@@ -177,17 +177,18 @@ struct WalkArgs {
     uint32_t segment_magic;    // fast divisor by segment_blocks
     uint32_t segment_shift;
     uint32_t prefetch_blocks;  // prefetch workgroups at the head of a segment
-    uint32_t window_vectors;   // 16-byte vectors of one window's source rows
-    uint32_t source_vectors;   // ... of all source rows
-    uint32_t segment_entries;       // list entries of a segment: ceil(entries / windows)
-    uint32_t segment_copy_entries;  // list entries the copy workgroups of a segment cover in one turn
-    // entry count on the device
+    uint32_t segment_entries;  // list entries of a segment: ceil(entries / windows)
+    // entry count on the device (the last of the 128 bytes a copy wavefront waits for before its list
+    // entry: one more cache line of arguments on that way costs the walk a microsecond)
     uint32_t windows;  // segments of the walk
     uint32_t windows_magic;  // fast divisor by it
     uint32_t windows_shift;
+    const int64_t* live_count;
+    // what only a few wavefronts need: a second turn, the prefetch workgroups, the plain list walk
+    uint32_t window_vectors;        // 16-byte vectors of one window's source rows
+    uint32_t source_vectors;        // ... of all source rows
     uint32_t rows_magic;  // fast divisor by rows_per_block
     uint32_t rows_shift;
-    const int64_t* live_count;
     // gap rows
     const int64_t* expert_counts;
     const int64_t* expert_offsets;
@@ -197,6 +198,7 @@ struct WalkArgs {
     uint32_t pad_groups_per_expert;
     uint32_t row_vectors;
 };
+static_assert(offsetof(WalkArgs, live_count) + sizeof(const int64_t*) == 128, "what a copy wavefront waits for fits two cache lines");
 
 // What a workgroup of the walk's grid does when it has no copy work: every XCD's copy workgroups are
 // followed by its share of the workgroups that clear the alignment gaps, each wavefront one whole
@@ -331,7 +333,7 @@ __device__ __forceinline__ uint32_t live_entries(int64_t word, uint32_t limit) {
 // One workgroup's turn at the slot-order walk; `block` is its position in the walk.
 // Without prefetch the walk is the list front to back, rows_per_block entries a workgroup.
 // With prefetch the walk is cut into one segment per window of the list: `prefetch_blocks`
-// workgroups that read the window's source rows, then `segment_copy_entries / rows_per_block`
+// workgroups that read the window's source rows, then `segment_blocks - prefetch_blocks`
 // workgroups that copy the segment's share of the list, entries [s * segment_entries, (s + 1) *
 // segment_entries) of it.  The windows hold nearly the same number of entries each, so equal shares
 // follow them closely (a skewed mask only costs locality).  With the entry count on the device the
@@ -406,14 +408,16 @@ __device__ __forceinline__ void walk_copy(const WalkArgs& a, uint32_t entries, u
         walk_copy_entry<kSpan>(a, entries, segment_first + in_segment, lane_vector);
     else
         walk_copy_packed<kPack, kSpan>(a, entries, segment_first + in_segment, lane_vector);
-    in_segment += a.segment_copy_entries;
+    // (list entries the copy workgroups of a segment cover in one turn)
+    const uint32_t turn_entries = (a.segment_blocks - a.prefetch_blocks) * a.rows_per_block;
+    in_segment += turn_entries;
     if (__builtin_expect(in_segment < segment_entries, 0)) {
         do {
             if (kPack == 1)
                 walk_copy_entry<kSpan>(a, entries, segment_first + in_segment, lane_vector);
             else
                 walk_copy_packed<kPack, kSpan>(a, entries, segment_first + in_segment, lane_vector);
-            in_segment += a.segment_copy_entries;
+            in_segment += turn_entries;
         } while (in_segment < segment_entries);
     }
 }
@@ -436,7 +440,7 @@ __global__ void __launch_bounds__(1024) dispatch_walk_kernel(const WalkArgs a) {
     NANOEP_FETCH_ARGS_2(a.recv_weights, a.weights);
     if (kPrefetch) {
         NANOEP_FETCH_ARGS_4(a.segment_blocks, a.segment_magic, a.segment_shift, a.prefetch_blocks);
-        NANOEP_FETCH_ARGS_2(a.segment_entries, a.segment_copy_entries);
+        NANOEP_FETCH_ARGS_2(a.segment_entries, a.segment_entries);
     }
     // the live count's load is on every copy wavefront's way to its list entry: it leaves with the
     // first batch of arguments and is in flight during the index arithmetic below
@@ -701,7 +705,6 @@ int nanoep_dispatch(const void* x, const float* weights, const int32_t* recv_met
         a.window_vectors = static_cast<uint32_t>(static_cast<int64_t>(window_tokens) * vectors);
         a.source_vectors = static_cast<uint32_t>(num_tokens * vectors);
         a.segment_entries = static_cast<uint32_t>(segment_entries);
-        a.segment_copy_entries = static_cast<uint32_t>(segment_copy_blocks * entries_per_block);
         a.windows = static_cast<uint32_t>(windows);
         a.windows_magic = windows_divisor.magic;
         a.windows_shift = windows_divisor.shift;
