@@ -151,6 +151,16 @@ constexpr int kRankMask = (1 << kRankBits) - 1;
 // so the order of one expert's assignments is the token order and a popcount prefix is the rank.
 // The token's routing ids are fetched in one batch of independent loads (kCap >= K of them, the
 // surplus re-reads id 0) and stay in registers for both passes over the bit matrix.
+// What a thread of the count pass knows at its end, for a kernel that goes on to the assignment
+// pass in the same workgroup and need not read it back from memory.
+template <int kCap>
+struct CountedToken {
+    int32_t packed[kCap];  // the token's entries of the rank table
+    int32_t row;           // the token's receive row within the block, -1 when it is not sent
+    int32_t first_count;   // the block's count of histogram row threadIdx.x (0 when there is no such row)
+    int32_t bad;           // the block's routing status bits
+};
+
 template <int kCap>
 __device__ __forceinline__ void layout_count_block(const int64_t* __restrict__ topk_idx,
                                                    int64_t num_tokens,
@@ -162,7 +172,8 @@ __device__ __forceinline__ void layout_count_block(const int64_t* __restrict__ t
                                                    int32_t* block_counts,
                                                    int32_t* block_status,
                                                    int32_t* packed_rank,
-                                                   int32_t* local_row) {
+                                                   int32_t* local_row,
+                                                   CountedToken<kCap>& counted) {
     extern __shared__ uint32_t layout_lds[];
     const int rows = local_experts + 1;
     // bit rows are words + 1 apart: an odd stride spreads the experts a wavefront touches over the LDS banks
@@ -241,6 +252,7 @@ __device__ __forceinline__ void layout_count_block(const int64_t* __restrict__ t
         atomicOr(&block_bad, bad);
     __syncthreads();
 
+    counted.first_count = 0;
     for (int row = threadIdx.x; row < rows; row += threads) {
         int running = 0;
         for (int w = 0; w < words; ++w) {
@@ -248,10 +260,17 @@ __device__ __forceinline__ void layout_count_block(const int64_t* __restrict__ t
             running += __popc(bits[static_cast<size_t>(row) * stride + w]);
         }
         block_counts[static_cast<int64_t>(blockIdx.x) * rows + row] = running;
+        if (row == static_cast<int>(threadIdx.x))
+            counted.first_count = running;
     }
     if (threadIdx.x == 0)
         block_status[blockIdx.x] = block_bad;
     __syncthreads();
+    counted.bad = block_bad;
+    counted.row = -1;
+#pragma unroll
+    for (int k = 0; k < kCap; ++k)
+        counted.packed[k] = -1;
 
     if (live) {
         const uint32_t below = bit - 1;
@@ -278,7 +297,11 @@ __device__ __forceinline__ void layout_count_block(const int64_t* __restrict__ t
                     packed_rank[token * num_topk + k] = packed[k];
         }
         const uint32_t received = bits[static_cast<size_t>(local_experts) * stride + word];
-        local_row[token] = (received & bit) ? prefix[static_cast<size_t>(local_experts) * words + word] + __popc(received & below) : -1;
+        counted.row = (received & bit) ? prefix[static_cast<size_t>(local_experts) * words + word] + __popc(received & below) : -1;
+        local_row[token] = counted.row;
+#pragma unroll
+        for (int k = 0; k < kCap; ++k)
+            counted.packed[k] = packed[k];
     }
 }
 
@@ -294,8 +317,9 @@ __global__ void __launch_bounds__(kMaxBlockTokens) layout_count_kernel(const int
                                                            int32_t* __restrict__ block_status,
                                                            int32_t* __restrict__ packed_rank,
                                                            int32_t* __restrict__ local_row) {
+    CountedToken<kCap> counted;
     layout_count_block<kCap>(topk_idx, num_tokens, num_topk, local_experts, words, threads, snapshot, block_counts,
-                             block_status, packed_rank, local_row);
+                             block_status, packed_rank, local_row, counted);
 }
 
 __device__ __forceinline__ int64_t round_up_to(int64_t value, int64_t alignment) {
@@ -511,7 +535,7 @@ __device__ __forceinline__ int64_t wave_inclusive_scan(int64_t value) {
 // Either way the workgroup also scans its own histogram over experts: that places every
 // assignment of the block in expert-major order inside the block's run of `slot_order`; the runs
 // of consecutive blocks follow each other without gaps and the unused tail of the list is -1.
-template <int kCap, bool kFusedScan>
+template <int kCap, bool kFusedScan, bool kOwnBlock = false>
 __device__ __forceinline__ void layout_assign_block(const int32_t* block_counts,
                                                     const int32_t* block_status,
                                                     int num_blocks,
@@ -535,7 +559,8 @@ __device__ __forceinline__ void layout_assign_block(const int32_t* block_counts,
                                                     int64_t* __restrict__ dst_slots,
                                                     int32_t* __restrict__ token_slots,
                                                     int64_t* __restrict__ slot_order,
-                                                    int publisher) {
+                                                    int publisher,
+                                                    const CountedToken<kCap>* own = nullptr) {
     extern __shared__ int32_t assign_lds[];
     __shared__ int64_t wave_padded[kMaxBlockTokens / kWave];
     __shared__ int64_t wave_assigned[kMaxBlockTokens / kWave];
@@ -556,19 +581,41 @@ __device__ __forceinline__ void layout_assign_block(const int32_t* block_counts,
     const int block = blockIdx.x;
     const int64_t token = static_cast<int64_t>(block) * tokens_per_block + tid;
     const bool live = tid < tokens_per_block && token < num_tokens;
-    const int row_in_block = live ? local_row[token] : -1;
-    // fetched here, ahead of the scans, so that the round trip overlaps them
+    // kOwnBlock: the count pass ran in this very workgroup (the batch is one block) and `own` holds
+    // what this thread found there; nothing of it is read back from memory.  With no more histogram
+    // rows than threads that goes for the histogram too: the block's counts are the totals, nothing
+    // lies before the block, and its window is the block.
+    const bool own_counts = kOwnBlock && rows <= threads;
+    int row_in_block;
     int32_t packed[kCap];
+    if (kOwnBlock) {
+        row_in_block = own->row;
 #pragma unroll
-    for (int k = 0; k < kCap; ++k)
-        packed[k] = live ? packed_rank[token * num_topk + (k < num_topk ? k : 0)] : -1;
+        for (int k = 0; k < kCap; ++k)
+            packed[k] = own->packed[k];
+    } else {
+        row_in_block = live ? local_row[token] : -1;
+        // fetched here, ahead of the scans, so that the round trip overlaps them
+#pragma unroll
+        for (int k = 0; k < kCap; ++k)
+            packed[k] = live ? packed_rank[token * num_topk + (k < num_topk ? k : 0)] : -1;
+    }
 
     // the publishing workgroup gathers the blocks' routing status; the first word a thread is fetched here, used
     // behind the histogram loads, so that its round trip is not a second one behind theirs
     int first_status = 0;
-    if (kFusedScan && block == publisher && tid < num_blocks)
+    if (kOwnBlock)
+        first_status = tid == 0 ? own->bad : 0;
+    else if (kFusedScan && block == publisher && tid < num_blocks)
         first_status = block_status[tid];
-    if (kFusedScan) {
+    if (own_counts) {
+        if (tid < rows) {
+            column_total[tid] = own->first_count;
+            slot_base[tid] = 0;
+            order_base[tid] = own->first_count;
+            window_before[tid] = 0;
+        }
+    } else if (kFusedScan) {
         for (int i = tid; i < 4 * rows; i += threads)
             assign_lds[i] = 0;
         if (tid == 0) {
@@ -729,7 +776,7 @@ __device__ __forceinline__ void layout_assign_block(const int32_t* block_counts,
         window_earlier += wave_window_before[w];
     }
     // this block's own assignments: the window's when the window is the block
-    const int own_total = kFusedScan ? own_assignments : window_total;
+    const int own_total = kFusedScan && !own_counts ? own_assignments : window_total;
     if (!kFusedScan)
         assigned = totals[0];
     for (int e = first; e < last; ++e) {
@@ -759,7 +806,7 @@ __device__ __forceinline__ void layout_assign_block(const int32_t* block_counts,
         recv_rank_prefix[0] = received;
         host_counts[1] = capacity;
         host_counts[2] = assigned;
-        host_counts[3] = status_bits;
+        host_counts[3] = kOwnBlock ? own->bad : status_bits;
         __threadfence_system();
         __hip_atomic_store(&host_counts[0], received, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_SYSTEM);
     }
@@ -823,7 +870,8 @@ __global__ void __launch_bounds__(kMaxBlockTokens) layout_assign_kernel(const in
 }
 
 // Whole layout in one launch when all tokens fit one block: the count pass, then (its results are
-// this workgroup's own global writes, made visible by the fence and the barrier) the assignment pass.
+// this workgroup's own global writes: the barrier orders them for the workgroup, and a fence of
+// wider scope in front of it would write the XCD's L2 back for nobody) the assignment pass.
 template <int kCap>
 __global__ void __launch_bounds__(kMaxBlockTokens) layout_single_block_kernel(const int64_t* topk_idx,
                                                                   int64_t num_tokens,
@@ -847,13 +895,14 @@ __global__ void __launch_bounds__(kMaxBlockTokens) layout_single_block_kernel(co
                                                                   int64_t* dst_slots,
                                                                   int32_t* token_slots,
                                                                   int64_t* slot_order) {
+    CountedToken<kCap> counted;
     layout_count_block<kCap>(topk_idx, num_tokens, num_topk, local_experts, words, threads, snapshot, block_counts,
-                             block_status, packed_rank, local_row);
-    __threadfence();
+                             block_status, packed_rank, local_row, counted);
     __syncthreads();
-    layout_assign_block<kCap, true>(block_counts, block_status, 1, num_tokens, num_topk, local_experts, words * 32, 1, threads,
-                                    expand, alignment, packed_rank, local_row, expert_counts, expert_offsets, send_counts,
-                                    recv_rank_prefix, nullptr, host_counts, recv_metadata, dst_slots, token_slots, slot_order, 0);
+    layout_assign_block<kCap, true, true>(block_counts, block_status, 1, num_tokens, num_topk, local_experts, words * 32, 1, threads,
+                                          expand, alignment, packed_rank, local_row, expert_counts, expert_offsets, send_counts,
+                                          recv_rank_prefix, nullptr, host_counts, recv_metadata, dst_slots, token_slots, slot_order, 0,
+                                          &counted);
 }
 
 
